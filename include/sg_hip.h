@@ -1,0 +1,221 @@
+/*
+ * sg_hip.h -- C ABI of the MI355X (gfx950) scatter-gather engine.
+ *
+ * Drop-in boundary for SplitRPC's p2p_rpc_sg_engine path.  Plain C: pointers
+ * and sizes only.  Every pointer named "device" must be addressable by the
+ * GPU the context was created on (hipMalloc, VMM mapping, or pinned host
+ * memory); the library never allocates or frees payload memory.
+ *
+ * Return convention: 0 on success, a negative SG_E_* code on failure (the
+ * reference's sg_on_gpu returns 1/0, src/transport/g_copy_ng.cu:169-223; the
+ * C++ engine above this ABI keeps that convention for its callers).
+ * sg_hip_last_error() gives the text of the last failure on a context.
+ * No exceptions cross the ABI.  A context is used by one thread at a time
+ * (the reference constructs and uses its engine on the shunter thread,
+ * src/splitrpc_server/p2p_rpc_dpdk_server.cc:79-87).
+ */
+#ifndef SG_HIP_H
+#define SG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SG_HIP_ABI_VERSION 1
+
+/* Error codes. */
+#define SG_OK 0
+#define SG_E_INVAL (-22)   /* bad argument, size beyond what the context was sized for */
+#define SG_E_NOMEM (-12)   /* context scratch could not be allocated */
+#define SG_E_HIP (-5)      /* a HIP call failed; see sg_hip_last_error() */
+#define SG_E_DATA (-74)    /* a kernel found tables or headers it refused to follow
+                              (slot index out of range, length beyond the slot, ...) */
+
+/* Wire-header profiles.  REF64 is the reference's p2p_rpc_hdr
+ * (src/p2p_rpc.h:10-17): 42 B Eth/IPv4/UDP, u64 req_token @42,
+ * i64 sock_perf_header @50, u16 seq_num @58, pad to 64; payload @64.
+ * BL58: u64 req_id @42, u16 frag_idx @50, u16 num_frags @52,
+ * u32 payload_len @54; payload @58. */
+#define SG_HDR_BL58 0u
+#define SG_HDR_REF64 1u
+
+/* Flags. */
+#define SG_F_IPV4_CSUM (1u << 0)       /* finished IPv4 header checksum (RFC 1071); the
+                                          reference leaves it to the NIC,
+                                          src/transport/dpdk_rx_tx.h:143 */
+#define SG_F_UDP_CSUM_PSEUDO (1u << 1) /* raw pseudo-header sum in udp.check, as
+                                          add_udp_cksum does, src/p2p_rpc.h:58-61 */
+#define SG_F_UDP_CSUM_FULL (1u << 2)   /* finished UDP checksum over header + payload (RFC 768) */
+#define SG_F_REF_QUIRKS (1u << 3)      /* pseudo sum takes UDP length as tot_len - version*4,
+                                          src/eth_common.h:111-112 */
+#define SG_F_ASYNC (1u << 16)          /* enqueue only; completion through sg_hip_sync() */
+#define SG_F_NO_XCD_REMAP (1u << 17)   /* launch-order = item order (for experiments) */
+
+#define SG_MAX_BI_SIZE 1024 /* src/p2p_bufs.h:10 */
+#define SG_MAX_TENSORS 4    /* src/p2p_rpc_app_stub.h:10 */
+
+/* Layout twins of the reference's fixed tables (src/p2p_bufs.h:15-40), so a
+ * P2pRpcRr's tables can be handed over without conversion. */
+#pragma pack(push, 1)
+typedef struct sg_hbufs {
+  uint64_t burst_items[SG_MAX_BI_SIZE];
+  uint16_t num_items;
+} sg_hbufs; /* == p2p_hbufs, 8194 B */
+
+typedef struct sg_sk_buf {
+  uint64_t i_buf[SG_MAX_BI_SIZE];
+  uint64_t o_buf[SG_MAX_BI_SIZE];
+  uint64_t len[SG_MAX_BI_SIZE - 1];
+  uint64_t num_items;
+} sg_sk_buf; /* == p2p_sk_buf == g_copy_params, 24576 B */
+#pragma pack(pop)
+
+typedef struct sg_hip_ctx sg_hip_ctx;
+
+typedef struct sg_hip_cfg {
+  uint32_t struct_size; /* sizeof(sg_hip_cfg), for ABI growth */
+  uint32_t max_reqs;    /* largest n_req of one batch call (0: 4096) */
+  uint32_t max_frames;  /* largest fragment / response-frame count of one batch call (0: 65536) */
+  uint32_t flags;       /* reserved, 0 */
+  void *stream;         /* hipStream_t to launch on; NULL: the context creates one */
+} sg_hip_cfg;
+
+/* A ring of packet-buffer slots in device memory. */
+typedef struct sg_ring_desc {
+  void *base;           /* device */
+  uint32_t n_slots;
+  uint32_t slot_size;   /* bytes, even */
+  uint32_t hdr_profile; /* SG_HDR_* */
+  uint32_t reserved;
+} sg_ring_desc;
+
+/* Where request bytes go and response bytes come from.
+ * n_tensors == 0: one packed arena addressed through the device-resident
+ * bump ring (P2pRpcTring::get_next, src/p2p_rpc_tring.h:27-33): request r
+ * starts where request r-1 ended, modulo arena_cap.  arena_mirrored != 0
+ * says the arena's pages are mapped twice back to back
+ * (src/p2p_rpc_app_rr_mem_pool.h:302-306) so that [arena, arena + 2*cap) is
+ * addressable and a request may run past the end; otherwise a run that
+ * crosses the end is split.
+ * n_tensors >= 1: tensor-major buffers in the sense of g_params_v2
+ * (src/p2p_rpc_app_stub.h:11-20): a request's byte stream is tensor 0's
+ * bytes, then tensor 1's, ...; tensor t of request r lives at
+ * tensor_base[t] + r * tensor_size[t]. */
+typedef struct sg_app_desc {
+  void *tensor_base[SG_MAX_TENSORS]; /* device */
+  uint64_t tensor_size[SG_MAX_TENSORS];
+  uint32_t n_tensors;
+  uint32_t arena_mirrored;
+  void *arena; /* device */
+  uint64_t arena_cap;
+} sg_app_desc;
+
+/* One gather batch: the fragment tables of n_req reassembled requests in
+ * compact CSR form (what P2pRpcRr::payload_bufs holds per request,
+ * src/p2p_rpc_rr_ng.h:29-31, with pointers reduced to slot indices). */
+typedef struct sg_gather_args {
+  sg_ring_desc ring;
+  const uint32_t *frag_slot; /* device, n_frags: ring slot of each fragment; requests in
+                                batch order, fragments in seq order inside a request */
+  const uint32_t *frag_len;  /* device, n_frags payload bytes, or NULL: read payload_len
+                                from each slot's header (BL58 only) */
+  const uint32_t *req_first; /* device, n_req + 1: first fragment of each request */
+  uint32_t n_req;
+  uint32_t n_frags;
+  sg_app_desc app;
+  uint64_t *offsets_out; /* device, n_req + 1 arena offsets (packed mode), or NULL */
+  uint32_t flags;
+  uint32_t reserved;
+} sg_gather_args;
+
+/* One scatter batch.  Response r has resp_size[r] bytes (fixed_resp_size when
+ * resp_size is NULL), cut into frames of at most mtu bytes by the reference's
+ * fragmenting rule (src/transport/dpdk_rx_tx.h:137-139).  Frame f of the
+ * batch is written to TX slot tx_slot[f]; its header is the header found in
+ * RX slot hdr_src_slot[f], rewritten (swap_eth_hdr + add_ip_udp_len +
+ * add_udp_cksum, src/p2p_rpc.h:51-83, and the routing fields rr_set_hdr
+ * writes, src/transport/dpdk_transport_ng.h:129-131).  tx may alias rx; then
+ * hdr_src_slot[f] must equal tx_slot[f] or be a slot no frame of the batch
+ * writes. */
+typedef struct sg_scatter_args {
+  sg_ring_desc rx;
+  sg_ring_desc tx;
+  const uint32_t *tx_slot;      /* device, n_frames */
+  const uint32_t *hdr_src_slot; /* device, n_frames */
+  const uint32_t *resp_first;   /* device, n_req + 1 */
+  const uint64_t *resp_size;    /* device, n_req, or NULL */
+  uint64_t fixed_resp_size;
+  uint32_t n_req;
+  uint32_t n_frames;
+  uint32_t mtu;
+  uint32_t flags; /* SG_F_* */
+  sg_app_desc app;
+  uint64_t *offsets_out; /* device, n_req + 1, or NULL */
+} sg_scatter_args;
+
+/* ---- lifetime -------------------------------------------------------------
+ * Replaces P2pRpcSgGpuEngine's constructor/destructor work
+ * (src/p2p_rpc_sg_engine.h:261-307: stubs, doorbells, streams, persistent
+ * kernel start and stop).  No persistent kernel is started: work is launched
+ * per call on the context's stream. */
+sg_hip_ctx *sg_hip_create(int device_id, const sg_hip_cfg *cfg);
+void sg_hip_destroy(sg_hip_ctx *ctx);
+const char *sg_hip_last_error(const sg_hip_ctx *ctx); /* ctx may be NULL: creation errors */
+int sg_hip_abi_version(void);
+void *sg_hip_stream(sg_hip_ctx *ctx); /* the hipStream_t work is launched on */
+
+/* Waits for everything enqueued on the context and returns SG_E_DATA if any
+ * kernel since the last sync refused part of its input. */
+int sg_hip_sync(sg_hip_ctx *ctx);
+
+/* ---- per-request entry points (API v0 / v1 parity) --------------------------
+ * Replace sg_on_gpu(CopyCtx*, p2p_sk_buf*) + the doorbell wait
+ * (src/transport/g_copy_ng.cu:186-223, src/p2p_rpc_sg_engine.h:198-239):
+ * copy every run of a host-built run table; i_buf/o_buf hold device
+ * addresses.  Synchronous: on return the bytes are in place. */
+int sg_hip_gather(sg_hip_ctx *ctx, const sg_sk_buf *skb);
+int sg_hip_scatter(sg_hip_ctx *ctx, const sg_sk_buf *skb);
+
+/* Replaces do_g_pp(ctx, p2p_hbufs*) (src/transport/g_udp_handler.cuh:20-24,
+ * g_udp_handler.cu:96-123,172-178) and swap_hdrs_on_cpu
+ * (src/transport/dpdk_transport_ng.h:70-84): rewrite in place the headers a
+ * table of device header pointers names; header i gets frag_idx i,
+ * num_frags = num_items and payload_len = min(remaining, mtu) of
+ * payload_size.  Synchronous. */
+int sg_hip_swap_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, uint32_t hdr_profile,
+                     uint64_t payload_size, uint32_t mtu, uint32_t flags);
+
+/* ---- batched entry points ----------------------------------------------------
+ * No counterpart call in the reference (which handles one request per
+ * doorbell round trip, src/p2p_rpc_sg_engine.h:198-218); the per-request
+ * semantics are those of P2pRpcSgCpuEngine::gather / scatter
+ * (src/p2p_rpc_sg_engine.h:150-164) applied to every request of the batch,
+ * with request offsets taken from the bump ring.  Synchronous unless
+ * SG_F_ASYNC is set. */
+int sg_hip_gather_batch(sg_hip_ctx *ctx, const sg_gather_args *args);
+int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
+
+/* Device-resident bump-ring cursors (P2pRpcTring::prev_offset,
+ * src/p2p_rpc_tring.h:14-16), one for the request arena (which = 0) and one
+ * for the response arena (which = 1).  Both calls synchronize. */
+int sg_hip_set_cursor(sg_hip_ctx *ctx, int which, uint64_t value);
+int sg_hip_get_cursor(sg_hip_ctx *ctx, int which, uint64_t *value);
+
+/* ---- measurement -------------------------------------------------------------
+ * With profiling on, every kernel launch is bracketed by HIP events on the
+ * context's stream (the PROFILE_MODE GDelay/SDelay vectors of the reference,
+ * src/p2p_rpc_sg_engine.h:83-92, at kernel granularity).  which: 0 descriptor
+ * build, 1 gather copy, 2 scatter copy + header rewrite, 3 per-request run
+ * copy, 4 header-only rewrite.  sg_hip_kernel_time synchronizes, returns the
+ * accumulated milliseconds and launch count since profiling was switched on,
+ * and leaves the accumulators running. */
+int sg_hip_set_profiling(sg_hip_ctx *ctx, int on);
+int sg_hip_kernel_time(sg_hip_ctx *ctx, int which, double *total_ms, uint64_t *launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SG_HIP_H */

@@ -1,0 +1,916 @@
+// sg_hip.hip -- kernels and C ABI of the gfx950 scatter-gather engine.
+//
+// Three kernels carry a batch:
+//   k_prep     one workgroup per request: block-wide exclusive scan of the
+//              fragment lengths (-> offset of every fragment inside its
+//              request, the running sum gather_skbs keeps,
+//              src/p2p_rpc_sg_engine.h:22-43), request totals, and -- in the
+//              workgroup that finishes last -- the scan of the request totals
+//              through the device-resident bump-ring cursor
+//              (src/p2p_rpc_tring.h:27-33).  Emits 16-byte run descriptors.
+//   k_gather   one wavefront per fragment run: ring slot payload -> tensor.
+//   k_scatter  one wavefront per response frame: tensor -> TX slot payload,
+//              header rewrite, checksums.
+// plus k_copy_runs / k_swap_hdrs for the per-request entry points.
+#include <hip/hip_runtime.h>
+
+#include <errno.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+#include <vector>
+
+#include "../../include/sg_hip.h"
+#include "sg_device.h"
+
+using namespace sg;
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// device-side argument blocks
+// ---------------------------------------------------------------------------
+
+struct AppDev {
+  uint8_t *tensor_base[SG_MAX_TENSORS];
+  uint64_t tensor_size[SG_MAX_TENSORS];
+  uint32_t n_tensors;
+  uint32_t mirrored;
+  uint8_t *arena;
+  uint64_t cap;
+};
+
+struct PrepArgs {
+  // mode 0 (gather): lengths from item_len[] or from the slot headers
+  // mode 1 (scatter): lengths from the fragmenting rule over sizes[] / fixed_size
+  uint32_t mode;
+  uint32_t n_req;
+  const uint8_t *ring;
+  uint32_t n_slots;
+  uint32_t slot_size;
+  uint32_t hl;
+  uint32_t mtu;
+  const uint32_t *item_slot;
+  const uint32_t *item_len;
+  const uint32_t *first;
+  const uint64_t *sizes;
+  uint64_t fixed_size;
+  uint32_t n_items;
+  uint32_t packed;
+  uint64_t cap;
+  uint64_t max_req_bytes;  // tensor-major: sum of tensor sizes
+  u32x4 *desc;             // {slot, len, offset in request, request}
+  uint64_t *req_size;
+  uint64_t *req_off;
+  uint64_t *cursor;
+  uint64_t *offsets_out;
+  uint32_t *ticket;
+  uint32_t *status;
+};
+
+// Block-wide exclusive scan of one value per thread (kBlock threads).
+// Returns the exclusive prefix; *total gets the block sum.
+__device__ __forceinline__ uint64_t block_exclusive_scan(uint64_t v, uint64_t *lds_wave_tot,
+                                                         uint64_t *total)
+{
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t wv = threadIdx.x / kWave;
+  uint64_t inc = v;
+#pragma unroll
+  for (int d = 1; d < (int)kWave; d <<= 1) {
+    uint64_t up = __shfl_up(inc, d, 64);
+    if ((int)lane >= d) inc += up;
+  }
+  if (lane == kWave - 1) lds_wave_tot[wv] = inc;
+  __syncthreads();
+  uint64_t base = 0, tot = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < kWavesPerBlock; i++) {
+    uint64_t t = lds_wave_tot[i];
+    if (i < wv) base += t;
+    tot += t;
+  }
+  __syncthreads();
+  *total = tot;
+  return base + inc - v;
+}
+
+__global__ __launch_bounds__(kBlock) void k_prep(PrepArgs a)
+{
+  __shared__ uint64_t wave_tot[kWavesPerBlock];
+  __shared__ uint32_t is_last;
+  const uint32_t r = blockIdx.x;
+  uint32_t f0 = a.first[r];
+  uint32_t f1 = a.first[r + 1];
+  uint32_t bad = 0;
+  uint64_t carry = 0;
+  // the table must tile [0, n_items) without gaps, or descriptors of an
+  // earlier call would be taken for this one's
+  if (f0 > f1 || f1 > a.n_items || (r == 0 && f0 != 0) || (r == a.n_req - 1 && f1 != a.n_items)) {
+    bad |= kStBadTable;
+    f0 = f1 = 0;
+  }
+
+  if (a.mode == 0) {
+    for (uint32_t base = f0; base < f1; base += kBlock) {
+      const uint32_t f = base + threadIdx.x;
+      uint32_t len = 0, slot = 0;
+      if (f < f1) {
+        slot = a.item_slot[f];
+        if (slot >= a.n_slots) {
+          bad |= kStBadSlot;
+        } else {
+          len = a.item_len ? a.item_len[f] : load32_any(a.ring + (size_t)slot * a.slot_size + 54);
+          if (len > a.slot_size - a.hl) { bad |= kStBadLen; len = 0; }
+        }
+      }
+      uint64_t tot;
+      uint64_t ex = block_exclusive_scan(len, wave_tot, &tot);
+      if (f < f1) {
+        u32x4 d = {slot, len, (uint32_t)(carry + ex), r};
+        a.desc[f] = d;
+      }
+      carry += tot;
+    }
+  } else {
+    const uint64_t size = a.sizes ? a.sizes[r] : a.fixed_size;
+    const uint64_t want = (size + a.mtu - 1) / a.mtu;
+    if (want != (uint64_t)(f1 - f0)) bad |= kStBadFrames;
+    for (uint32_t f = f0 + threadIdx.x; f < f1; f += kBlock) {
+      const uint64_t i = f - f0;
+      const uint64_t taken = i * a.mtu;
+      uint64_t rem = taken < size ? size - taken : 0;
+      uint32_t len = (uint32_t)(rem <= a.mtu ? rem : a.mtu);
+      uint32_t slot = a.item_slot[f];
+      uint32_t owner = r;
+      if (slot >= a.n_slots) { bad |= kStBadSlot; owner = kInvalidReq; }
+      if ((bad & kStBadFrames) || size > 0xffffffffull) owner = kInvalidReq;
+      u32x4 d = {slot, len, (uint32_t)taken, owner};
+      a.desc[f] = d;
+    }
+    carry = (bad & kStBadFrames) ? 0 : size;
+  }
+  if (carry > 0xffffffffull) bad |= kStBadSize;
+  if (!a.packed && carry > a.max_req_bytes) bad |= kStBadSize;
+  if (a.packed && carry > a.cap) bad |= kStBadSize;
+  if (bad) atomicOr(a.status, bad);
+
+  // hand the request total to whichever workgroup finishes last
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&a.req_size[r], carry, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();
+    const uint32_t t = atomicAdd(a.ticket, 1u);
+    is_last = (t == a.n_req - 1);
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+
+  // scan of the request totals through the bump ring:
+  //   ret = base + off; off = (off + size) % capacity
+  uint64_t run = a.packed ? *a.cursor % a.cap : 0;
+  for (uint32_t base = 0; base < a.n_req; base += kBlock) {
+    const uint32_t q = base + threadIdx.x;
+    uint64_t sz = 0;
+    if (q < a.n_req) sz = __hip_atomic_load(&a.req_size[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t tot;
+    uint64_t ex = block_exclusive_scan(sz, wave_tot, &tot);
+    if (q < a.n_req) {
+      uint64_t off = a.packed ? (run + ex) % a.cap : 0;
+      a.req_off[q] = off;
+      if (a.offsets_out) a.offsets_out[q] = off;
+    }
+    run += tot;
+    if (a.packed) run %= a.cap;
+  }
+  if (threadIdx.x == 0) {
+    if (a.packed) {
+      *a.cursor = run;
+      if (a.offsets_out) a.offsets_out[a.n_req] = run;
+    }
+    *a.ticket = 0;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gather / scatter
+// ---------------------------------------------------------------------------
+
+// Which item a wavefront works on.  Workgroups are dealt round-robin to the
+// eight XCDs, each with its own L2; giving XCD x the x-th contiguous eighth of
+// the items keeps neighbouring runs -- which share the cache lines at their
+// common destination boundary -- in one L2.
+__device__ __forceinline__ uint32_t item_of_wave(uint32_t n_groups_per_xcd, bool remap)
+{
+  uint32_t g = blockIdx.x;
+  if (remap) g = (blockIdx.x % kXcds) * n_groups_per_xcd + blockIdx.x / kXcds;
+  return g * kWavesPerBlock + threadIdx.x / kWave;
+}
+
+struct GatherArgs {
+  const u32x4 *desc;
+  const uint64_t *req_off;
+  const uint8_t *ring;
+  uint32_t slot_size;
+  uint32_t hl;
+  uint32_t n_items;
+  uint32_t groups_per_xcd;
+  uint32_t remap;
+  const uint32_t *status;
+  AppDev app;
+};
+
+// Move [off, off+len) of request r's byte stream between a packet payload and
+// the application buffers.  TO_APP: packet -> app.
+template <bool TO_APP, bool CSUM>
+__device__ __forceinline__ uint32_t move_run(const AppDev &app, uint64_t req_off, uint32_t r,
+                                             uint32_t off, uint8_t *pkt, uint32_t len, uint32_t lane)
+{
+  uint32_t acc = 0;
+  if (app.n_tensors == 0) {
+    const uint64_t o = req_off + off;  // < 2 * cap
+    if ((uint64_t)off + len > app.cap) return 0;  // request larger than the arena: refused by k_prep
+    if (app.mirrored || o + len <= app.cap) {
+      uint8_t *p = app.arena + o;
+      if (!app.mirrored && o >= app.cap) p -= app.cap;
+      acc = TO_APP ? copy_run<CSUM>(pkt, p, len, lane) : copy_run<CSUM>(p, pkt, len, lane);
+    } else {
+      copy_run_wrapped(pkt, app.arena, app.cap, o, len, lane, TO_APP, pkt);
+      if (CSUM) {
+        for (uint32_t i = lane; i < len; i += kWave) {
+          uint32_t b = pkt[i];  // this lane wrote it
+          acc += ((uintptr_t)(pkt + i) & 1u) ? (b << 8) : b;
+        }
+      }
+    }
+    return acc;
+  }
+  uint64_t t0 = 0;
+  uint32_t done = 0;
+  for (uint32_t t = 0; t < app.n_tensors && done < len; t++) {
+    const uint64_t t1 = t0 + app.tensor_size[t];
+    const uint64_t cur = (uint64_t)off + done;
+    if (cur < t1) {
+      const uint64_t room = t1 - cur;
+      const uint32_t n = room < (uint64_t)(len - done) ? (uint32_t)room : (len - done);
+      uint8_t *p = app.tensor_base[t] + (uint64_t)r * app.tensor_size[t] + (cur - t0);
+      if (TO_APP) copy_run<false>(pkt + done, p, n, lane);
+      else acc += copy_run<CSUM>(p, pkt + done, n, lane);
+      done += n;
+    }
+    t0 = t1;
+  }
+  return acc;
+}
+
+__global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
+{
+  const uint32_t item = item_of_wave(a.groups_per_xcd, a.remap != 0);
+  if (item >= a.n_items) return;
+  if (*a.status) return;  // k_prep refused the batch: move nothing
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const u32x4 d = a.desc[item];
+  if (d[1] == 0 || d[3] == kInvalidReq) return;
+  const uint64_t ro = a.app.n_tensors == 0 ? a.req_off[d[3]] : 0;
+  uint8_t *pkt = const_cast<uint8_t *>(a.ring) + (size_t)d[0] * a.slot_size + a.hl;
+  move_run<true, false>(a.app, ro, d[3], d[2], pkt, d[1], lane);
+}
+
+struct ScatterArgs {
+  const u32x4 *desc;
+  const uint64_t *req_off;
+  const uint32_t *first;         // resp_first CSR (for frag_idx / num_frags)
+  const uint32_t *hdr_src_slot;
+  const uint8_t *rx;
+  uint32_t rx_slot_size;
+  uint32_t rx_n_slots;
+  uint8_t *tx;
+  uint32_t tx_slot_size;
+  uint32_t hl;
+  uint32_t ref64;
+  uint32_t flags;
+  uint32_t n_items;
+  uint32_t groups_per_xcd;
+  uint32_t remap;
+  uint32_t *status;
+  AppDev app;
+};
+
+template <bool FULL_CSUM>
+__global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
+{
+  const uint32_t item = item_of_wave(a.groups_per_xcd, a.remap != 0);
+  if (item >= a.n_items) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  if (*a.status) return;  // k_prep refused the batch: move nothing
+  const u32x4 d = a.desc[item];
+  const uint32_t r = d[3];
+  if (r == kInvalidReq) return;
+  const uint32_t f0 = a.first[r];
+  const uint32_t nf = a.first[r + 1] - f0;
+  uint32_t hs = a.hdr_src_slot[item];
+  if (hs >= a.rx_n_slots) {
+    if (lane == 0) atomicOr(a.status, kStBadSlot);
+    return;
+  }
+  const uint64_t ro = a.app.n_tensors == 0 ? a.req_off[r] : 0;
+  uint8_t *slot = a.tx + (size_t)d[0] * a.tx_slot_size;
+
+  // read the request header before anything of this slot is overwritten
+  // (the TX slot may be the very slot the header comes from)
+  const uint8_t *hin = a.rx + (size_t)hs * a.rx_slot_size;
+  HdrFields hf{a.hl, a.ref64, a.flags, item - f0, nf, d[1]};
+  uint32_t hb = 0;
+  if (!FULL_CSUM) hb = hdr_rewrite(hin, lane, hf, 0);
+
+  uint32_t acc = 0;
+  if (d[1]) acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
+  if (FULL_CSUM) {
+    // the payload copy wrote past the header only, so in place the request
+    // header is still intact here
+    const uint32_t psum = wave_sum(acc);
+    hb = hdr_rewrite(hin, lane, hf, psum);
+  }
+  if (lane < a.hl) slot[lane] = (uint8_t)hb;
+}
+
+// ---------------------------------------------------------------------------
+// per-request entry points
+// ---------------------------------------------------------------------------
+
+struct Run {
+  uint64_t src;
+  uint64_t dst;
+  uint64_t len;
+};
+
+__global__ __launch_bounds__(kBlock) void k_copy_runs(const Run *runs, uint32_t n)
+{
+  const uint32_t item = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (item >= n) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const Run r = runs[item];
+  copy_run<false>(reinterpret_cast<const uint8_t *>(r.src), reinterpret_cast<uint8_t *>(r.dst),
+                  (uint32_t)r.len, lane);
+}
+
+__global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, uint32_t n,
+                                                      uint32_t hl, uint32_t ref64, uint32_t flags,
+                                                      uint64_t payload_size, uint32_t mtu)
+{
+  const uint32_t item = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (item >= n) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint8_t *h = reinterpret_cast<uint8_t *>(hdr_ptrs[item]);
+  const uint64_t taken = (uint64_t)item * mtu;
+  const uint64_t rem = taken < payload_size ? payload_size - taken : 0;
+  HdrFields hf{hl, ref64, flags & ~(1u << 2), item, n, (uint32_t)(rem <= mtu ? rem : mtu)};
+  const uint32_t b = hdr_rewrite(h, lane, hf, 0);
+  if (lane < hl) h[lane] = (uint8_t)b;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+struct EvPair {
+  hipEvent_t a, b;
+  int which;
+};
+
+struct sg_hip_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  bool own_stream = false;
+  uint32_t max_reqs = 0, max_frames = 0;
+  // device scratch
+  u32x4 *desc = nullptr;
+  uint64_t *req_size = nullptr;
+  uint64_t *req_off = nullptr;
+  uint64_t *cursors = nullptr;  // [0] request arena, [1] response arena
+  uint32_t *ticket = nullptr;
+  uint32_t *status = nullptr;
+  // pinned staging for the per-request entry points (device reads it in place)
+  Run *h_runs = nullptr;
+  uint32_t h_runs_cap = 0;
+  uint64_t *h_ptrs = nullptr;
+  uint32_t *h_status = nullptr;  // pinned mirror of status
+  // profiling
+  bool profiling = false;
+  std::vector<EvPair> ev_used, ev_free;
+  double prof_ms[5] = {0, 0, 0, 0, 0};
+  uint64_t prof_n[5] = {0, 0, 0, 0, 0};
+  char err[512] = {0};
+};
+
+static char g_create_err[512];
+
+static int fail(sg_hip_ctx *c, int code, const char *fmt, ...)
+{
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(c ? c->err : g_create_err, 512, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HIP_TRY(c, call)                                                                      \
+  do {                                                                                        \
+    hipError_t e_ = (call);                                                                   \
+    if (e_ != hipSuccess)                                                                     \
+      return fail((c), SG_E_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_),       \
+                  __FILE__, __LINE__);                                                        \
+  } while (0)
+
+namespace {
+
+struct DeviceGuard {
+  int prev = -1;
+  bool ok = false;
+  explicit DeviceGuard(int dev)
+  {
+    if (hipGetDevice(&prev) == hipSuccess) {
+      if (prev == dev) ok = true;
+      else ok = hipSetDevice(dev) == hipSuccess;
+    }
+  }
+  ~DeviceGuard()
+  {
+    if (ok && prev >= 0) (void)hipSetDevice(prev);
+  }
+};
+
+uint32_t hdr_len_of(uint32_t profile) { return profile == SG_HDR_REF64 ? 64u : 58u; }
+
+int check_ring(sg_hip_ctx *c, const sg_ring_desc &r, const char *what)
+{
+  if (!r.base || r.n_slots == 0) return fail(c, SG_E_INVAL, "%s ring: null base or no slots", what);
+  if (r.hdr_profile > SG_HDR_REF64) return fail(c, SG_E_INVAL, "%s ring: unknown header profile %u", what, r.hdr_profile);
+  if (r.slot_size < hdr_len_of(r.hdr_profile) || (r.slot_size & 1u))
+    return fail(c, SG_E_INVAL, "%s ring: slot size %u must be even and hold a header", what, r.slot_size);
+  if ((uintptr_t)r.base & 1u) return fail(c, SG_E_INVAL, "%s ring: base address must be even", what);
+  return SG_OK;
+}
+
+int check_app(sg_hip_ctx *c, const sg_app_desc &a, AppDev *out, uint64_t *max_req_bytes)
+{
+  if (a.n_tensors > SG_MAX_TENSORS) return fail(c, SG_E_INVAL, "n_tensors %u > %d", a.n_tensors, SG_MAX_TENSORS);
+  memset(out, 0, sizeof *out);
+  out->n_tensors = a.n_tensors;
+  *max_req_bytes = 0;
+  if (a.n_tensors == 0) {
+    if (!a.arena || a.arena_cap == 0) return fail(c, SG_E_INVAL, "packed mode needs an arena and a capacity");
+    out->arena = static_cast<uint8_t *>(a.arena);
+    out->cap = a.arena_cap;
+    out->mirrored = a.arena_mirrored ? 1u : 0u;
+    return SG_OK;
+  }
+  for (uint32_t t = 0; t < a.n_tensors; t++) {
+    if (!a.tensor_base[t] || a.tensor_size[t] == 0)
+      return fail(c, SG_E_INVAL, "tensor %u: null base or zero size", t);
+    out->tensor_base[t] = static_cast<uint8_t *>(a.tensor_base[t]);
+    out->tensor_size[t] = a.tensor_size[t];
+    *max_req_bytes += a.tensor_size[t];
+  }
+  return SG_OK;
+}
+
+// Launch geometry for one wavefront per item with the XCD-aware order.
+void geometry(uint32_t n_items, bool remap, uint32_t *grid, uint32_t *groups_per_xcd)
+{
+  const uint32_t groups = (n_items + kWavesPerBlock - 1) / kWavesPerBlock;
+  if (remap && groups >= 2 * kXcds) {
+    *groups_per_xcd = (groups + kXcds - 1) / kXcds;
+    *grid = *groups_per_xcd * kXcds;
+  } else {
+    *groups_per_xcd = 0;
+    *grid = groups;
+  }
+}
+
+int prof_begin(sg_hip_ctx *c, int which)
+{
+  if (!c->profiling) return SG_OK;
+  EvPair p;
+  if (!c->ev_free.empty()) {
+    p = c->ev_free.back();
+    c->ev_free.pop_back();
+  } else {
+    HIP_TRY(c, hipEventCreate(&p.a));
+    HIP_TRY(c, hipEventCreate(&p.b));
+  }
+  p.which = which;
+  HIP_TRY(c, hipEventRecord(p.a, c->stream));
+  c->ev_used.push_back(p);
+  return SG_OK;
+}
+
+int prof_end(sg_hip_ctx *c)
+{
+  if (!c->profiling) return SG_OK;
+  HIP_TRY(c, hipEventRecord(c->ev_used.back().b, c->stream));
+  return SG_OK;
+}
+
+int prof_drain(sg_hip_ctx *c)
+{
+  for (EvPair &p : c->ev_used) {
+    float ms = 0.f;
+    HIP_TRY(c, hipEventElapsedTime(&ms, p.a, p.b));
+    c->prof_ms[p.which] += ms;
+    c->prof_n[p.which] += 1;
+    c->ev_free.push_back(p);
+  }
+  c->ev_used.clear();
+  return SG_OK;
+}
+
+int finish(sg_hip_ctx *c, uint32_t flags)
+{
+  HIP_TRY(c, hipGetLastError());
+  if (flags & SG_F_ASYNC) {
+    // keep the event list bounded on long asynchronous runs
+    if (c->profiling && c->ev_used.size() > 4096) return sg_hip_sync(c);
+    return SG_OK;
+  }
+  return sg_hip_sync(c);
+}
+
+}  // namespace
+
+extern "C" {
+
+int sg_hip_abi_version(void) { return SG_HIP_ABI_VERSION; }
+
+const char *sg_hip_last_error(const sg_hip_ctx *ctx) { return ctx ? ctx->err : g_create_err; }
+
+void *sg_hip_stream(sg_hip_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
+{
+  int n_dev = 0;
+  HIP_TRY(nullptr, hipGetDeviceCount(&n_dev));
+  if (device_id < 0 || device_id >= n_dev)
+    return fail(nullptr, SG_E_INVAL, "device %d not present (%d devices)", device_id, n_dev);
+  c->device = device_id;
+  DeviceGuard g(device_id);
+  if (!g.ok) return fail(nullptr, SG_E_HIP, "cannot select device %d", device_id);
+  hipDeviceProp_t prop;
+  HIP_TRY(nullptr, hipGetDeviceProperties(&prop, device_id));
+  if (prop.warpSize != (int)kWave)
+    return fail(nullptr, SG_E_INVAL, "device %d has %d-wide wavefronts; this library is built for 64", device_id, prop.warpSize);
+  c->max_reqs = cfg && cfg->max_reqs ? cfg->max_reqs : 4096u;
+  c->max_frames = cfg && cfg->max_frames ? cfg->max_frames : 65536u;
+  if (cfg && cfg->stream) {
+    c->stream = static_cast<hipStream_t>(cfg->stream);
+  } else {
+    HIP_TRY(nullptr, hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    c->own_stream = true;
+  }
+  HIP_TRY(nullptr, hipMalloc(&c->desc, sizeof(u32x4) * (size_t)c->max_frames));
+  HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
+  HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
+  HIP_TRY(nullptr, hipMalloc(&c->cursors, 2 * sizeof(uint64_t)));
+  HIP_TRY(nullptr, hipMalloc(&c->ticket, sizeof(uint32_t)));
+  HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
+  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 2 * sizeof(uint64_t), c->stream));
+  HIP_TRY(nullptr, hipMemsetAsync(c->ticket, 0, sizeof(uint32_t), c->stream));
+  HIP_TRY(nullptr, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
+  c->h_runs_cap = 8192;
+  HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
+  HIP_TRY(nullptr, hipHostMalloc(&c->h_ptrs, sizeof(uint64_t) * SG_MAX_BI_SIZE, hipHostMallocDefault));
+  HIP_TRY(nullptr, hipHostMalloc(&c->h_status, sizeof(uint32_t), hipHostMallocDefault));
+  HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
+  return SG_OK;
+}
+
+sg_hip_ctx *sg_hip_create(int device_id, const sg_hip_cfg *cfg)
+{
+  g_create_err[0] = 0;
+  if (cfg && cfg->struct_size != sizeof(sg_hip_cfg)) {
+    fail(nullptr, SG_E_INVAL, "sg_hip_cfg.struct_size %u != %zu", cfg->struct_size, sizeof(sg_hip_cfg));
+    return nullptr;
+  }
+  sg_hip_ctx *c = new (std::nothrow) sg_hip_ctx();
+  if (!c) {
+    fail(nullptr, SG_E_NOMEM, "out of host memory");
+    return nullptr;
+  }
+  if (create_impl(c, device_id, cfg) != SG_OK) {
+    sg_hip_destroy(c);
+    return nullptr;
+  }
+  return c;
+}
+
+void sg_hip_destroy(sg_hip_ctx *c)
+{
+  if (!c) return;
+  DeviceGuard g(c->device);
+  if (c->stream) (void)hipStreamSynchronize(c->stream);
+  for (EvPair &p : c->ev_used) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+  for (EvPair &p : c->ev_free) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+  (void)hipFree(c->desc);
+  (void)hipFree(c->req_size);
+  (void)hipFree(c->req_off);
+  (void)hipFree(c->cursors);
+  (void)hipFree(c->ticket);
+  (void)hipFree(c->status);
+  if (c->h_runs) (void)hipHostFree(c->h_runs);
+  if (c->h_ptrs) (void)hipHostFree(c->h_ptrs);
+  if (c->h_status) (void)hipHostFree(c->h_status);
+  if (c->own_stream && c->stream) (void)hipStreamDestroy(c->stream);
+  delete c;
+}
+
+int sg_hip_sync(sg_hip_ctx *c)
+{
+  if (!c) return SG_E_INVAL;
+  DeviceGuard g(c->device);
+  HIP_TRY(c, hipMemcpyAsync(c->h_status, c->status, sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  int rc = prof_drain(c);
+  if (rc != SG_OK) return rc;
+  const uint32_t st = *c->h_status;
+  if (st) {
+    HIP_TRY(c, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return fail(c, SG_E_DATA, "kernel refused input:%s%s%s%s%s",
+                (st & kStBadSlot) ? " slot index beyond ring;" : "",
+                (st & kStBadLen) ? " fragment longer than a slot holds;" : "",
+                (st & kStBadSize) ? " request larger than its destination;" : "",
+                (st & kStBadFrames) ? " frame count disagrees with size/mtu;" : "",
+                (st & kStBadTable) ? " CSR table does not tile the items;" : "");
+  }
+  return SG_OK;
+}
+
+int sg_hip_set_cursor(sg_hip_ctx *c, int which, uint64_t value)
+{
+  if (!c || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
+  DeviceGuard g(c->device);
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  HIP_TRY(c, hipMemcpy(c->cursors + which, &value, sizeof value, hipMemcpyHostToDevice));
+  return SG_OK;
+}
+
+int sg_hip_get_cursor(sg_hip_ctx *c, int which, uint64_t *value)
+{
+  if (!c || !value || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
+  DeviceGuard g(c->device);
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  HIP_TRY(c, hipMemcpy(value, c->cursors + which, sizeof *value, hipMemcpyDeviceToHost));
+  return SG_OK;
+}
+
+int sg_hip_set_profiling(sg_hip_ctx *c, int on)
+{
+  if (!c) return SG_E_INVAL;
+  int rc = sg_hip_sync(c);
+  c->profiling = on != 0;
+  for (int i = 0; i < 5; i++) { c->prof_ms[i] = 0; c->prof_n[i] = 0; }
+  return rc;
+}
+
+int sg_hip_kernel_time(sg_hip_ctx *c, int which, double *total_ms, uint64_t *launches)
+{
+  if (!c || which < 0 || which > 4) return fail(c, SG_E_INVAL, "kernel index %d", which);
+  int rc = sg_hip_sync(c);
+  if (total_ms) *total_ms = c->prof_ms[which];
+  if (launches) *launches = c->prof_n[which];
+  return rc;
+}
+
+// ---- per-request ------------------------------------------------------------
+
+// Runs longer than this are cut so that no single wavefront walks megabytes.
+static const uint64_t kRunChunk = 16384;
+
+static int copy_skb(sg_hip_ctx *c, const sg_sk_buf *skb)
+{
+  if (!c || !skb) return fail(c, SG_E_INVAL, "null argument");
+  if (skb->num_items > SG_MAX_BI_SIZE - 1)
+    return fail(c, SG_E_INVAL, "run table holds %llu runs; len[] has room for %d",
+                (unsigned long long)skb->num_items, SG_MAX_BI_SIZE - 1);
+  DeviceGuard g(c->device);
+  // the pinned staging buffer is reused: the previous launch must have read it
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  uint32_t n = 0;
+  for (uint64_t i = 0; i < skb->num_items; i++) {
+    uint64_t src = skb->i_buf[i], dst = skb->o_buf[i], len = skb->len[i];
+    if (len && (!src || !dst)) return fail(c, SG_E_INVAL, "run %llu has a null address", (unsigned long long)i);
+    while (len) {
+      uint64_t piece = len;
+      if (piece > kRunChunk) {
+        // cut where the destination is 16-byte aligned so later pieces need no head bytes
+        piece = kRunChunk - (dst & 15u);
+      }
+      if (n == c->h_runs_cap) {
+        // flush what is staged and start over
+        int rc = prof_begin(c, 3);
+        if (rc != SG_OK) return rc;
+        k_copy_runs<<<(n + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(c->h_runs, n);
+        rc = prof_end(c);
+        if (rc != SG_OK) return rc;
+        HIP_TRY(c, hipStreamSynchronize(c->stream));
+        n = 0;
+      }
+      c->h_runs[n++] = Run{src, dst, piece};
+      src += piece; dst += piece; len -= piece;
+    }
+  }
+  if (n) {
+    int rc = prof_begin(c, 3);
+    if (rc != SG_OK) return rc;
+    k_copy_runs<<<(n + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(c->h_runs, n);
+    rc = prof_end(c);
+    if (rc != SG_OK) return rc;
+  }
+  return finish(c, 0);
+}
+
+int sg_hip_gather(sg_hip_ctx *c, const sg_sk_buf *skb) { return copy_skb(c, skb); }
+int sg_hip_scatter(sg_hip_ctx *c, const sg_sk_buf *skb) { return copy_skb(c, skb); }
+
+int sg_hip_swap_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, uint32_t profile, uint64_t payload_size,
+                     uint32_t mtu, uint32_t flags)
+{
+  if (!c || !hdrs) return fail(c, SG_E_INVAL, "null argument");
+  if (profile > SG_HDR_REF64) return fail(c, SG_E_INVAL, "unknown header profile %u", profile);
+  if (hdrs->num_items > SG_MAX_BI_SIZE) return fail(c, SG_E_INVAL, "header table holds %u entries", hdrs->num_items);
+  if (mtu == 0) return fail(c, SG_E_INVAL, "mtu is zero");
+  if (flags & SG_F_UDP_CSUM_FULL) return fail(c, SG_E_INVAL, "a header-only rewrite cannot finish the UDP checksum");
+  const uint32_t n = hdrs->num_items;
+  if (n == 0) return SG_OK;
+  DeviceGuard g(c->device);
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  for (uint32_t i = 0; i < n; i++) {
+    if (!hdrs->burst_items[i]) return fail(c, SG_E_INVAL, "header %u is null", i);
+    c->h_ptrs[i] = hdrs->burst_items[i];
+  }
+  int rc = prof_begin(c, 4);
+  if (rc != SG_OK) return rc;
+  k_swap_hdrs<<<(n + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(
+      c->h_ptrs, n, hdr_len_of(profile), profile == SG_HDR_REF64, flags & 0xfu, payload_size, mtu);
+  rc = prof_end(c);
+  if (rc != SG_OK) return rc;
+  return finish(c, 0);
+}
+
+// ---- batched ------------------------------------------------------------------
+
+int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
+{
+  if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
+  int rc = check_ring(c, a->ring, "rx");
+  if (rc != SG_OK) return rc;
+  if (a->n_req == 0) return SG_OK;
+  if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
+  if (a->n_frags > c->max_frames) return fail(c, SG_E_INVAL, "n_frags %u > max_frames %u of this context", a->n_frags, c->max_frames);
+  if (!a->frag_slot || !a->req_first) return fail(c, SG_E_INVAL, "null fragment tables");
+  if (!a->frag_len && a->ring.hdr_profile != SG_HDR_BL58)
+    return fail(c, SG_E_INVAL, "REF64 headers carry no payload length: frag_len is required");
+  AppDev app;
+  uint64_t max_req_bytes;
+  rc = check_app(c, a->app, &app, &max_req_bytes);
+  if (rc != SG_OK) return rc;
+  DeviceGuard g(c->device);
+
+  PrepArgs p;
+  memset(&p, 0, sizeof p);
+  p.mode = 0;
+  p.n_req = a->n_req;
+  p.ring = static_cast<const uint8_t *>(a->ring.base);
+  p.n_slots = a->ring.n_slots;
+  p.slot_size = a->ring.slot_size;
+  p.hl = hdr_len_of(a->ring.hdr_profile);
+  p.item_slot = a->frag_slot;
+  p.item_len = a->frag_len;
+  p.first = a->req_first;
+  p.n_items = a->n_frags;
+  p.packed = app.n_tensors == 0;
+  p.cap = app.cap;
+  p.max_req_bytes = max_req_bytes;
+  p.desc = c->desc;
+  p.req_size = c->req_size;
+  p.req_off = c->req_off;
+  p.cursor = c->cursors + 0;
+  p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
+  p.ticket = c->ticket;
+  p.status = c->status;
+  rc = prof_begin(c, 0);
+  if (rc != SG_OK) return rc;
+  k_prep<<<a->n_req, kBlock, 0, c->stream>>>(p);
+  rc = prof_end(c);
+  if (rc != SG_OK) return rc;
+
+  if (a->n_frags) {
+    GatherArgs ga;
+    memset(&ga, 0, sizeof ga);
+    ga.desc = c->desc;
+    ga.req_off = c->req_off;
+    ga.ring = p.ring;
+    ga.slot_size = p.slot_size;
+    ga.hl = p.hl;
+    ga.n_items = a->n_frags;
+    ga.status = c->status;
+    ga.app = app;
+    uint32_t grid;
+    geometry(a->n_frags, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.groups_per_xcd);
+    ga.remap = ga.groups_per_xcd != 0;
+    rc = prof_begin(c, 1);
+    if (rc != SG_OK) return rc;
+    k_gather<<<grid, kBlock, 0, c->stream>>>(ga);
+    rc = prof_end(c);
+    if (rc != SG_OK) return rc;
+  }
+  return finish(c, a->flags);
+}
+
+int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
+{
+  if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
+  int rc = check_ring(c, a->rx, "rx");
+  if (rc != SG_OK) return rc;
+  rc = check_ring(c, a->tx, "tx");
+  if (rc != SG_OK) return rc;
+  if (a->rx.hdr_profile != a->tx.hdr_profile) return fail(c, SG_E_INVAL, "rx and tx rings differ in header profile");
+  if (a->n_req == 0) return SG_OK;
+  if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
+  if (a->n_frames > c->max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u of this context", a->n_frames, c->max_frames);
+  if (!a->tx_slot || !a->hdr_src_slot || !a->resp_first) return fail(c, SG_E_INVAL, "null frame tables");
+  const uint32_t hl = hdr_len_of(a->tx.hdr_profile);
+  if (a->mtu == 0 || (uint64_t)a->mtu + hl > a->tx.slot_size)
+    return fail(c, SG_E_INVAL, "mtu %u + %u header bytes does not fit a %u-byte slot", a->mtu, hl, a->tx.slot_size);
+  if ((uint64_t)a->mtu + (hl - 42u) + 28u > 0xffffu) return fail(c, SG_E_INVAL, "mtu %u overflows the IPv4 length field", a->mtu);
+  AppDev app;
+  uint64_t max_req_bytes;
+  rc = check_app(c, a->app, &app, &max_req_bytes);
+  if (rc != SG_OK) return rc;
+  DeviceGuard g(c->device);
+
+  PrepArgs p;
+  memset(&p, 0, sizeof p);
+  p.mode = 1;
+  p.n_req = a->n_req;
+  p.n_slots = a->tx.n_slots;
+  p.slot_size = a->tx.slot_size;
+  p.hl = hl;
+  p.mtu = a->mtu;
+  p.item_slot = a->tx_slot;
+  p.first = a->resp_first;
+  p.sizes = a->resp_size;
+  p.fixed_size = a->fixed_resp_size;
+  p.n_items = a->n_frames;
+  p.packed = app.n_tensors == 0;
+  p.cap = app.cap;
+  p.max_req_bytes = max_req_bytes;
+  p.desc = c->desc;
+  p.req_size = c->req_size;
+  p.req_off = c->req_off;
+  p.cursor = c->cursors + 1;
+  p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
+  p.ticket = c->ticket;
+  p.status = c->status;
+  rc = prof_begin(c, 0);
+  if (rc != SG_OK) return rc;
+  k_prep<<<a->n_req, kBlock, 0, c->stream>>>(p);
+  rc = prof_end(c);
+  if (rc != SG_OK) return rc;
+
+  if (a->n_frames) {
+    ScatterArgs sa;
+    memset(&sa, 0, sizeof sa);
+    sa.desc = c->desc;
+    sa.req_off = c->req_off;
+    sa.first = a->resp_first;
+    sa.hdr_src_slot = a->hdr_src_slot;
+    sa.rx = static_cast<const uint8_t *>(a->rx.base);
+    sa.rx_slot_size = a->rx.slot_size;
+    sa.rx_n_slots = a->rx.n_slots;
+    sa.tx = static_cast<uint8_t *>(a->tx.base);
+    sa.tx_slot_size = a->tx.slot_size;
+    sa.hl = hl;
+    sa.ref64 = a->tx.hdr_profile == SG_HDR_REF64;
+    sa.flags = a->flags & 0xfu;
+    sa.n_items = a->n_frames;
+    sa.status = c->status;
+    sa.app = app;
+    uint32_t grid;
+    geometry(a->n_frames, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.groups_per_xcd);
+    sa.remap = sa.groups_per_xcd != 0;
+    rc = prof_begin(c, 2);
+    if (rc != SG_OK) return rc;
+    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true><<<grid, kBlock, 0, c->stream>>>(sa);
+    else k_scatter<false><<<grid, kBlock, 0, c->stream>>>(sa);
+    rc = prof_end(c);
+    if (rc != SG_OK) return rc;
+  }
+  return finish(c, a->flags);
+}
+
+}  // extern "C"

@@ -1,0 +1,275 @@
+"""Thin Python face of the C ABI for tests, the smoke check and the benchmark.
+
+torch is used for device memory and streams only; every operation goes through
+``libsg_hip.so``.  Tables are int32 / int64 tensors holding the bit patterns of
+the ABI's uint32 / uint64 arrays.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import capi
+from .synth import Workload
+
+
+class SgError(RuntimeError):
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"sg_hip error {code}: {msg}")
+        self.code = code
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def to_dev(a: np.ndarray, device) -> torch.Tensor:
+    """Upload a numpy array, keeping its bits (uint32 -> int32, uint64 -> int64)."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    elif a.dtype == np.uint64:
+        a = a.view(np.int64)
+    return torch.from_numpy(a.copy()).to(device)
+
+
+@dataclass
+class RingRef:
+    buf: torch.Tensor  # uint8
+    n_slots: int
+    slot_size: int
+    profile: int
+
+    def desc(self) -> capi.RingDesc:
+        assert self.buf.dtype == torch.uint8 and self.buf.is_contiguous()
+        assert self.buf.numel() >= self.n_slots * self.slot_size
+        return capi.RingDesc(self.buf.data_ptr(), self.n_slots, self.slot_size, self.profile, 0)
+
+
+@dataclass
+class AppRef:
+    """Packed arena (``arena``, ``cap``) or tensor-major buffers (``tensors`` with
+    per-request ``sizes``)."""
+    arena: Optional[torch.Tensor] = None
+    cap: int = 0
+    mirrored: bool = False
+    tensors: Sequence[torch.Tensor] = ()
+    sizes: Sequence[int] = ()
+
+    def desc(self) -> capi.AppDesc:
+        d = capi.AppDesc()
+        d.n_tensors = len(self.tensors)
+        for i, (t, s) in enumerate(zip(self.tensors, self.sizes)):
+            d.tensor_base[i] = t.data_ptr()
+            d.tensor_size[i] = int(s)
+        if self.arena is not None:
+            d.arena = self.arena.data_ptr()
+            d.arena_cap = int(self.cap)
+        d.arena_mirrored = 1 if self.mirrored else 0
+        return d
+
+
+class SgContext:
+    def __init__(self, device: int = 0, max_reqs: int = 4096, max_frames: int = 65536,
+                 stream: Optional[int] = None):
+        self.lib = capi.load()
+        cfg = capi.Cfg(C.sizeof(capi.Cfg), max_reqs, max_frames, 0, stream)
+        self.h = self.lib.sg_hip_create(device, C.byref(cfg))
+        if not self.h:
+            raise SgError(capi.SG_E_HIP, self.lib.sg_hip_last_error(None).decode())
+        self.device = device
+
+    def close(self) -> None:
+        if getattr(self, "h", None):
+            self.lib.sg_hip_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, rc: int) -> None:
+        if rc != capi.SG_OK:
+            raise SgError(rc, self.lib.sg_hip_last_error(self.h).decode())
+
+    @property
+    def stream(self) -> int:
+        return int(self.lib.sg_hip_stream(self.h) or 0)
+
+    def sync(self) -> None:
+        self._check(self.lib.sg_hip_sync(self.h))
+
+    def set_cursor(self, which: int, value: int) -> None:
+        self._check(self.lib.sg_hip_set_cursor(self.h, which, value))
+
+    def get_cursor(self, which: int) -> int:
+        v = C.c_uint64(0)
+        self._check(self.lib.sg_hip_get_cursor(self.h, which, C.byref(v)))
+        return int(v.value)
+
+    def set_profiling(self, on: bool) -> None:
+        self._check(self.lib.sg_hip_set_profiling(self.h, 1 if on else 0))
+
+    def kernel_time(self, which: int):
+        ms, n = C.c_double(0), C.c_uint64(0)
+        self._check(self.lib.sg_hip_kernel_time(self.h, which, C.byref(ms), C.byref(n)))
+        return float(ms.value), int(n.value)
+
+    # -- batched -----------------------------------------------------------
+    def gather_batch(self, ring: RingRef, frag_slot: torch.Tensor, frag_len: Optional[torch.Tensor],
+                     req_first: torch.Tensor, n_req: int, n_frags: int, app: AppRef,
+                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0) -> None:
+        a = capi.GatherArgs()
+        a.ring = ring.desc()
+        a.frag_slot = frag_slot.data_ptr()
+        a.frag_len = frag_len.data_ptr() if frag_len is not None else None
+        a.req_first = req_first.data_ptr()
+        a.n_req = n_req
+        a.n_frags = n_frags
+        a.app = app.desc()
+        a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
+        a.flags = flags
+        self._check(self.lib.sg_hip_gather_batch(self.h, C.byref(a)))
+
+    def scatter_batch(self, rx: RingRef, tx: RingRef, tx_slot: torch.Tensor,
+                      hdr_src_slot: torch.Tensor, resp_first: torch.Tensor,
+                      resp_size: Optional[torch.Tensor], fixed_resp_size: int, n_req: int,
+                      n_frames: int, mtu: int, app: AppRef,
+                      offsets_out: Optional[torch.Tensor] = None, flags: int = 0) -> None:
+        a = capi.ScatterArgs()
+        a.rx = rx.desc()
+        a.tx = tx.desc()
+        a.tx_slot = tx_slot.data_ptr()
+        a.hdr_src_slot = hdr_src_slot.data_ptr()
+        a.resp_first = resp_first.data_ptr()
+        a.resp_size = resp_size.data_ptr() if resp_size is not None else None
+        a.fixed_resp_size = int(fixed_resp_size)
+        a.n_req = n_req
+        a.n_frames = n_frames
+        a.mtu = mtu
+        a.flags = flags
+        a.app = app.desc()
+        a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
+        self._check(self.lib.sg_hip_scatter_batch(self.h, C.byref(a)))
+
+    # -- per request ---------------------------------------------------------
+    def copy_runs(self, src: Sequence[int], dst: Sequence[int], lens: Sequence[int],
+                  scatter: bool = False) -> None:
+        skb = capi.SkBuf()
+        n = len(lens)
+        assert n <= capi.MAX_BI_SIZE - 1
+        for i in range(n):
+            skb.i_buf[i] = src[i]
+            skb.o_buf[i] = dst[i]
+            skb.len[i] = lens[i]
+        skb.num_items = n
+        fn = self.lib.sg_hip_scatter if scatter else self.lib.sg_hip_gather
+        self._check(fn(self.h, C.byref(skb)))
+
+    def swap_hdrs(self, hdr_ptrs: Sequence[int], profile: int, payload_size: int, mtu: int,
+                  flags: int) -> None:
+        hb = capi.HBufs()
+        for i, p in enumerate(hdr_ptrs):
+            hb.burst_items[i] = p
+        hb.num_items = len(hdr_ptrs)
+        self._check(self.lib.sg_hip_swap_hdrs(self.h, C.byref(hb), profile, payload_size, mtu, flags))
+
+
+class DeviceWorkload:
+    """A synthetic workload staged in one GPU's memory: the landing-zone ring,
+    the fragment tables and the application buffers."""
+
+    def __init__(self, w: Workload, device="cuda:0", arena_slack: int = 0, copies: int = 1):
+        """``copies`` > 1 lays that many copies of the ring (and of the tables,
+        slot indices shifted) side by side, so that one call moves ``copies``
+        batches and the working set outgrows the caches."""
+        self.w = w
+        self.copies = copies
+        dev = torch.device(device)
+        self.dev = dev
+        k = copies
+        self.n_req = w.n_req * k
+        self.n_frags = w.n_frags * k
+        self.n_frames = w.n_resp_frames * k
+        ring1 = torch.from_numpy(w.ring).to(dev)
+        self.ring = ring1.repeat(k) if k > 1 else ring1
+        self.rx = RingRef(self.ring, w.n_slots * k, w.slot_size, w.profile)
+
+        def tile_slots(a: np.ndarray, n_slots: int) -> np.ndarray:
+            return np.concatenate([a.astype(np.uint32) + np.uint32(i * n_slots) for i in range(k)])
+
+        def tile_csr(first: np.ndarray) -> np.ndarray:
+            body = [first[:-1].astype(np.uint32) + np.uint32(i * int(first[-1])) for i in range(k)]
+            return np.concatenate(body + [np.array([int(first[-1]) * k], dtype=np.uint32)])
+
+        self.frag_slot = to_dev(tile_slots(w.frag_slot, w.n_slots), dev)
+        self.frag_len = to_dev(np.tile(w.frag_len, k), dev)
+        self.req_first = to_dev(tile_csr(w.req_first), dev)
+        self.tx_slot = to_dev(tile_slots(w.tx_slot, w.tx_n_slots), dev)
+        self.hdr_src_slot = to_dev(tile_slots(w.hdr_src_slot, w.n_slots), dev)
+        self.resp_first = to_dev(tile_csr(w.resp_first), dev)
+        self.resp_size = to_dev(np.tile(w.resp_sizes, k), dev)
+        if w.tx_in_place:
+            self.tx_ring = self.ring
+        else:
+            t1 = torch.from_numpy(w.tx_ring_init).to(dev)
+            self.tx_ring = t1.repeat(k) if k > 1 else t1
+        self.tx = RingRef(self.tx_ring, w.tx_n_slots * k, w.slot_size, w.profile)
+
+        # request side application buffers
+        if w.in_tensor_sizes:
+            self.in_tensors = [torch.zeros(self.n_req * s, dtype=torch.uint8, device=dev)
+                               for s in w.in_tensor_sizes]
+            self.req_app = AppRef(tensors=self.in_tensors, sizes=w.in_tensor_sizes)
+            self.req_offsets = None
+        else:
+            cap = int(w.req_sizes.sum()) * k + arena_slack
+            self.req_arena = torch.zeros(max(cap, 16), dtype=torch.uint8, device=dev)
+            self.req_app = AppRef(arena=self.req_arena, cap=max(cap, 16))
+            self.req_offsets = torch.zeros(self.n_req + 1, dtype=torch.int64, device=dev)
+        # response side
+        resp1 = torch.from_numpy(w.resp_payload).to(dev)
+        if w.out_tensor_sizes:
+            assert len(w.out_tensor_sizes) == 1 or True
+            # responses concatenated in batch order are tensor-major already when there is one tensor
+            self.out_tensors = self._split_outputs(w, k, dev)
+            self.resp_app = AppRef(tensors=self.out_tensors, sizes=w.out_tensor_sizes)
+            self.resp_offsets = None
+        elif w.tx_in_place:
+            # echo: responses are read from where gather put the requests
+            self.resp_app = self.req_app
+            self.resp_offsets = torch.zeros(self.n_req + 1, dtype=torch.int64, device=dev)
+        else:
+            self.resp_arena = resp1.repeat(k) if k > 1 else resp1
+            cap = int(self.resp_arena.numel())
+            if cap < 16:
+                self.resp_arena = torch.zeros(16, dtype=torch.uint8, device=dev)
+            self.resp_app = AppRef(arena=self.resp_arena, cap=max(cap, 16))
+            self.resp_offsets = torch.zeros(self.n_req + 1, dtype=torch.int64, device=dev)
+
+    @staticmethod
+    def _split_outputs(w: Workload, k: int, dev) -> List[torch.Tensor]:
+        per_req = int(sum(w.out_tensor_sizes))
+        rp = w.resp_payload.reshape(w.n_req, per_req)
+        outs, o = [], 0
+        for s in w.out_tensor_sizes:
+            t = torch.from_numpy(np.ascontiguousarray(rp[:, o:o + s]).reshape(-1)).to(dev)
+            outs.append(t.repeat(k) if k > 1 else t)
+            o += s
+        return outs
+
+    def gather(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False) -> None:
+        ctx.gather_batch(self.rx, self.frag_slot, self.frag_len if use_frag_len else None,
+                         self.req_first, self.n_req, self.n_frags, self.req_app,
+                         self.req_offsets, flags)
+
+    def scatter(self, ctx: SgContext, flags: int = 0) -> None:
+        ctx.scatter_batch(self.rx, self.tx, self.tx_slot, self.hdr_src_slot, self.resp_first,
+                          self.resp_size, 0, self.n_req, self.n_frames, self.w.mtu, self.resp_app,
+                          self.resp_offsets, self.w.flags | flags)
