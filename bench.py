@@ -1,0 +1,246 @@
+#!/usr/bin/env python3
+"""Benchmark of the gather + scatter hot path on one MI355X.
+
+One step = one pass of the hot path (descriptor build, gather, descriptor
+build, scatter + header rewrite) over one call's worth of synthetic input that
+is already resident in HBM.  The default workload is the ResNet-50-sized one:
+16 requests x 602112 B in 431 frames of <= 1400 B, 2048-byte slots, frames
+permuted inside a request; `--batches-per-launch B` lays B such batches side by
+side in the ring so that one call moves B batches (B = 1 is the single-batch
+call).  Ring copies are rotated between steps so that reads come from HBM and
+not from the 256 MB memory-side cache.
+
+Prints ONE JSON line: whole-job GB/s over the algorithmic bytes
+(2*payload + 16*frames gather, 2*payload + 2*58*frames scatter), the roofline
+of the dominant kernel from HIP-event kernel times, requests/s of all five
+workloads and the CPU oracle timed on this host as a baseline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import threading
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", type=int, default=2, help="1..5")
+    ap.add_argument("--batches-per-launch", type=int, default=0,
+                    help="batches laid side by side per call (0: default of the workload)")
+    ap.add_argument("--rotate-mb", type=int, default=1024,
+                    help="rotate over ring copies until the working set exceeds this many MB")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip requests/s of the other workloads")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-remap", action="store_true", help="disable the XCD-aware launch order")
+    return ap.parse_args()
+
+
+DEFAULT_BPL = {1: 256, 2: 32, 3: 64, 4: 8, 5: 4}
+
+
+class Pool:
+    """R device copies of one workload, rotated between steps."""
+
+    def __init__(self, w, bpl: int, rotate_mb: int, extra_flags: int = 0):
+        from splitrpc_amd.engine import DeviceWorkload
+        per = (w.ring.nbytes + int(w.req_sizes.sum()) + w.tx_n_slots * w.slot_size
+               + int(w.resp_sizes.sum())) * bpl
+        r = max(2, min(64, -(-rotate_mb * (1 << 20) // max(per, 1))))
+        self.items = [DeviceWorkload(w, copies=bpl) for _ in range(r)]
+        self.w = w
+        self.bpl = bpl
+        self.extra_flags = extra_flags
+        self.gather_bytes = w.gather_bytes() * bpl
+        self.scatter_bytes = w.scatter_bytes() * bpl
+        self.n_req = w.n_req * bpl
+
+    def step(self, ctx, i: int, flags: int) -> None:
+        dw = self.items[i % len(self.items)]
+        dw.gather(ctx, flags | self.extra_flags)
+        dw.scatter(ctx, flags | self.extra_flags)
+
+
+def timed(ctx, pool: Pool, steps: int, warmup: int):
+    import torch
+    from splitrpc_amd import capi
+    for i in range(warmup):
+        pool.step(ctx, i, capi.F_ASYNC)
+    ctx.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        pool.step(ctx, warmup + i, capi.F_ASYNC)
+    ctx.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return dt / steps
+
+
+def kernel_times(ctx, pool: Pool, steps: int):
+    """Average duration of each kernel from HIP events recorded around every
+    launch on the stream the kernels run on."""
+    from splitrpc_amd import capi
+    ctx.set_profiling(True)
+    for i in range(steps):
+        pool.step(ctx, i, capi.F_ASYNC)
+    out = {}
+    for which, name in ((0, "k_prep"), (1, "k_gather"), (2, "k_scatter")):
+        ms, n = ctx.kernel_time(which)
+        out[name] = (ms / n if n else 0.0, n)
+    ctx.set_profiling(False)
+    return out
+
+
+def cpu_baseline(w, seconds: float):
+    """The CPU oracle (a restatement of the reference's CPU scatter-gather
+    path) timed single-threaded on this host over rotated ring copies."""
+    import numpy as np
+    import oracle
+    n_copies = max(2, min(16, (512 << 20) // max(w.ring.nbytes, 1)))
+    rings = [w.ring.copy() for _ in range(n_copies)]
+    txs = [w.tx_ring_init.copy() if w.tx_ring_init is not None else None for _ in range(n_copies)]
+    src = w.resp_payload
+    if w.out_tensor_sizes:
+        rp = w.resp_payload.reshape(w.n_req, int(sum(w.out_tensor_sizes)))
+        src, o = [], 0
+        for s in w.out_tensor_sizes:
+            src.append(np.ascontiguousarray(rp[:, o:o + s]).reshape(-1))
+            o += s
+    dst, _, _ = oracle.gather(w)  # destination reused by every pass
+    t_end = time.perf_counter() + seconds
+    it = 0
+    orig = w.ring
+    t0 = time.perf_counter()
+    while time.perf_counter() < t_end or it < 2:
+        k = it % n_copies
+        w.ring = rings[k]
+        arena, _, _ = oracle.gather(w, out=dst)
+        if w.tx_in_place:
+            oracle.scatter(w, rings[k], rings[k], arena)
+        else:
+            oracle.scatter(w, rings[k], txs[k], src)
+        it += 1
+    dt = time.perf_counter() - t0
+    w.ring = orig
+    bytes_per = w.gather_bytes() + w.scatter_bytes()
+    return {"value": round(bytes_per * it / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "requests_per_sec": round(w.n_req * it / dt, 1),
+            "sample": f"{it} passes of gather+scatter over one {w.name} batch "
+                      f"({w.n_req} requests), {n_copies} rotated ring copies, {dt:.1f} s, "
+                      "C oracle -O3, one thread"}
+
+
+def main() -> int:
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        return 2
+    import torch
+    from splitrpc_amd import capi, synth
+    from splitrpc_amd.engine import SgContext
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (cuda:0)", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    extra = capi.F_NO_XCD_REMAP if a.no_remap else 0
+    bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
+    w = synth.make_workload(a.workload)
+    ctx = SgContext(0, max_reqs=max(4096, w.n_req * bpl), max_frames=max(65536, max(w.n_frags, w.n_resp_frames) * bpl))
+    pool = Pool(w, bpl, a.rotate_mb, extra)
+
+    sec = timed(ctx, pool, a.steps, a.warmup)
+    kt = kernel_times(ctx, pool, min(a.steps, 100))
+    total_bytes = pool.gather_bytes + pool.scatter_bytes
+    value = total_bytes / sec / 1e9
+    dom = "k_gather" if pool.gather_bytes >= pool.scatter_bytes else "k_scatter"
+    dom_bytes = pool.gather_bytes if dom == "k_gather" else pool.scatter_bytes
+    dom_ms = kt[dom][0]
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+
+    # the single-batch call of the same workload, for the record
+    single = None
+    if bpl != 1:
+        p1 = Pool(w, 1, a.rotate_mb, extra)
+        s1 = timed(ctx, p1, a.steps, a.warmup)
+        k1 = kernel_times(ctx, p1, min(a.steps, 100))
+        b1 = p1.gather_bytes + p1.scatter_bytes
+        single = {"ms_per_step": round(s1 * 1e3, 5), "GBps": round(b1 / s1 / 1e9, 2),
+                  "requests_per_sec": round(p1.n_req / s1, 1),
+                  "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in k1.items()},
+                  "k_gather_GBps": round(p1.gather_bytes / (k1["k_gather"][0] * 1e-3) / 1e9, 1)
+                  if k1["k_gather"][0] > 0 else None}
+        del p1
+
+    rps = {WORKLOAD_NAMES[a.workload]: round(pool.n_req / sec, 1)}
+    sweep = {}
+    if not a.no_sweep:
+        for cfg in (1, 2, 3, 4, 5):
+            if cfg == a.workload:
+                continue
+            wc = synth.make_workload(cfg)
+            b = DEFAULT_BPL[cfg]
+            c2 = SgContext(0, max_reqs=max(4096, wc.n_req * b),
+                           max_frames=max(65536, max(wc.n_frags, wc.n_resp_frames) * b))
+            pc = Pool(wc, b, a.rotate_mb, extra)
+            sc = timed(c2, pc, max(20, a.steps // 4), max(5, a.warmup // 4))
+            rps[wc.name] = round(pc.n_req / sc, 1)
+            sweep[wc.name] = {"batches_per_launch": b, "ms_per_step": round(sc * 1e3, 5),
+                              "GBps": round((pc.gather_bytes + pc.scatter_bytes) / sc / 1e9, 2)}
+            del pc
+            c2.close()
+            torch.cuda.empty_cache()
+
+    out = {
+        "metric": "gather+scatter GB/s (algorithmic bytes) on 1 MI355X",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(sec * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: {w.n_req} requests x {int(w.req_sizes[0])} B in "
+                               f"{w.n_frags // w.n_req} frames of <= {w.mtu} B, {w.slot_size}-B slots, "
+                               f"{w.n_resp_frames // w.n_req} response frames per request",
+                   "batches_per_launch": bpl, "rotated_ring_copies": len(pool.items),
+                   "requests_per_step": pool.n_req, "header_profile": "BL58",
+                   "flags": w.flags},
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "requests_per_sec": rps,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3)},
+        "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in kt.items()},
+        "single_batch_call": single,
+        "other_workloads": sweep,
+    }
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(w, a.cpu_seconds)
+    print(json.dumps(out))
+    ctx.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

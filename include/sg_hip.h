@@ -129,6 +129,11 @@ typedef struct sg_gather_args {
   uint64_t *offsets_out; /* device, n_req + 1 arena offsets (packed mode), or NULL */
   uint32_t flags;
   uint32_t reserved;
+  uint64_t fixed_req_size; /* non-zero: every request must total exactly this many bytes (the
+                              reference's server-wide request size, is_rr_ready,
+                              src/p2p_rpc_rr_ng.h:107-110); a batch holding another size is
+                              refused with SG_E_DATA.  0: sizes are whatever the fragments add
+                              up to and offsets come from a prefix scan */
 } sg_gather_args;
 
 /* One scatter batch.  Response r has resp_size[r] bytes (fixed_resp_size when

@@ -149,11 +149,13 @@ def _app(tensor_sizes, tensors, arena: Optional[np.ndarray], cap: int) -> AppBuf
     return a
 
 
-def gather(w, arena_cap: Optional[int] = None, cursor: int = 0, use_frag_len: bool = True):
+def gather(w, arena_cap: Optional[int] = None, cursor: int = 0, use_frag_len: bool = True,
+           out=None):
     """Run the CPU gather composite on workload ``w``.
 
     Packed mode returns (arena bytes, offsets[n_req+1], cursor_after);
-    tensor-major mode returns (list of tensors, None, cursor)."""
+    tensor-major mode returns (list of tensors, None, cursor).  ``out`` reuses
+    a destination (arena array or tensor list) instead of allocating one."""
     L = lib()
     ring = _ring(w.ring, w.n_slots, w.slot_size, w.profile)
     fl = np.ascontiguousarray(w.frag_len, dtype=np.uint32) if use_frag_len else None
@@ -161,13 +163,14 @@ def gather(w, arena_cap: Optional[int] = None, cursor: int = 0, use_frag_len: bo
     rf = np.ascontiguousarray(w.req_first, dtype=np.uint32)
     cur = np.array([cursor], dtype=np.uint64)
     if w.in_tensor_sizes:
-        tensors = [np.zeros(w.n_req * s, dtype=np.uint8) for s in w.in_tensor_sizes]
+        tensors = out if out is not None else [np.zeros(w.n_req * s, dtype=np.uint8)
+                                               for s in w.in_tensor_sizes]
         app = _app(w.in_tensor_sizes, tensors, None, 0)
         rc = L.sgo_gather_batch(C.byref(ring), _p(fs), _p(fl), _p(rf), w.n_req, C.byref(app), _p(cur), None)
         assert rc >= 0
         return tensors, None, int(cur[0])
     cap = int(arena_cap if arena_cap is not None else max(int(w.req_sizes.sum()), 1))
-    arena = np.zeros(cap, dtype=np.uint8)
+    arena = out if out is not None else np.zeros(cap, dtype=np.uint8)
     offs = np.zeros(w.n_req + 1, dtype=np.uint64)
     app = _app([], [], arena, cap)
     rc = L.sgo_gather_batch(C.byref(ring), _p(fs), _p(fl), _p(rf), w.n_req, C.byref(app), _p(cur), _p(offs))

@@ -71,7 +71,7 @@ class GatherArgs(C.Structure):
     _fields_ = [("ring", RingDesc), ("frag_slot", C.c_void_p), ("frag_len", C.c_void_p),
                 ("req_first", C.c_void_p), ("n_req", C.c_uint32), ("n_frags", C.c_uint32),
                 ("app", AppDesc), ("offsets_out", C.c_void_p), ("flags", C.c_uint32),
-                ("reserved", C.c_uint32)]
+                ("reserved", C.c_uint32), ("fixed_req_size", C.c_uint64)]
 
 
 class ScatterArgs(C.Structure):

@@ -59,6 +59,13 @@ __device__ __forceinline__ uint32_t wave_sum(uint32_t v)
   return v;
 }
 
+__device__ __forceinline__ uint32_t wave_or(uint32_t v)
+{
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v |= __shfl_xor(v, m, 64);
+  return v;
+}
+
 __device__ __forceinline__ uint32_t fold16(uint32_t s)
 {
   s = (s & 0xffffu) + (s >> 16);
@@ -66,10 +73,79 @@ __device__ __forceinline__ uint32_t fold16(uint32_t s)
   return s;
 }
 
+// Lane i receives lane i+1's value (lane 63 receives 0): DPP wave shift left
+// by one, a GFX9-family cross-lane move that needs no LDS.
+__device__ __forceinline__ uint32_t wave_shl1(uint32_t v)
+{
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x130, 0xf, 0xf, false);
+}
+
+// Bytes [p, p+16) of the 32-byte window {lo, hi}; 0 < p < 16.
+template <int Q>
+__device__ __forceinline__ u32x4 funnel_q(u32x4 lo, u32x4 hi, uint32_t bs)
+{
+  const uint32_t D[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  u32x4 o;
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    o[j] = __builtin_amdgcn_alignbyte(D[Q + j + 1 > 7 ? 7 : Q + j + 1], D[Q + j], bs);
+  return o;
+}
+
+__device__ __forceinline__ u32x4 funnel(u32x4 lo, u32x4 hi, uint32_t p)
+{
+  const uint32_t bs = p & 3u;
+  switch (p >> 2) {
+    case 0: return funnel_q<0>(lo, hi, bs);
+    case 1: return funnel_q<1>(lo, hi, bs);
+    case 2: return funnel_q<2>(lo, hi, bs);
+    default: return funnel_q<3>(lo, hi, bs);
+  }
+}
+
+// N x 63 destination chunks starting at chunk `base`, source phase p != 0.
+// Every lane loads one ALIGNED 16-byte source chunk per sub-step (64 chunks =
+// exactly eight 128-byte lines), takes its upper neighbour's chunk through a
+// DPP wave shift and funnels the two into the destination chunk, so 64 loaded
+// chunks yield 63 stored ones.  The source chunks touched all hold at least
+// one byte of the run, so nothing outside the run's own 16-byte-aligned hull
+// is read.
+template <int N, bool CSUM>
+__device__ __forceinline__ uint32_t funnel_step(const uint8_t *__restrict__ sa, uint8_t *__restrict__ d,
+                                                uint32_t base, uint32_t body, uint32_t p,
+                                                uint32_t lane)
+{
+  u32x4 v[N];
+  uint32_t acc = 0;
+#pragma unroll
+  for (int k = 0; k < N; k++) {
+    const uint32_t c = base + 63u * k + lane;
+    v[k] = (u32x4){0, 0, 0, 0};
+    if (c <= body) v[k] = *reinterpret_cast<const u32x4 *>(sa + ((size_t)c << 4));
+  }
+#pragma unroll
+  for (int k = 0; k < N; k++) {
+    const uint32_t c = base + 63u * k + lane;
+    u32x4 nx;
+#pragma unroll
+    for (int j = 0; j < 4; j++) nx[j] = wave_shl1(v[k][j]);
+    const u32x4 o = funnel(v[k], nx, p);
+    if (lane < 63 && c < body) {
+      store16_aligned(d + ((size_t)c << 4), o);
+      if (CSUM) acc += words_sum(o);
+    }
+  }
+  return acc;
+}
+
 // Copy `len` bytes src -> dst with one wavefront.  Stores are 16-byte aligned
-// (the destination decides the phase); loads take whatever phase that leaves
-// the source in.  The up-to-15 bytes before the first aligned store and after
-// the last one move as single bytes on lanes 0..15 and 16..31.
+// (the destination decides the phase).  A source that is then at least
+// 4-byte aligned is read with plain 16-byte loads; any other source phase is
+// read with aligned loads and realigned in registers (funnel_step), because a
+// 16-byte load from an address that is not a multiple of 4 costs about an
+// eighth of the achievable bandwidth.  The up-to-15 bytes before the first
+// aligned store and after the last one move as single bytes on lanes 0..15
+// and 16..31.
 // With CSUM the function also returns this lane's share of the sum of the
 // 16-bit little-endian words the run's bytes fall into, a byte's position in
 // its word being the parity of its DESTINATION ADDRESS (packet offsets and
@@ -100,28 +176,36 @@ __device__ __forceinline__ uint32_t copy_run(const uint8_t *__restrict__ src,
 
   const uint8_t *s = src + head;
   uint8_t *d = dst + head;
-  uint32_t c = lane;
-  // four chunks in flight per lane while they last
-  for (; c + 3 * kWave < body; c += 4 * kWave) {
-    u32x4 v0 = load16_any(s + ((size_t)c << 4));
-    u32x4 v1 = load16_any(s + ((size_t)(c + kWave) << 4));
-    u32x4 v2 = load16_any(s + ((size_t)(c + 2 * kWave) << 4));
-    u32x4 v3 = load16_any(s + ((size_t)(c + 3 * kWave) << 4));
-    store16_aligned(d + ((size_t)c << 4), v0);
-    store16_aligned(d + ((size_t)(c + kWave) << 4), v1);
-    store16_aligned(d + ((size_t)(c + 2 * kWave) << 4), v2);
-    store16_aligned(d + ((size_t)(c + 3 * kWave) << 4), v3);
-    if (CSUM) acc += words_sum(v0) + words_sum(v1) + words_sum(v2) + words_sum(v3);
-  }
-  // then two at a time, the second one predicated
-  for (; c < body; c += 2 * kWave) {
-    const bool two = c + kWave < body;
-    u32x4 v0 = load16_any(s + ((size_t)c << 4));
-    u32x4 v1 = {0, 0, 0, 0};
-    if (two) v1 = load16_any(s + ((size_t)(c + kWave) << 4));
-    store16_aligned(d + ((size_t)c << 4), v0);
-    if (two) store16_aligned(d + ((size_t)(c + kWave) << 4), v1);
-    if (CSUM) acc += words_sum(v0) + words_sum(v1);
+  const uint32_t p = (uint32_t)(uintptr_t)s & 15u;
+  if ((p & 3u) == 0) {
+    uint32_t c = lane;
+    // four chunks in flight per lane while they last
+    for (; c + 3 * kWave < body; c += 4 * kWave) {
+      u32x4 v0 = load16_any(s + ((size_t)c << 4));
+      u32x4 v1 = load16_any(s + ((size_t)(c + kWave) << 4));
+      u32x4 v2 = load16_any(s + ((size_t)(c + 2 * kWave) << 4));
+      u32x4 v3 = load16_any(s + ((size_t)(c + 3 * kWave) << 4));
+      store16_aligned(d + ((size_t)c << 4), v0);
+      store16_aligned(d + ((size_t)(c + kWave) << 4), v1);
+      store16_aligned(d + ((size_t)(c + 2 * kWave) << 4), v2);
+      store16_aligned(d + ((size_t)(c + 3 * kWave) << 4), v3);
+      if (CSUM) acc += words_sum(v0) + words_sum(v1) + words_sum(v2) + words_sum(v3);
+    }
+    // then two at a time, the second one predicated
+    for (; c < body; c += 2 * kWave) {
+      const bool two = c + kWave < body;
+      u32x4 v0 = load16_any(s + ((size_t)c << 4));
+      u32x4 v1 = {0, 0, 0, 0};
+      if (two) v1 = load16_any(s + ((size_t)(c + kWave) << 4));
+      store16_aligned(d + ((size_t)c << 4), v0);
+      if (two) store16_aligned(d + ((size_t)(c + kWave) << 4), v1);
+      if (CSUM) acc += words_sum(v0) + words_sum(v1);
+    }
+  } else {
+    const uint8_t *sa = s - p;
+    uint32_t base = 0;
+    for (; base + 126u < body; base += 252u) acc += funnel_step<4, CSUM>(sa, d, base, body, p, lane);
+    for (; base < body; base += 126u) acc += funnel_step<2, CSUM>(sa, d, base, body, p, lane);
   }
   if (edge) {
     dst[eoff] = (uint8_t)eb;

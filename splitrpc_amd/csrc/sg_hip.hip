@@ -1,13 +1,14 @@
 // sg_hip.hip -- kernels and C ABI of the gfx950 scatter-gather engine.
 //
 // Three kernels carry a batch:
-//   k_prep     one workgroup per request: block-wide exclusive scan of the
-//              fragment lengths (-> offset of every fragment inside its
-//              request, the running sum gather_skbs keeps,
-//              src/p2p_rpc_sg_engine.h:22-43), request totals, and -- in the
-//              workgroup that finishes last -- the scan of the request totals
-//              through the device-resident bump-ring cursor
-//              (src/p2p_rpc_tring.h:27-33).  Emits 16-byte run descriptors.
+//   k_prep_*   one workgroup (or, for short requests, one wavefront) per
+//              request: exclusive scan of the fragment lengths (-> offset of
+//              every fragment inside its request, the running sum gather_skbs
+//              keeps, src/p2p_rpc_sg_engine.h:22-43) and the request total.
+//              Emits 16-byte run descriptors.  k_req_scan then scans the
+//              request totals through the device-resident bump-ring cursor
+//              (src/p2p_rpc_tring.h:27-33); with one size for all requests the
+//              offsets are multiples and k_prep_* writes them itself.
 //   k_gather   one wavefront per fragment run: ring slot payload -> tensor.
 //   k_scatter  one wavefront per response frame: tensor -> TX slot payload,
 //              header rewrite, checksums.
@@ -56,25 +57,29 @@ struct PrepArgs {
   const uint32_t *item_len;
   const uint32_t *first;
   const uint64_t *sizes;
-  uint64_t fixed_size;
+  uint64_t fixed_size;     // mode 1: response size when sizes == NULL
+                           // mode 0: size every request must have (0: any)
   uint32_t n_items;
   uint32_t packed;
+  uint32_t fixed_offsets;  // packed: request r starts at cursor + r * fixed_size, no scan needed
   uint64_t cap;
   uint64_t max_req_bytes;  // tensor-major: sum of tensor sizes
   u32x4 *desc;             // {slot, len, offset in request, request}
   uint64_t *req_size;
   uint64_t *req_off;
-  uint64_t *cursor;
+  const uint64_t *cursor_in;
+  uint64_t *cursor_out;
   uint64_t *offsets_out;
-  uint32_t *ticket;
   uint32_t *status;
 };
 
-// Block-wide exclusive scan of one value per thread (kBlock threads).
-// Returns the exclusive prefix; *total gets the block sum.
+// Exclusive scan over the threads of a workgroup of BLOCK threads, built from
+// wavefront scans (DPP/permute shuffles) and one LDS slot per wavefront.
+template <int BLOCK>
 __device__ __forceinline__ uint64_t block_exclusive_scan(uint64_t v, uint64_t *lds_wave_tot,
                                                          uint64_t *total)
 {
+  constexpr uint32_t kWaves = BLOCK / kWave;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t wv = threadIdx.x / kWave;
   uint64_t inc = v;
@@ -83,11 +88,15 @@ __device__ __forceinline__ uint64_t block_exclusive_scan(uint64_t v, uint64_t *l
     uint64_t up = __shfl_up(inc, d, 64);
     if ((int)lane >= d) inc += up;
   }
+  if (kWaves == 1) {
+    *total = __shfl(inc, kWave - 1, 64);
+    return inc - v;
+  }
   if (lane == kWave - 1) lds_wave_tot[wv] = inc;
   __syncthreads();
   uint64_t base = 0, tot = 0;
 #pragma unroll
-  for (uint32_t i = 0; i < kWavesPerBlock; i++) {
+  for (uint32_t i = 0; i < kWaves; i++) {
     uint64_t t = lds_wave_tot[i];
     if (i < wv) base += t;
     tot += t;
@@ -97,100 +106,170 @@ __device__ __forceinline__ uint64_t block_exclusive_scan(uint64_t v, uint64_t *l
   return base + inc - v;
 }
 
-__global__ __launch_bounds__(kBlock) void k_prep(PrepArgs a)
+// Length and slot of item f of request r; raises status bits for what it refuses.
+__device__ __forceinline__ void prep_item(const PrepArgs &a, uint32_t f, uint32_t i, uint64_t size,
+                                          uint32_t *slot, uint32_t *len, uint32_t *bad)
 {
-  __shared__ uint64_t wave_tot[kWavesPerBlock];
-  __shared__ uint32_t is_last;
-  const uint32_t r = blockIdx.x;
-  uint32_t f0 = a.first[r];
-  uint32_t f1 = a.first[r + 1];
-  uint32_t bad = 0;
-  uint64_t carry = 0;
-  // the table must tile [0, n_items) without gaps, or descriptors of an
-  // earlier call would be taken for this one's
-  if (f0 > f1 || f1 > a.n_items || (r == 0 && f0 != 0) || (r == a.n_req - 1 && f1 != a.n_items)) {
-    bad |= kStBadTable;
-    f0 = f1 = 0;
-  }
-
-  if (a.mode == 0) {
-    for (uint32_t base = f0; base < f1; base += kBlock) {
-      const uint32_t f = base + threadIdx.x;
-      uint32_t len = 0, slot = 0;
-      if (f < f1) {
-        slot = a.item_slot[f];
-        if (slot >= a.n_slots) {
-          bad |= kStBadSlot;
-        } else {
-          len = a.item_len ? a.item_len[f] : load32_any(a.ring + (size_t)slot * a.slot_size + 54);
-          if (len > a.slot_size - a.hl) { bad |= kStBadLen; len = 0; }
-        }
-      }
-      uint64_t tot;
-      uint64_t ex = block_exclusive_scan(len, wave_tot, &tot);
-      if (f < f1) {
-        u32x4 d = {slot, len, (uint32_t)(carry + ex), r};
-        a.desc[f] = d;
-      }
-      carry += tot;
+  uint32_t s = a.item_slot[f];
+  uint32_t l = 0;
+  if (s >= a.n_slots) {
+    *bad |= kStBadSlot;
+    s = 0;
+  } else if (a.mode == 0) {
+    l = a.item_len ? a.item_len[f] : load32_any(a.ring + (size_t)s * a.slot_size + 54);
+    if (l > a.slot_size - a.hl) {
+      *bad |= kStBadLen;
+      l = 0;
     }
   } else {
-    const uint64_t size = a.sizes ? a.sizes[r] : a.fixed_size;
-    const uint64_t want = (size + a.mtu - 1) / a.mtu;
-    if (want != (uint64_t)(f1 - f0)) bad |= kStBadFrames;
-    for (uint32_t f = f0 + threadIdx.x; f < f1; f += kBlock) {
-      const uint64_t i = f - f0;
-      const uint64_t taken = i * a.mtu;
-      uint64_t rem = taken < size ? size - taken : 0;
-      uint32_t len = (uint32_t)(rem <= a.mtu ? rem : a.mtu);
-      uint32_t slot = a.item_slot[f];
-      uint32_t owner = r;
-      if (slot >= a.n_slots) { bad |= kStBadSlot; owner = kInvalidReq; }
-      if ((bad & kStBadFrames) || size > 0xffffffffull) owner = kInvalidReq;
-      u32x4 d = {slot, len, (uint32_t)taken, owner};
+    // frame i carries min(remaining, mtu) (src/transport/dpdk_rx_tx.h:137-139)
+    const uint64_t taken = (uint64_t)i * a.mtu;
+    const uint64_t rem = taken < size ? size - taken : 0;
+    l = (uint32_t)(rem <= a.mtu ? rem : a.mtu);
+  }
+  *slot = s;
+  *len = l;
+}
+
+// Checks on one request's slice of the CSR table and on its total; returns the
+// (possibly emptied) item range.
+__device__ __forceinline__ uint32_t prep_range(const PrepArgs &a, uint32_t r, uint32_t *f0,
+                                               uint32_t *f1, uint64_t *size)
+{
+  uint32_t bad = 0;
+  *f0 = a.first[r];
+  *f1 = a.first[r + 1];
+  // the table must tile [0, n_items) without gaps, or descriptors of an
+  // earlier call would be taken for this one's
+  if (*f0 > *f1 || *f1 > a.n_items || (r == 0 && *f0 != 0) ||
+      (r == a.n_req - 1 && *f1 != a.n_items)) {
+    bad |= kStBadTable;
+    *f0 = *f1 = 0;
+  }
+  *size = 0;
+  if (a.mode == 1) {
+    *size = a.sizes ? a.sizes[r] : a.fixed_size;
+    const uint64_t want = (*size + a.mtu - 1) / a.mtu;
+    if (want != (uint64_t)(*f1 - *f0) || *size > 0xffffffffull) {
+      bad |= kStBadFrames;
+      *f0 = *f1 = 0;
+      *size = 0;
+    }
+  }
+  return bad;
+}
+
+// What one request's owner (a thread) publishes once the request total is known.
+__device__ __forceinline__ void prep_finish(const PrepArgs &a, uint32_t r, uint64_t total, uint32_t bad)
+{
+  if (total > 0xffffffffull) bad |= kStBadSize;
+  if (!a.packed && total > a.max_req_bytes) bad |= kStBadSize;
+  if (a.packed && total > a.cap) bad |= kStBadSize;
+  if (a.mode == 0 && a.fixed_size && total != a.fixed_size) bad |= kStBadSize;
+  if (bad) atomicOr(a.status, bad);
+  a.req_size[r] = total;
+  if (a.packed && a.fixed_offsets) {
+    // bump ring with equal sizes: ret = base + off; off = (off + size) % capacity
+    const uint64_t c0 = *a.cursor_in % a.cap;
+    const uint64_t off = (c0 + (uint64_t)r * (a.fixed_size % a.cap)) % a.cap;
+    a.req_off[r] = off;
+    if (a.offsets_out) a.offsets_out[r] = off;
+    if (r == a.n_req - 1) {
+      const uint64_t end = (off + a.fixed_size) % a.cap;
+      *a.cursor_out = end;
+      if (a.offsets_out) a.offsets_out[a.n_req] = end;
+    }
+  }
+}
+
+// One workgroup of BLOCK threads per request: block-wide exclusive scan of the
+// fragment lengths, all header reads of a pass in flight together.
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void k_prep_block(PrepArgs a)
+{
+  __shared__ uint64_t wave_tot[BLOCK / kWave];
+  const uint32_t r = blockIdx.x;
+  uint32_t f0, f1;
+  uint64_t size;
+  uint32_t bad = prep_range(a, r, &f0, &f1, &size);
+  uint64_t carry = 0;
+  for (uint32_t base = f0; base < f1; base += BLOCK) {
+    const uint32_t f = base + threadIdx.x;
+    uint32_t len = 0, slot = 0;
+    if (f < f1) prep_item(a, f, f - f0, size, &slot, &len, &bad);
+    uint64_t tot;
+    const uint64_t ex = block_exclusive_scan<BLOCK>(len, wave_tot, &tot);
+    if (f < f1) {
+      u32x4 d = {slot, len, (uint32_t)(carry + ex), r};
       a.desc[f] = d;
     }
-    carry = (bad & kStBadFrames) ? 0 : size;
+    carry += tot;
   }
-  if (carry > 0xffffffffull) bad |= kStBadSize;
-  if (!a.packed && carry > a.max_req_bytes) bad |= kStBadSize;
-  if (a.packed && carry > a.cap) bad |= kStBadSize;
-  if (bad) atomicOr(a.status, bad);
+  // fold the status bits of all threads into thread 0
+  bad = wave_or(bad);
+  if ((threadIdx.x & (kWave - 1)) == 0 && bad) atomicOr(a.status, bad);
+  if (threadIdx.x == 0) prep_finish(a, r, carry, 0);
+}
 
-  // hand the request total to whichever workgroup finishes last
-  if (threadIdx.x == 0) {
-    __hip_atomic_store(&a.req_size[r], carry, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();
-    const uint32_t t = atomicAdd(a.ticket, 1u);
-    is_last = (t == a.n_req - 1);
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-
-  // scan of the request totals through the bump ring:
-  //   ret = base + off; off = (off + size) % capacity
-  uint64_t run = a.packed ? *a.cursor % a.cap : 0;
-  for (uint32_t base = 0; base < a.n_req; base += kBlock) {
-    const uint32_t q = base + threadIdx.x;
-    uint64_t sz = 0;
-    if (q < a.n_req) sz = __hip_atomic_load(&a.req_size[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// One wavefront per request (requests of at most a few dozen fragments).
+__global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
+{
+  const uint32_t r = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (r >= a.n_req) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t f0, f1;
+  uint64_t size;
+  uint32_t bad = prep_range(a, r, &f0, &f1, &size);
+  uint64_t carry = 0;
+  for (uint32_t base = f0; base < f1; base += kWave) {
+    const uint32_t f = base + lane;
+    uint32_t len = 0, slot = 0;
+    if (f < f1) prep_item(a, f, f - f0, size, &slot, &len, &bad);
     uint64_t tot;
-    uint64_t ex = block_exclusive_scan(sz, wave_tot, &tot);
-    if (q < a.n_req) {
-      uint64_t off = a.packed ? (run + ex) % a.cap : 0;
-      a.req_off[q] = off;
-      if (a.offsets_out) a.offsets_out[q] = off;
+    const uint64_t ex = block_exclusive_scan<kWave>(len, nullptr, &tot);
+    if (f < f1) {
+      u32x4 d = {slot, len, (uint32_t)(carry + ex), r};
+      a.desc[f] = d;
     }
-    run += tot;
-    if (a.packed) run %= a.cap;
+    carry += tot;
+  }
+  bad = wave_or(bad);
+  if (lane == 0) prep_finish(a, r, carry, bad);
+}
+
+// Scan of the request totals through the bump ring (one workgroup):
+//   ret = base + off; off = (off + size) % capacity   (src/p2p_rpc_tring.h:27-33)
+constexpr int kScanBlock = 1024;
+constexpr int kScanPerThread = 4;
+__global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
+{
+  __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  uint64_t run = *a.cursor_in % a.cap;
+  for (uint32_t base = 0; base < a.n_req; base += kScanBlock * kScanPerThread) {
+    const uint32_t q0 = base + threadIdx.x * kScanPerThread;
+    uint64_t sz[kScanPerThread];
+    uint64_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPerThread; k++) {
+      sz[k] = (q0 + k < a.n_req) ? a.req_size[q0 + k] : 0;
+      mine += sz[k];
+    }
+    uint64_t tot;
+    uint64_t ex = block_exclusive_scan<kScanBlock>(mine, wave_tot, &tot);
+#pragma unroll
+    for (int k = 0; k < kScanPerThread; k++) {
+      if (q0 + k < a.n_req) {
+        const uint64_t off = (run + ex) % a.cap;
+        a.req_off[q0 + k] = off;
+        if (a.offsets_out) a.offsets_out[q0 + k] = off;
+      }
+      ex += sz[k];
+    }
+    run = (run + tot) % a.cap;
   }
   if (threadIdx.x == 0) {
-    if (a.packed) {
-      *a.cursor = run;
-      if (a.offsets_out) a.offsets_out[a.n_req] = run;
-    }
-    *a.ticket = 0;
+    *a.cursor_out = run;
+    if (a.offsets_out) a.offsets_out[a.n_req] = run;
   }
 }
 
@@ -199,14 +278,19 @@ __global__ __launch_bounds__(kBlock) void k_prep(PrepArgs a)
 // ---------------------------------------------------------------------------
 
 // Which item a wavefront works on.  Workgroups are dealt round-robin to the
-// eight XCDs, each with its own L2; giving XCD x the x-th contiguous eighth of
-// the items keeps neighbouring runs -- which share the cache lines at their
-// common destination boundary -- in one L2.
-__device__ __forceinline__ uint32_t item_of_wave(uint32_t n_groups_per_xcd, bool remap)
+// eight XCDs, each with its own L2.  Runs of kXcdRun consecutive workgroups'
+// worth of items are given to one XCD, so that neighbouring fragment runs --
+// which share the cache lines at their common destination boundary -- meet in
+// one L2, while all XCDs still walk the same region of memory together.
+constexpr uint32_t kXcdRun = 32;
+__device__ __forceinline__ uint32_t item_of_wave(bool remap)
 {
   uint32_t g = blockIdx.x;
-  if (remap) g = (blockIdx.x % kXcds) * n_groups_per_xcd + blockIdx.x / kXcds;
-  return g * kWavesPerBlock + threadIdx.x / kWave;
+  if (remap) {
+    const uint32_t xcd = g % kXcds, k = g / kXcds;
+    g = ((k / kXcdRun) * kXcds + xcd) * kXcdRun + (k % kXcdRun);
+  }
+  return __builtin_amdgcn_readfirstlane(g * kWavesPerBlock + threadIdx.x / kWave);
 }
 
 struct GatherArgs {
@@ -216,7 +300,6 @@ struct GatherArgs {
   uint32_t slot_size;
   uint32_t hl;
   uint32_t n_items;
-  uint32_t groups_per_xcd;
   uint32_t remap;
   const uint32_t *status;
   AppDev app;
@@ -267,7 +350,7 @@ __device__ __forceinline__ uint32_t move_run(const AppDev &app, uint64_t req_off
 
 __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
 {
-  const uint32_t item = item_of_wave(a.groups_per_xcd, a.remap != 0);
+  const uint32_t item = item_of_wave(a.remap != 0);
   if (item >= a.n_items) return;
   if (*a.status) return;  // k_prep refused the batch: move nothing
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -292,7 +375,6 @@ struct ScatterArgs {
   uint32_t ref64;
   uint32_t flags;
   uint32_t n_items;
-  uint32_t groups_per_xcd;
   uint32_t remap;
   uint32_t *status;
   AppDev app;
@@ -301,7 +383,7 @@ struct ScatterArgs {
 template <bool FULL_CSUM>
 __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
-  const uint32_t item = item_of_wave(a.groups_per_xcd, a.remap != 0);
+  const uint32_t item = item_of_wave(a.remap != 0);
   if (item >= a.n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   if (*a.status) return;  // k_prep refused the batch: move nothing
@@ -391,8 +473,10 @@ struct sg_hip_ctx {
   u32x4 *desc = nullptr;
   uint64_t *req_size = nullptr;
   uint64_t *req_off = nullptr;
-  uint64_t *cursors = nullptr;  // [0] request arena, [1] response arena
-  uint32_t *ticket = nullptr;
+  // bump-ring cursors: request arena at [0 + parity], response arena at
+  // [2 + parity]; a launch reads one parity and writes the other
+  uint64_t *cursors = nullptr;
+  uint32_t parity[2] = {0, 0};
   uint32_t *status = nullptr;
   // pinned staging for the per-request entry points (device reads it in place)
   Run *h_runs = nullptr;
@@ -479,16 +563,18 @@ int check_app(sg_hip_ctx *c, const sg_app_desc &a, AppDev *out, uint64_t *max_re
   return SG_OK;
 }
 
-// Launch geometry for one wavefront per item with the XCD-aware order.
-void geometry(uint32_t n_items, bool remap, uint32_t *grid, uint32_t *groups_per_xcd)
+// Launch geometry for one wavefront per item; with the XCD-aware order the
+// grid is padded to whole rounds of kXcds * kXcdRun workgroups.
+void geometry(uint32_t n_items, bool want_remap, uint32_t *grid, uint32_t *remap)
 {
   const uint32_t groups = (n_items + kWavesPerBlock - 1) / kWavesPerBlock;
-  if (remap && groups >= 2 * kXcds) {
-    *groups_per_xcd = (groups + kXcds - 1) / kXcds;
-    *grid = *groups_per_xcd * kXcds;
+  const uint32_t round = kXcds * kXcdRun;
+  if (want_remap && groups >= 2 * round) {
+    *grid = (groups + round - 1) / round * round;
+    *remap = 1;
   } else {
-    *groups_per_xcd = 0;
     *grid = groups;
+    *remap = 0;
   }
 }
 
@@ -527,6 +613,24 @@ int prof_drain(sg_hip_ctx *c)
   }
   c->ev_used.clear();
   return SG_OK;
+}
+
+// Descriptor build: kernel shape by the average request, then the bump-ring
+// scan of the request totals where offsets are not plain multiples.
+int launch_prep(sg_hip_ctx *c, const PrepArgs &p)
+{
+  int rc = prof_begin(c, 0);
+  if (rc != SG_OK) return rc;
+  const uint32_t avg = p.n_items / p.n_req;
+  if (avg <= 32) {
+    k_prep_wave<<<(p.n_req + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(p);
+  } else if (avg <= 256) {
+    k_prep_block<256><<<p.n_req, 256, 0, c->stream>>>(p);
+  } else {
+    k_prep_block<1024><<<p.n_req, 1024, 0, c->stream>>>(p);
+  }
+  if (p.packed && !p.fixed_offsets) k_req_scan<<<1, kScanBlock, 0, c->stream>>>(p);
+  return prof_end(c);
 }
 
 int finish(sg_hip_ctx *c, uint32_t flags)
@@ -574,11 +678,9 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMalloc(&c->desc, sizeof(u32x4) * (size_t)c->max_frames));
   HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
-  HIP_TRY(nullptr, hipMalloc(&c->cursors, 2 * sizeof(uint64_t)));
-  HIP_TRY(nullptr, hipMalloc(&c->ticket, sizeof(uint32_t)));
+  HIP_TRY(nullptr, hipMalloc(&c->cursors, 4 * sizeof(uint64_t)));
   HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
-  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 2 * sizeof(uint64_t), c->stream));
-  HIP_TRY(nullptr, hipMemsetAsync(c->ticket, 0, sizeof(uint32_t), c->stream));
+  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 4 * sizeof(uint64_t), c->stream));
   HIP_TRY(nullptr, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
   c->h_runs_cap = 8192;
   HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
@@ -618,7 +720,6 @@ void sg_hip_destroy(sg_hip_ctx *c)
   (void)hipFree(c->req_size);
   (void)hipFree(c->req_off);
   (void)hipFree(c->cursors);
-  (void)hipFree(c->ticket);
   (void)hipFree(c->status);
   if (c->h_runs) (void)hipHostFree(c->h_runs);
   if (c->h_ptrs) (void)hipHostFree(c->h_ptrs);
@@ -654,7 +755,7 @@ int sg_hip_set_cursor(sg_hip_ctx *c, int which, uint64_t value)
   if (!c || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
-  HIP_TRY(c, hipMemcpy(c->cursors + which, &value, sizeof value, hipMemcpyHostToDevice));
+  HIP_TRY(c, hipMemcpy(c->cursors + 2 * which + c->parity[which], &value, sizeof value, hipMemcpyHostToDevice));
   return SG_OK;
 }
 
@@ -663,7 +764,7 @@ int sg_hip_get_cursor(sg_hip_ctx *c, int which, uint64_t *value)
   if (!c || !value || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
-  HIP_TRY(c, hipMemcpy(value, c->cursors + which, sizeof *value, hipMemcpyDeviceToHost));
+  HIP_TRY(c, hipMemcpy(value, c->cursors + 2 * which + c->parity[which], sizeof *value, hipMemcpyDeviceToHost));
   return SG_OK;
 }
 
@@ -798,14 +899,14 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   p.desc = c->desc;
   p.req_size = c->req_size;
   p.req_off = c->req_off;
-  p.cursor = c->cursors + 0;
+  p.fixed_size = a->fixed_req_size;
+  p.fixed_offsets = p.packed && a->fixed_req_size != 0;
+  p.cursor_in = c->cursors + 0 + c->parity[0];
+  p.cursor_out = c->cursors + 0 + (c->parity[0] ^ 1u);
+  if (p.packed) c->parity[0] ^= 1u;
   p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
-  p.ticket = c->ticket;
   p.status = c->status;
-  rc = prof_begin(c, 0);
-  if (rc != SG_OK) return rc;
-  k_prep<<<a->n_req, kBlock, 0, c->stream>>>(p);
-  rc = prof_end(c);
+  rc = launch_prep(c, p);
   if (rc != SG_OK) return rc;
 
   if (a->n_frags) {
@@ -820,8 +921,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.status = c->status;
     ga.app = app;
     uint32_t grid;
-    geometry(a->n_frags, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.groups_per_xcd);
-    ga.remap = ga.groups_per_xcd != 0;
+    geometry(a->n_frags, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
     k_gather<<<grid, kBlock, 0, c->stream>>>(ga);
@@ -872,14 +972,13 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   p.desc = c->desc;
   p.req_size = c->req_size;
   p.req_off = c->req_off;
-  p.cursor = c->cursors + 1;
+  p.fixed_offsets = p.packed && a->resp_size == nullptr;
+  p.cursor_in = c->cursors + 2 + c->parity[1];
+  p.cursor_out = c->cursors + 2 + (c->parity[1] ^ 1u);
+  if (p.packed) c->parity[1] ^= 1u;
   p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
-  p.ticket = c->ticket;
   p.status = c->status;
-  rc = prof_begin(c, 0);
-  if (rc != SG_OK) return rc;
-  k_prep<<<a->n_req, kBlock, 0, c->stream>>>(p);
-  rc = prof_end(c);
+  rc = launch_prep(c, p);
   if (rc != SG_OK) return rc;
 
   if (a->n_frames) {
@@ -901,8 +1000,7 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.status = c->status;
     sa.app = app;
     uint32_t grid;
-    geometry(a->n_frames, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.groups_per_xcd);
-    sa.remap = sa.groups_per_xcd != 0;
+    geometry(a->n_frames, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
     if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true><<<grid, kBlock, 0, c->stream>>>(sa);

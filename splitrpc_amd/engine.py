@@ -122,9 +122,11 @@ class SgContext:
         return float(ms.value), int(n.value)
 
     # -- batched -----------------------------------------------------------
-    def gather_batch(self, ring: RingRef, frag_slot: torch.Tensor, frag_len: Optional[torch.Tensor],
-                     req_first: torch.Tensor, n_req: int, n_frags: int, app: AppRef,
-                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0) -> None:
+    @staticmethod
+    def gather_args(ring: RingRef, frag_slot: torch.Tensor, frag_len: Optional[torch.Tensor],
+                    req_first: torch.Tensor, n_req: int, n_frags: int, app: AppRef,
+                    offsets_out: Optional[torch.Tensor] = None, flags: int = 0,
+                    fixed_req_size: int = 0) -> capi.GatherArgs:
         a = capi.GatherArgs()
         a.ring = ring.desc()
         a.frag_slot = frag_slot.data_ptr()
@@ -135,13 +137,23 @@ class SgContext:
         a.app = app.desc()
         a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
         a.flags = flags
-        self._check(self.lib.sg_hip_gather_batch(self.h, C.byref(a)))
+        a.fixed_req_size = int(fixed_req_size)
+        return a
 
-    def scatter_batch(self, rx: RingRef, tx: RingRef, tx_slot: torch.Tensor,
-                      hdr_src_slot: torch.Tensor, resp_first: torch.Tensor,
-                      resp_size: Optional[torch.Tensor], fixed_resp_size: int, n_req: int,
-                      n_frames: int, mtu: int, app: AppRef,
-                      offsets_out: Optional[torch.Tensor] = None, flags: int = 0) -> None:
+    def gather_batch(self, *args, **kw) -> None:
+        self.gather_batch_raw(self.gather_args(*args, **kw))
+
+    def gather_batch_raw(self, a: capi.GatherArgs) -> None:
+        rc = self.lib.sg_hip_gather_batch(self.h, C.byref(a))
+        if rc != capi.SG_OK:
+            self._check(rc)
+
+    @staticmethod
+    def scatter_args(rx: RingRef, tx: RingRef, tx_slot: torch.Tensor,
+                     hdr_src_slot: torch.Tensor, resp_first: torch.Tensor,
+                     resp_size: Optional[torch.Tensor], fixed_resp_size: int, n_req: int,
+                     n_frames: int, mtu: int, app: AppRef,
+                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0) -> capi.ScatterArgs:
         a = capi.ScatterArgs()
         a.rx = rx.desc()
         a.tx = tx.desc()
@@ -156,7 +168,15 @@ class SgContext:
         a.flags = flags
         a.app = app.desc()
         a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
-        self._check(self.lib.sg_hip_scatter_batch(self.h, C.byref(a)))
+        return a
+
+    def scatter_batch(self, *args, **kw) -> None:
+        self.scatter_batch_raw(self.scatter_args(*args, **kw))
+
+    def scatter_batch_raw(self, a: capi.ScatterArgs) -> None:
+        rc = self.lib.sg_hip_scatter_batch(self.h, C.byref(a))
+        if rc != capi.SG_OK:
+            self._check(rc)
 
     # -- per request ---------------------------------------------------------
     def copy_runs(self, src: Sequence[int], dst: Sequence[int], lens: Sequence[int],
@@ -191,6 +211,7 @@ class DeviceWorkload:
         batches and the working set outgrows the caches."""
         self.w = w
         self.copies = copies
+        self._args = {}
         dev = torch.device(device)
         self.dev = dev
         k = copies
@@ -264,12 +285,32 @@ class DeviceWorkload:
             o += s
         return outs
 
-    def gather(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False) -> None:
-        ctx.gather_batch(self.rx, self.frag_slot, self.frag_len if use_frag_len else None,
-                         self.req_first, self.n_req, self.n_frags, self.req_app,
-                         self.req_offsets, flags)
+    def gather(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False,
+               fixed: bool = True) -> None:
+        """``fixed``: declare the common request size when all requests have one
+        (offsets are then multiples of it instead of a prefix scan)."""
+        key = ("g", use_frag_len, fixed)
+        a = self._args.get(key)
+        if a is None:
+            need_len = use_frag_len or self.w.profile != 0
+            sizes = self.w.req_sizes
+            fx = int(sizes[0]) if fixed and len(sizes) and bool((sizes == sizes[0]).all()) else 0
+            a = ctx.gather_args(self.rx, self.frag_slot, self.frag_len if need_len else None,
+                                self.req_first, self.n_req, self.n_frags, self.req_app,
+                                self.req_offsets, 0, fixed_req_size=fx)
+            self._args[key] = a
+        a.flags = flags
+        ctx.gather_batch_raw(a)
 
-    def scatter(self, ctx: SgContext, flags: int = 0) -> None:
-        ctx.scatter_batch(self.rx, self.tx, self.tx_slot, self.hdr_src_slot, self.resp_first,
-                          self.resp_size, 0, self.n_req, self.n_frames, self.w.mtu, self.resp_app,
-                          self.resp_offsets, self.w.flags | flags)
+    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True) -> None:
+        key = ("s", fixed)
+        a = self._args.get(key)
+        if a is None:
+            sizes = self.w.resp_sizes
+            fx = int(sizes[0]) if fixed and len(sizes) and bool((sizes == sizes[0]).all()) else 0
+            a = ctx.scatter_args(self.rx, self.tx, self.tx_slot, self.hdr_src_slot, self.resp_first,
+                                 None if fx else self.resp_size, fx, self.n_req, self.n_frames,
+                                 self.w.mtu, self.resp_app, self.resp_offsets, 0)
+            self._args[key] = a
+        a.flags = self.w.flags | flags
+        ctx.scatter_batch_raw(a)

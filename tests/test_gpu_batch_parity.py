@@ -14,15 +14,17 @@ pytestmark = pytest.mark.gpu
 CASES = [(1, None), (2, None), (3, None), (4, None), (5, None), (2, 1), (4, 7), (5, 2)]
 
 
+@pytest.mark.parametrize("fixed", [True, False], ids=["fixed", "scan"])
 @pytest.mark.parametrize("cfg,n_req", CASES)
-def test_gather_scatter_bit_exact(ctx, cfg, n_req):
+def test_gather_scatter_bit_exact(ctx, cfg, n_req, fixed):
     w = synth.make_workload(cfg, n_req)
-    print(f"case cfg={cfg} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames}", flush=True)
+    print(f"case cfg={cfg} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} fixed={fixed}",
+          flush=True)
     dw = DeviceWorkload(w)
     ctx.set_cursor(0, 0)
     ctx.set_cursor(1, 0)
 
-    dw.gather(ctx)
+    dw.gather(ctx, fixed=fixed)
     if w.in_tensor_sizes:
         exp, _, _ = expected_gather(w)
         for t, e in zip(dw.in_tensors, exp):
@@ -37,7 +39,7 @@ def test_gather_scatter_bit_exact(ctx, cfg, n_req):
         assert ctx.get_cursor(0) == cur
         gathered = exp
 
-    dw.scatter(ctx)
+    dw.scatter(ctx, fixed=fixed)
     exp_tx, offs, cur = expected_scatter(w, gathered, resp_cap=dw.resp_app.cap if not w.out_tensor_sizes else None)
     got_tx = dw.tx_ring.cpu().numpy()
     assert np.array_equal(got_tx, exp_tx), first_diff(got_tx, exp_tx)
