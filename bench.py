@@ -46,6 +46,8 @@ def parse():
     ap.add_argument("--no-sweep", action="store_true", help="skip requests/s of the other workloads")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-remap", action="store_true", help="disable the XCD-aware launch order")
+    ap.add_argument("--general", action="store_true",
+                    help="always run the descriptor pass (do not declare the fragmenting rule)")
     return ap.parse_args()
 
 
@@ -55,7 +57,7 @@ DEFAULT_BPL = {1: 256, 2: 32, 3: 64, 4: 8, 5: 4}
 class Pool:
     """R device copies of one workload, rotated between steps."""
 
-    def __init__(self, w, bpl: int, rotate_mb: int, extra_flags: int = 0):
+    def __init__(self, w, bpl: int, rotate_mb: int, extra_flags: int = 0, rule: bool = True):
         from splitrpc_amd.engine import DeviceWorkload
         per = (w.ring.nbytes + int(w.req_sizes.sum()) + w.tx_n_slots * w.slot_size
                + int(w.resp_sizes.sum())) * bpl
@@ -64,14 +66,15 @@ class Pool:
         self.w = w
         self.bpl = bpl
         self.extra_flags = extra_flags
+        self.rule = rule  # declare size + fragmenting rule where the workload has one size
         self.gather_bytes = w.gather_bytes() * bpl
         self.scatter_bytes = w.scatter_bytes() * bpl
         self.n_req = w.n_req * bpl
 
     def step(self, ctx, i: int, flags: int) -> None:
         dw = self.items[i % len(self.items)]
-        dw.gather(ctx, flags | self.extra_flags)
-        dw.scatter(ctx, flags | self.extra_flags)
+        dw.gather(ctx, flags | self.extra_flags, rule=self.rule)
+        dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule)
 
 
 def timed(ctx, pool: Pool, steps: int, warmup: int):
@@ -162,7 +165,7 @@ def main() -> int:
     bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
     w = synth.make_workload(a.workload)
     ctx = SgContext(0, max_reqs=max(4096, w.n_req * bpl), max_frames=max(65536, max(w.n_frags, w.n_resp_frames) * bpl))
-    pool = Pool(w, bpl, a.rotate_mb, extra)
+    pool = Pool(w, bpl, a.rotate_mb, extra, rule=not a.general)
 
     sec = timed(ctx, pool, a.steps, a.warmup)
     kt = kernel_times(ctx, pool, min(a.steps, 100))
@@ -176,7 +179,7 @@ def main() -> int:
     # the single-batch call of the same workload, for the record
     single = None
     if bpl != 1:
-        p1 = Pool(w, 1, a.rotate_mb, extra)
+        p1 = Pool(w, 1, a.rotate_mb, extra, rule=not a.general)
         s1 = timed(ctx, p1, a.steps, a.warmup)
         k1 = kernel_times(ctx, p1, min(a.steps, 100))
         b1 = p1.gather_bytes + p1.scatter_bytes
@@ -197,7 +200,7 @@ def main() -> int:
             b = DEFAULT_BPL[cfg]
             c2 = SgContext(0, max_reqs=max(4096, wc.n_req * b),
                            max_frames=max(65536, max(wc.n_frags, wc.n_resp_frames) * b))
-            pc = Pool(wc, b, a.rotate_mb, extra)
+            pc = Pool(wc, b, a.rotate_mb, extra, rule=not a.general)
             sc = timed(c2, pc, max(20, a.steps // 4), max(5, a.warmup // 4))
             rps[wc.name] = round(pc.n_req / sc, 1)
             sweep[wc.name] = {"batches_per_launch": b, "ms_per_step": round(sc * 1e3, 5),
@@ -224,6 +227,8 @@ def main() -> int:
                                f"{w.n_resp_frames // w.n_req} response frames per request",
                    "batches_per_launch": bpl, "rotated_ring_copies": len(pool.items),
                    "requests_per_step": pool.n_req, "header_profile": "BL58",
+                   "descriptor_pass": "general (prefix scan)" if a.general else
+                   "fused where the workload has one size (fragmenting rule declared and checked)",
                    "flags": w.flags},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "requests_per_sec": rps,

@@ -51,6 +51,16 @@ extern "C" {
 #define SG_F_UDP_CSUM_FULL (1u << 2)   /* finished UDP checksum over header + payload (RFC 768) */
 #define SG_F_REF_QUIRKS (1u << 3)      /* pseudo sum takes UDP length as tot_len - version*4,
                                           src/eth_common.h:111-112 */
+#define SG_F_RULE_FRAGS (1u << 4)       /* gather: the caller states that every request has
+                                          fixed_req_size bytes cut by the fragmenting rule at mtu
+                                          (all fragments mtu bytes, the last the remainder,
+                                          src/transport/dpdk_rx_tx.h:137-139).  Offsets are then
+                                          multiples and no descriptor pass runs; every fragment's
+                                          real length is held against the rule and a batch that
+                                          departs from it is refused with SG_E_DATA (its
+                                          destination bytes are then undefined). */
+#define SG_F_NO_FUSE (1u << 5)          /* scatter: run the descriptor pass even where the copy
+                                          kernel could derive the descriptors (for experiments) */
 #define SG_F_ASYNC (1u << 16)          /* enqueue only; completion through sg_hip_sync() */
 #define SG_F_NO_XCD_REMAP (1u << 17)   /* launch-order = item order (for experiments) */
 
@@ -128,7 +138,7 @@ typedef struct sg_gather_args {
   sg_app_desc app;
   uint64_t *offsets_out; /* device, n_req + 1 arena offsets (packed mode), or NULL */
   uint32_t flags;
-  uint32_t reserved;
+  uint32_t mtu;            /* payload bytes per full fragment; used with SG_F_RULE_FRAGS */
   uint64_t fixed_req_size; /* non-zero: every request must total exactly this many bytes (the
                               reference's server-wide request size, is_rr_ready,
                               src/p2p_rpc_rr_ng.h:107-110); a batch holding another size is

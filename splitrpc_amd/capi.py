@@ -25,6 +25,8 @@ F_IPV4_CSUM = 1 << 0
 F_UDP_CSUM_PSEUDO = 1 << 1
 F_UDP_CSUM_FULL = 1 << 2
 F_REF_QUIRKS = 1 << 3
+F_RULE_FRAGS = 1 << 4
+F_NO_FUSE = 1 << 5
 F_ASYNC = 1 << 16
 F_NO_XCD_REMAP = 1 << 17
 
@@ -71,7 +73,7 @@ class GatherArgs(C.Structure):
     _fields_ = [("ring", RingDesc), ("frag_slot", C.c_void_p), ("frag_len", C.c_void_p),
                 ("req_first", C.c_void_p), ("n_req", C.c_uint32), ("n_frags", C.c_uint32),
                 ("app", AppDesc), ("offsets_out", C.c_void_p), ("flags", C.c_uint32),
-                ("reserved", C.c_uint32), ("fixed_req_size", C.c_uint64)]
+                ("mtu", C.c_uint32), ("fixed_req_size", C.c_uint64)]
 
 
 class ScatterArgs(C.Structure):

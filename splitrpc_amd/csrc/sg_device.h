@@ -2,8 +2,7 @@
 // engine: wavefront copy of one run, wavefront reductions, response-header
 // rewrite with one header byte per lane.
 //
-// gfx950 only: 64-wide wavefronts, unaligned global access enabled (a 16-byte
-// load from any byte address is one global_load_dwordx4).
+// gfx950 only: 64-wide wavefronts, DPP wave shifts.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -22,6 +21,7 @@ constexpr uint32_t kStBadLen = 1u << 1;      // fragment longer than a slot can 
 constexpr uint32_t kStBadSize = 1u << 2;     // request larger than its destination
 constexpr uint32_t kStBadFrames = 1u << 3;   // response frame count disagrees with the fragmenting rule
 constexpr uint32_t kStBadTable = 1u << 4;    // CSR table is not a gap-free tiling of the items
+constexpr uint32_t kStNotRule = 1u << 5;     // a fragment's length departs from the fragmenting rule
 constexpr uint32_t kInvalidReq = 0xffffffffu; // owner field of a descriptor the kernels must skip
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -41,6 +41,17 @@ __device__ __forceinline__ uint32_t load32_any(const uint8_t *p)
 __device__ __forceinline__ void store16_aligned(uint8_t *p, u32x4 v)
 {
   *reinterpret_cast<u32x4 *>(p) = v;
+}
+
+// Load through the scalar data cache: for wave-uniform addresses of data that
+// NO wavefront of the running kernel writes (tables and cursors produced by an
+// earlier kernel, ring headers in a kernel that only reads the ring).  The
+// scalar cache is read-only here and is invalidated at kernel boundaries.
+template <class T>
+__device__ __forceinline__ T sload(const T *p)
+{
+  typedef const __attribute__((address_space(4))) T *cptr;
+  return *(cptr)(uintptr_t)p;
 }
 
 // Sum of the eight 16-bit little-endian words of a 16-byte chunk.
@@ -80,9 +91,9 @@ __device__ __forceinline__ uint32_t wave_shl1(uint32_t v)
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x130, 0xf, 0xf, false);
 }
 
-// Bytes [p, p+16) of the 32-byte window {lo, hi}; 0 < p < 16.
+// Bytes [p, p+16) of the 32-byte window {lo, hi}, p = 4*Q + bs.
 template <int Q>
-__device__ __forceinline__ u32x4 funnel_q(u32x4 lo, u32x4 hi, uint32_t bs)
+__device__ __forceinline__ u32x4 window_q(u32x4 lo, u32x4 hi, uint32_t bs)
 {
   const uint32_t D[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   u32x4 o;
@@ -92,126 +103,136 @@ __device__ __forceinline__ u32x4 funnel_q(u32x4 lo, u32x4 hi, uint32_t bs)
   return o;
 }
 
-__device__ __forceinline__ u32x4 funnel(u32x4 lo, u32x4 hi, uint32_t p)
+// The destination chunk a lane stores, from the aligned source chunk it loaded
+// (`v`) and the one its upper neighbour loaded; p is the source phase 0..15.
+__device__ __forceinline__ u32x4 realign(u32x4 v, uint32_t p)
 {
+  u32x4 nx;
+#pragma unroll
+  for (int j = 0; j < 4; j++) nx[j] = wave_shl1(v[j]);
   const uint32_t bs = p & 3u;
   switch (p >> 2) {
-    case 0: return funnel_q<0>(lo, hi, bs);
-    case 1: return funnel_q<1>(lo, hi, bs);
-    case 2: return funnel_q<2>(lo, hi, bs);
-    default: return funnel_q<3>(lo, hi, bs);
+    case 0: return window_q<0>(v, nx, bs);
+    case 1: return window_q<1>(v, nx, bs);
+    case 2: return window_q<2>(v, nx, bs);
+    default: return window_q<3>(v, nx, bs);
   }
 }
 
-// N x 63 destination chunks starting at chunk `base`, source phase p != 0.
-// Every lane loads one ALIGNED 16-byte source chunk per sub-step (64 chunks =
-// exactly eight 128-byte lines), takes its upper neighbour's chunk through a
-// DPP wave shift and funnels the two into the destination chunk, so 64 loaded
-// chunks yield 63 stored ones.  The source chunks touched all hold at least
-// one byte of the run, so nothing outside the run's own 16-byte-aligned hull
-// is read.
-template <int N, bool CSUM>
-__device__ __forceinline__ uint32_t funnel_step(const uint8_t *__restrict__ sa, uint8_t *__restrict__ d,
-                                                uint32_t base, uint32_t body, uint32_t p,
-                                                uint32_t lane)
-{
-  u32x4 v[N];
-  uint32_t acc = 0;
-#pragma unroll
-  for (int k = 0; k < N; k++) {
-    const uint32_t c = base + 63u * k + lane;
-    v[k] = (u32x4){0, 0, 0, 0};
-    if (c <= body) v[k] = *reinterpret_cast<const u32x4 *>(sa + ((size_t)c << 4));
-  }
-#pragma unroll
-  for (int k = 0; k < N; k++) {
-    const uint32_t c = base + 63u * k + lane;
-    u32x4 nx;
-#pragma unroll
-    for (int j = 0; j < 4; j++) nx[j] = wave_shl1(v[k][j]);
-    const u32x4 o = funnel(v[k], nx, p);
-    if (lane < 63 && c < body) {
-      store16_aligned(d + ((size_t)c << 4), o);
-      if (CSUM) acc += words_sum(o);
-    }
-  }
-  return acc;
-}
+// One run (a contiguous piece of payload) in the hands of one wavefront.
+//
+// Stores are 16-byte aligned: the destination decides the phase.  Loads are
+// 16-byte ALIGNED too, whatever phase that leaves the source in: every lane
+// loads one aligned source chunk per step (64 chunks = exactly eight 128-byte
+// lines), takes its upper neighbour's chunk through a DPP wave shift and
+// byte-aligns the 32-byte window into one destination chunk, so 64 loaded
+// chunks yield 63 stored ones.  (A 16-byte load from an address that is not a
+// multiple of 4 costs about an eighth of the achievable bandwidth.)  All loaded
+// chunks hold at least one byte of the run, so nothing outside the run's own
+// 16-byte-aligned hull is read.  The up-to-15 bytes before the first aligned
+// store and after the last one move as single bytes on lanes 0..15 / 16..31.
+//
+// run_begin issues the edge-byte load and the loads of the first two steps
+// (126 destination chunks, 2016 bytes); run_end realigns, stores and walks the
+// rest.  A wavefront that begins several runs before ending the first keeps
+// that many runs' loads in flight.
+struct RunState {
+  const uint8_t *src;
+  uint8_t *dst;
+  const uint8_t *sa;  // source of the first aligned store, rounded down to 16
+  uint8_t *d;         // first aligned store
+  uint32_t body;      // number of aligned 16-byte stores
+  uint32_t lim;       // last source chunk to load (body when the phase is non-zero)
+  uint32_t p;         // source phase
+  uint32_t eoff;      // this lane's edge byte, if any
+  uint32_t eb;
+  bool edge;
+  u32x4 v0, v1;
+};
 
-// Copy `len` bytes src -> dst with one wavefront.  Stores are 16-byte aligned
-// (the destination decides the phase).  A source that is then at least
-// 4-byte aligned is read with plain 16-byte loads; any other source phase is
-// read with aligned loads and realigned in registers (funnel_step), because a
-// 16-byte load from an address that is not a multiple of 4 costs about an
-// eighth of the achievable bandwidth.  The up-to-15 bytes before the first
-// aligned store and after the last one move as single bytes on lanes 0..15
-// and 16..31.
-// With CSUM the function also returns this lane's share of the sum of the
-// 16-bit little-endian words the run's bytes fall into, a byte's position in
-// its word being the parity of its DESTINATION ADDRESS (packet offsets and
-// addresses have the same parity: ring bases, slot sizes and header lengths
-// are even).
-template <bool CSUM>
-__device__ __forceinline__ uint32_t copy_run(const uint8_t *__restrict__ src,
-                                             uint8_t *__restrict__ dst, uint32_t len, uint32_t lane)
+__device__ __forceinline__ void run_begin(RunState &r, const uint8_t *__restrict__ src,
+                                          uint8_t *__restrict__ dst, uint32_t len, uint32_t lane)
 {
-  uint32_t acc = 0;
   uint32_t head = (uint32_t)(-(uintptr_t)dst) & 15u;
   head = head < len ? head : len;
   const uint32_t body = (len - head) >> 4;
   const uint32_t tail = (len - head) & 15u;
-
-  // edge bytes
-  bool edge = false;
-  uint32_t eoff = 0;
+  r.src = src;
+  r.dst = dst;
+  r.body = body;
+  r.edge = false;
+  r.eoff = 0;
   if (lane < 16) {
-    edge = lane < head;
-    eoff = lane;
+    r.edge = lane < head;
+    r.eoff = lane;
   } else if (lane < 32) {
-    edge = (lane - 16) < tail;
-    eoff = head + (body << 4) + (lane - 16);
+    r.edge = (lane - 16) < tail;
+    r.eoff = head + (body << 4) + (lane - 16);
   }
-  uint32_t eb = 0;
-  if (edge) eb = src[eoff];
-
+  r.eb = 0;
+  if (r.edge) r.eb = src[r.eoff];
   const uint8_t *s = src + head;
-  uint8_t *d = dst + head;
-  const uint32_t p = (uint32_t)(uintptr_t)s & 15u;
-  if ((p & 3u) == 0) {
-    uint32_t c = lane;
-    // four chunks in flight per lane while they last
-    for (; c + 3 * kWave < body; c += 4 * kWave) {
-      u32x4 v0 = load16_any(s + ((size_t)c << 4));
-      u32x4 v1 = load16_any(s + ((size_t)(c + kWave) << 4));
-      u32x4 v2 = load16_any(s + ((size_t)(c + 2 * kWave) << 4));
-      u32x4 v3 = load16_any(s + ((size_t)(c + 3 * kWave) << 4));
-      store16_aligned(d + ((size_t)c << 4), v0);
-      store16_aligned(d + ((size_t)(c + kWave) << 4), v1);
-      store16_aligned(d + ((size_t)(c + 2 * kWave) << 4), v2);
-      store16_aligned(d + ((size_t)(c + 3 * kWave) << 4), v3);
-      if (CSUM) acc += words_sum(v0) + words_sum(v1) + words_sum(v2) + words_sum(v3);
-    }
-    // then two at a time, the second one predicated
-    for (; c < body; c += 2 * kWave) {
-      const bool two = c + kWave < body;
-      u32x4 v0 = load16_any(s + ((size_t)c << 4));
-      u32x4 v1 = {0, 0, 0, 0};
-      if (two) v1 = load16_any(s + ((size_t)(c + kWave) << 4));
-      store16_aligned(d + ((size_t)c << 4), v0);
-      if (two) store16_aligned(d + ((size_t)(c + kWave) << 4), v1);
-      if (CSUM) acc += words_sum(v0) + words_sum(v1);
-    }
-  } else {
-    const uint8_t *sa = s - p;
-    uint32_t base = 0;
-    for (; base + 126u < body; base += 252u) acc += funnel_step<4, CSUM>(sa, d, base, body, p, lane);
-    for (; base < body; base += 126u) acc += funnel_step<2, CSUM>(sa, d, base, body, p, lane);
+  r.d = dst + head;
+  r.p = (uint32_t)(uintptr_t)s & 15u;
+  r.sa = s - r.p;
+  r.lim = r.p ? body : body - 1;  // body == 0: lim wraps, guarded below
+  r.v0 = (u32x4){0, 0, 0, 0};
+  r.v1 = (u32x4){0, 0, 0, 0};
+  if (body) {
+    if (lane <= r.lim) r.v0 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)lane << 4));
+    if (63u + lane <= r.lim) r.v1 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)(63u + lane) << 4));
   }
-  if (edge) {
-    dst[eoff] = (uint8_t)eb;
-    if (CSUM) acc += ((uintptr_t)(dst + eoff) & 1u) ? (eb << 8) : eb;
+}
+
+// With CSUM returns this lane's share of the sum of the 16-bit little-endian
+// words the run's bytes fall into, a byte's position in its word being the
+// parity of its DESTINATION ADDRESS (packet offsets and addresses have the
+// same parity: ring bases, slot sizes and header lengths are even).
+template <bool CSUM>
+__device__ __forceinline__ uint32_t run_end(RunState &r, uint32_t lane)
+{
+  uint32_t acc = 0;
+  const u32x4 o0 = realign(r.v0, r.p);
+  const u32x4 o1 = realign(r.v1, r.p);
+  if (lane < 63 && lane < r.body) {
+    store16_aligned(r.d + ((size_t)lane << 4), o0);
+    if (CSUM) acc += words_sum(o0);
+  }
+  if (lane < 63 && 63u + lane < r.body) {
+    store16_aligned(r.d + ((size_t)(63u + lane) << 4), o1);
+    if (CSUM) acc += words_sum(o1);
+  }
+  for (uint32_t base = 126; base < r.body; base += 126) {
+    const uint32_t c0 = base + lane, c1 = base + 63u + lane;
+    u32x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+    if (c0 <= r.lim) v0 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c0 << 4));
+    if (c1 <= r.lim) v1 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c1 << 4));
+    const u32x4 q0 = realign(v0, r.p);
+    const u32x4 q1 = realign(v1, r.p);
+    if (lane < 63 && c0 < r.body) {
+      store16_aligned(r.d + ((size_t)c0 << 4), q0);
+      if (CSUM) acc += words_sum(q0);
+    }
+    if (lane < 63 && c1 < r.body) {
+      store16_aligned(r.d + ((size_t)c1 << 4), q1);
+      if (CSUM) acc += words_sum(q1);
+    }
+  }
+  if (r.edge) {
+    r.dst[r.eoff] = (uint8_t)r.eb;
+    if (CSUM) acc += ((uintptr_t)(r.dst + r.eoff) & 1u) ? (r.eb << 8) : r.eb;
   }
   return acc;
+}
+
+// Copy `len` bytes src -> dst with one wavefront.
+template <bool CSUM>
+__device__ __forceinline__ uint32_t copy_run(const uint8_t *__restrict__ src,
+                                             uint8_t *__restrict__ dst, uint32_t len, uint32_t lane)
+{
+  RunState r;
+  run_begin(r, src, dst, len, lane);
+  return run_end<CSUM>(r, lane);
 }
 
 // Byte-wise copy into / out of a bump-ring arena that is NOT mirrored, for a

@@ -293,6 +293,26 @@ __device__ __forceinline__ uint32_t item_of_wave(bool remap)
   return __builtin_amdgcn_readfirstlane(g * kWavesPerBlock + threadIdx.x / kWave);
 }
 
+// What the fused kernels need to derive a descriptor themselves when all
+// requests (responses) have one size and are cut by the fragmenting rule:
+// item f belongs to request f / per_req, is its fragment f % per_req, carries
+// min(remaining, mtu) bytes and starts i * mtu bytes into the request; request
+// r starts at cursor + r * size in the bump ring.
+struct RuleArgs {
+  const uint32_t *item_slot;
+  const uint32_t *item_len;  // gather: optional explicit lengths to hold against the rule
+  const uint32_t *first;     // CSR table to hold against the rule
+  uint64_t size;
+  uint32_t mtu;
+  uint32_t per_req;
+  uint32_t n_req;
+  uint32_t n_slots;
+  uint32_t single_wrap;  // n_req * size <= capacity: a request offset wraps at most once
+  const uint64_t *cursor_in;
+  uint64_t *cursor_out;
+  uint64_t *offsets_out;
+};
+
 struct GatherArgs {
   const u32x4 *desc;
   const uint64_t *req_off;
@@ -301,25 +321,63 @@ struct GatherArgs {
   uint32_t hl;
   uint32_t n_items;
   uint32_t remap;
-  const uint32_t *status;
+  uint32_t *status;
   AppDev app;
 };
 
+// Descriptor of item `item` from the rule; publishes the request offset and, on
+// the batch's last item, the advanced cursor.  Returns status bits.
+__device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &app, uint32_t item,
+                                              uint32_t n_items, uint32_t lane, uint32_t *slot,
+                                              uint32_t *len, uint32_t *off, uint32_t *r,
+                                              uint32_t *i, uint64_t *req_off)
+{
+  uint32_t bad = 0;
+  *r = item / g.per_req;
+  *i = item - *r * g.per_req;
+  *off = *i * g.mtu;
+  const uint64_t rem = g.size - *off;
+  *len = (uint32_t)(rem <= g.mtu ? rem : g.mtu);
+  *slot = g.item_slot[item];
+  if (*slot >= g.n_slots) bad |= kStBadSlot;
+  if (*i == 0 && g.first[*r] != item) bad |= kStBadTable;
+  *req_off = 0;
+  if (app.n_tensors == 0) {
+    uint64_t c0 = *g.cursor_in;
+    if (c0 >= app.cap) c0 %= app.cap;  // only after a set_cursor beyond the capacity
+    uint64_t o = c0 + (uint64_t)*r * g.size;
+    if (g.single_wrap) o = o >= app.cap ? o - app.cap : o;  // n_req * size <= capacity
+    else o %= app.cap;
+    *req_off = o;
+    if (lane == 0) {
+      if (*i == 0 && g.offsets_out) g.offsets_out[*r] = *req_off;
+      if (item == n_items - 1) {
+        uint64_t end = *req_off + g.size;  // size <= capacity
+        end = end >= app.cap ? end - app.cap : end;
+        *g.cursor_out = end;
+        if (g.offsets_out) g.offsets_out[g.n_req] = end;
+      }
+    }
+  }
+  return bad;
+}
+
 // Move [off, off+len) of request r's byte stream between a packet payload and
-// the application buffers.  TO_APP: packet -> app.
+// the application buffers.  TO_APP: packet -> app.  One copy_run call site:
+// the packed arena is walked as a single piece, tensor-major buffers as up to
+// SG_MAX_TENSORS pieces.
 template <bool TO_APP, bool CSUM>
 __device__ __forceinline__ uint32_t move_run(const AppDev &app, uint64_t req_off, uint32_t r,
                                              uint32_t off, uint8_t *pkt, uint32_t len, uint32_t lane)
 {
   uint32_t acc = 0;
-  if (app.n_tensors == 0) {
+  const bool packed = app.n_tensors == 0;
+  uint8_t *packed_ptr = nullptr;
+  if (packed) {
     const uint64_t o = req_off + off;  // < 2 * cap
-    if ((uint64_t)off + len > app.cap) return 0;  // request larger than the arena: refused by k_prep
-    if (app.mirrored || o + len <= app.cap) {
-      uint8_t *p = app.arena + o;
-      if (!app.mirrored && o >= app.cap) p -= app.cap;
-      acc = TO_APP ? copy_run<CSUM>(pkt, p, len, lane) : copy_run<CSUM>(p, pkt, len, lane);
-    } else {
+    if ((uint64_t)off + len > app.cap) return 0;  // request larger than the arena: refused elsewhere
+    if (!app.mirrored && o < app.cap && o + len > app.cap) {
+      // a run that crosses the end of an arena that is not mapped twice
       copy_run_wrapped(pkt, app.arena, app.cap, o, len, lane, TO_APP, pkt);
       if (CSUM) {
         for (uint32_t i = lane; i < len; i += kWave) {
@@ -327,38 +385,271 @@ __device__ __forceinline__ uint32_t move_run(const AppDev &app, uint64_t req_off
           acc += ((uintptr_t)(pkt + i) & 1u) ? (b << 8) : b;
         }
       }
+      return acc;
     }
-    return acc;
+    packed_ptr = app.arena + ((!app.mirrored && o >= app.cap) ? o - app.cap : o);
   }
+  const uint32_t n_pieces = packed ? 1u : app.n_tensors;
   uint64_t t0 = 0;
   uint32_t done = 0;
-  for (uint32_t t = 0; t < app.n_tensors && done < len; t++) {
-    const uint64_t t1 = t0 + app.tensor_size[t];
-    const uint64_t cur = (uint64_t)off + done;
-    if (cur < t1) {
+  for (uint32_t t = 0; t < n_pieces && done < len; t++) {
+    uint8_t *p;
+    uint32_t n;
+    if (packed) {
+      p = packed_ptr;
+      n = len;
+    } else {
+      const uint64_t t1 = t0 + app.tensor_size[t];
+      const uint64_t cur = (uint64_t)off + done;
+      t0 = t1;
+      if (cur >= t1) continue;
       const uint64_t room = t1 - cur;
-      const uint32_t n = room < (uint64_t)(len - done) ? (uint32_t)room : (len - done);
-      uint8_t *p = app.tensor_base[t] + (uint64_t)r * app.tensor_size[t] + (cur - t0);
-      if (TO_APP) copy_run<false>(pkt + done, p, n, lane);
-      else acc += copy_run<CSUM>(p, pkt + done, n, lane);
-      done += n;
+      n = room < (uint64_t)(len - done) ? (uint32_t)room : (len - done);
+      p = app.tensor_base[t] + (uint64_t)r * app.tensor_size[t] + (cur - (t1 - app.tensor_size[t]));
     }
-    t0 = t1;
+    acc += TO_APP ? copy_run<CSUM>(pkt + done, p, n, lane) : copy_run<CSUM>(p, pkt + done, n, lane);
+    done += n;
   }
   return acc;
 }
 
+// Keeps a kernel argument in a scalar register from this point on.  Placed on
+// every argument the hot path needs, at the top of a kernel, it makes the
+// compiler fetch them all in one burst of scalar loads instead of one
+// dependent round trip per first use.
+#define SG_PIN(x) asm volatile("" ::"s"(x))
+
+// Where [off, off+len) of request r's byte stream lives when that is ONE
+// contiguous piece of application memory; false when it is not (a run that
+// crosses the end of an arena mapped once, or a tensor boundary).
+__device__ __forceinline__ bool plain_target(const AppDev &app, uint64_t req_off, uint32_t r,
+                                             uint32_t off, uint32_t len, uint8_t **to)
+{
+  if (app.n_tensors == 0) {
+    if ((uint64_t)off + len > app.cap) return false;
+    uint64_t o = req_off + off;  // < 2 * capacity
+    if (!app.mirrored) {
+      if (o >= app.cap) o -= app.cap;
+      else if (o + len > app.cap) return false;
+    }
+    *to = app.arena + o;
+    return true;
+  }
+  uint64_t t0 = 0;
+  for (uint32_t t = 0; t < app.n_tensors; t++) {
+    const uint64_t t1 = t0 + app.tensor_size[t];
+    if (off < t1) {
+      if ((uint64_t)off + len > t1) return false;
+      *to = app.tensor_base[t] + (uint64_t)r * app.tensor_size[t] + (off - t0);
+      return true;
+    }
+    t0 = t1;
+  }
+  return false;
+}
+
+// A gather wavefront takes kGatherPerWave consecutive fragment runs and has the
+// loads of all of them in flight before it stores the first.  Measured on
+// 1400-byte fragments, one run per wavefront is fastest (two cost 2 %, three
+// 13 %): the wavefront count, not the bytes in flight per wavefront, is what
+// covers the HBM latency here.
+#ifndef SG_GATHER_PER_WAVE
+#define SG_GATHER_PER_WAVE 1
+#endif
+constexpr uint32_t kGatherPerWave = SG_GATHER_PER_WAVE;
+
+struct GatherItem {
+  bool live;    // there is something to move
+  bool plain;   // one contiguous destination piece: begin/end path
+  uint8_t *pkt; // payload in the slot
+  uint8_t *to;
+  uint32_t len, off, r;
+  uint64_t ro;
+};
+
+// Gather from descriptors written by the descriptor pass.
 __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
 {
-  const uint32_t item = item_of_wave(a.remap != 0);
-  if (item >= a.n_items) return;
-  if (*a.status) return;  // k_prep refused the batch: move nothing
+  const u32x4 *desc = a.desc;
+  const uint64_t *req_off = a.req_off;
+  const uint8_t *ring = a.ring;
+  const uint32_t slot_size = a.slot_size, hl = a.hl, n_items = a.n_items, remap = a.remap;
+  const uint32_t *status = a.status;
+  SG_PIN(desc); SG_PIN(req_off); SG_PIN(ring); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_items);
+  SG_PIN(remap); SG_PIN(status);
+  const uint32_t item0 = item_of_wave(remap != 0) * kGatherPerWave;
+  if (item0 >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  const u32x4 d = a.desc[item];
-  if (d[1] == 0 || d[3] == kInvalidReq) return;
-  const uint64_t ro = a.app.n_tensors == 0 ? a.req_off[d[3]] : 0;
-  uint8_t *pkt = const_cast<uint8_t *>(a.ring) + (size_t)d[0] * a.slot_size + a.hl;
-  move_run<true, false>(a.app, ro, d[3], d[2], pkt, d[1], lane);
+  if (sload(status)) return;  // the descriptor pass refused the batch: move nothing
+
+  GatherItem it[kGatherPerWave];
+  RunState rs[kGatherPerWave];
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++) {
+    const bool in = item0 + k < n_items;
+    const u32x4 d = sload(desc + (in ? item0 + k : item0));
+    it[k].live = in && d[1] != 0 && d[3] != kInvalidReq;
+    it[k].len = d[1];
+    it[k].off = d[2];
+    it[k].r = d[3];
+    it[k].ro = 0;
+    it[k].plain = false;
+    it[k].pkt = const_cast<uint8_t *>(ring) + (size_t)d[0] * slot_size + hl;
+    if (it[k].live) {
+      if (a.app.n_tensors == 0) it[k].ro = sload(req_off + d[3]);
+      it[k].plain = plain_target(a.app, it[k].ro, d[3], d[2], d[1], &it[k].to);
+    }
+  }
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++)
+    if (it[k].live && it[k].plain) run_begin(rs[k], it[k].pkt, it[k].to, it[k].len, lane);
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++) {
+    if (!it[k].live) continue;
+    if (it[k].plain) run_end<false>(rs[k], lane);
+    else move_run<true, false>(a.app, it[k].ro, it[k].r, it[k].off, it[k].pkt, it[k].len, lane);
+  }
+}
+
+// Gather without a descriptor pass: all requests have `size` bytes cut by the
+// fragmenting rule, so a wavefront derives its descriptors from its item
+// numbers (item f belongs to request f / per_req, is its fragment f % per_req,
+// carries min(remaining, mtu) bytes and starts i * mtu bytes into the request;
+// request r starts at cursor + r * size in the bump ring) and holds every
+// fragment's real length against the rule.
+struct GatherRuleArgs {
+  // hot: what a wavefront needs before its first payload load (64 bytes)
+  const uint8_t *ring;
+  const uint32_t *frag_slot;
+  uint8_t *dst;               // arena (packed) or the tensor (one tensor-major buffer)
+  const uint64_t *cursor_in;  // packed only
+  uint64_t size;
+  uint64_t cap;               // packed: arena capacity; 0: tensor-major
+  uint32_t n_items;
+  uint32_t per_req;
+  uint32_t mtu;
+  uint32_t slot_size;
+  // warm
+  uint32_t hl;
+  uint32_t n_slots;
+  uint32_t n_req;
+  uint32_t opts;  // kOptRemap | kOptMirrored | kOptSingleWrap | kOptMultiTensor
+  const uint32_t *frag_len;
+  const uint32_t *first;
+  uint64_t *offsets_out;
+  uint64_t *cursor_out;
+  uint32_t *status;
+  AppDev app;  // consulted for several tensor-major buffers only
+};
+constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptSingleWrap = 4u, kOptMultiTensor = 8u;
+
+// Does the payload_len of a BL58 header (u32 at byte 54) equal `len`?  Read as
+// the two aligned dwords around it through the scalar cache and compared half
+// by half (a combined value would be fetched with one misaligned vector load).
+// For kernels that only read the ring.
+__device__ __forceinline__ bool bl58_len_is(const uint8_t *slot, uint32_t len)
+{
+  const uint32_t w0 = sload(reinterpret_cast<const uint32_t *>(slot + 52));
+  const uint32_t w1 = sload(reinterpret_cast<const uint32_t *>(slot + 56));
+  return ((w0 >> 16) == (len & 0xffffu)) & ((w1 & 0xffffu) == (len >> 16));
+}
+
+__global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
+{
+  const uint8_t *ring = a.ring;
+  const uint32_t *frag_slot = a.frag_slot;
+  uint8_t *dst = a.dst;
+  const uint64_t *cursor_in = a.cursor_in;
+  const uint64_t size = a.size, cap = a.cap;
+  const uint32_t n_items = a.n_items, per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
+  const uint32_t hl = a.hl, n_slots = a.n_slots, opts = a.opts;
+  SG_PIN(ring); SG_PIN(frag_slot); SG_PIN(dst); SG_PIN(cursor_in); SG_PIN(size); SG_PIN(cap);
+  SG_PIN(n_items); SG_PIN(per_req); SG_PIN(mtu); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_slots);
+  SG_PIN(opts);
+
+  const uint32_t item0 = item_of_wave((opts & kOptRemap) != 0) * kGatherPerWave;
+  if (item0 >= n_items) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t slot[kGatherPerWave];
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++)
+    slot[k] = sload(frag_slot + (item0 + k < n_items ? item0 + k : item0));
+  uint64_t c0 = cap ? sload(cursor_in) : 0;
+  if (c0 >= cap && cap) c0 %= cap;  // only after a set_cursor beyond the capacity
+
+  GatherItem it[kGatherPerWave];
+  RunState rs[kGatherPerWave];
+  uint32_t idx[kGatherPerWave];
+  uint32_t bad = 0;
+  const uint32_t r0 = item0 / per_req;
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++) {
+    const uint32_t item = item0 + k;
+    // items of one wavefront are consecutive: at most one request boundary apart
+    uint32_t r = r0, i = item - r0 * per_req;
+    if (i >= per_req) { r += 1; i -= per_req; }
+    idx[k] = i;
+    it[k].live = item < n_items;
+    it[k].r = r;
+    it[k].off = i * mtu;
+    const uint64_t rem = size - it[k].off;
+    it[k].len = (uint32_t)(rem <= mtu ? rem : mtu);
+    if (it[k].live && slot[k] >= n_slots) {
+      bad |= kStBadSlot;
+      it[k].live = false;
+    }
+    it[k].pkt = const_cast<uint8_t *>(ring) + (size_t)slot[k] * slot_size;
+    it[k].ro = 0;
+    it[k].plain = !(opts & kOptMultiTensor);
+    it[k].to = nullptr;
+    if (!it[k].live) continue;
+    if (cap) {
+      // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
+      uint64_t ro = c0 + (uint64_t)r * size;
+      if (opts & kOptSingleWrap) ro = ro >= cap ? ro - cap : ro;  // n_req * size <= capacity
+      else ro %= cap;
+      it[k].ro = ro;
+      if (lane == 0) {
+        if (i == 0 && a.offsets_out) a.offsets_out[r] = ro;
+        if (item == n_items - 1) {
+          uint64_t end = ro + size;  // size <= capacity
+          end = end >= cap ? end - cap : end;
+          *a.cursor_out = end;
+          if (a.offsets_out) a.offsets_out[a.n_req] = end;
+        }
+      }
+      if (it[k].plain) {
+        uint64_t o = ro + it[k].off;  // < 2 * capacity
+        if (!(opts & kOptMirrored)) {
+          if (o >= cap) o -= cap;
+          else if (o + it[k].len > cap) it[k].plain = false;  // crosses the end of an arena mapped once
+        }
+        it[k].to = dst + o;
+      }
+    } else if (it[k].plain) {
+      it[k].to = dst + (uint64_t)r * size + it[k].off;
+    }
+  }
+  // copying the ruled length stays inside the slot whatever the header says
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++)
+    if (it[k].live && it[k].plain) run_begin(rs[k], it[k].pkt + hl, it[k].to, it[k].len, lane);
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++) {
+    if (!it[k].live) continue;
+    if (it[k].plain) run_end<false>(rs[k], lane);
+    else move_run<true, false>(a.app, it[k].ro, it[k].r, it[k].off, it[k].pkt + hl, it[k].len, lane);
+  }
+#pragma unroll
+  for (uint32_t k = 0; k < kGatherPerWave; k++) {
+    if (!it[k].live) continue;
+    const uint32_t item = item0 + k;
+    const bool as_ruled = a.frag_len ? sload(a.frag_len + item) == it[k].len
+                                     : bl58_len_is(it[k].pkt, it[k].len);
+    if (!as_ruled) bad |= kStNotRule;
+    if (idx[k] == 0 && sload(a.first + it[k].r) != item) bad |= kStBadTable;
+  }
+  if (bad && lane == 0) atomicOr(a.status, bad);
 }
 
 struct ScatterArgs {
@@ -377,27 +668,43 @@ struct ScatterArgs {
   uint32_t n_items;
   uint32_t remap;
   uint32_t *status;
+  RuleArgs rule;
   AppDev app;
 };
 
-template <bool FULL_CSUM>
+template <bool FULL_CSUM, bool FUSED>
 __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
   const uint32_t item = item_of_wave(a.remap != 0);
   if (item >= a.n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  if (*a.status) return;  // k_prep refused the batch: move nothing
-  const u32x4 d = a.desc[item];
-  const uint32_t r = d[3];
-  if (r == kInvalidReq) return;
-  const uint32_t f0 = a.first[r];
-  const uint32_t nf = a.first[r + 1] - f0;
+  u32x4 d;
+  uint32_t r, f0, nf;
+  uint64_t ro;
+  if (!FUSED) {
+    if (*a.status) return;  // the descriptor pass refused the batch: move nothing
+    d = a.desc[item];
+    r = d[3];
+    if (r == kInvalidReq) return;
+    f0 = a.first[r];
+    nf = a.first[r + 1] - f0;
+    ro = a.app.n_tensors == 0 ? a.req_off[r] : 0;
+  } else {
+    uint32_t slot_i, len, off, i;
+    const uint32_t bad = rule_desc(a.rule, a.app, item, a.n_items, lane, &slot_i, &len, &off, &r, &i, &ro);
+    if (bad) {
+      if (lane == 0) atomicOr(a.status, bad);
+      return;
+    }
+    d = (u32x4){slot_i, len, off, r};
+    f0 = item - i;
+    nf = a.rule.per_req;
+  }
   uint32_t hs = a.hdr_src_slot[item];
   if (hs >= a.rx_n_slots) {
     if (lane == 0) atomicOr(a.status, kStBadSlot);
     return;
   }
-  const uint64_t ro = a.app.n_tensors == 0 ? a.req_off[r] : 0;
   uint8_t *slot = a.tx + (size_t)d[0] * a.tx_slot_size;
 
   // read the request header before anything of this slot is overwritten
@@ -565,9 +872,10 @@ int check_app(sg_hip_ctx *c, const sg_app_desc &a, AppDev *out, uint64_t *max_re
 
 // Launch geometry for one wavefront per item; with the XCD-aware order the
 // grid is padded to whole rounds of kXcds * kXcdRun workgroups.
-void geometry(uint32_t n_items, bool want_remap, uint32_t *grid, uint32_t *remap)
+void geometry(uint32_t n_items, uint32_t per_wave, bool want_remap, uint32_t *grid, uint32_t *remap)
 {
-  const uint32_t groups = (n_items + kWavesPerBlock - 1) / kWavesPerBlock;
+  const uint32_t per_group = kWavesPerBlock * per_wave;
+  const uint32_t groups = (n_items + per_group - 1) / per_group;
   const uint32_t round = kXcds * kXcdRun;
   if (want_remap && groups >= 2 * round) {
     *grid = (groups + round - 1) / round * round;
@@ -740,12 +1048,13 @@ int sg_hip_sync(sg_hip_ctx *c)
   if (st) {
     HIP_TRY(c, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
     HIP_TRY(c, hipStreamSynchronize(c->stream));
-    return fail(c, SG_E_DATA, "kernel refused input:%s%s%s%s%s",
+    return fail(c, SG_E_DATA, "kernel refused input:%s%s%s%s%s%s",
                 (st & kStBadSlot) ? " slot index beyond ring;" : "",
                 (st & kStBadLen) ? " fragment longer than a slot holds;" : "",
                 (st & kStBadSize) ? " request larger than its destination;" : "",
                 (st & kStBadFrames) ? " frame count disagrees with size/mtu;" : "",
-                (st & kStBadTable) ? " CSR table does not tile the items;" : "");
+                (st & kStBadTable) ? " CSR table does not tile the items;" : "",
+                (st & kStNotRule) ? " a fragment's length departs from the fragmenting rule;" : "");
   }
   return SG_OK;
 }
@@ -881,6 +1190,50 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   if (rc != SG_OK) return rc;
   DeviceGuard g(c->device);
 
+  const uint32_t hl0 = hdr_len_of(a->ring.hdr_profile);
+  if (a->flags & SG_F_RULE_FRAGS) {
+    // one size, cut by the rule: no descriptor pass, the copy kernel derives everything
+    if (!a->fixed_req_size || !a->mtu) return fail(c, SG_E_INVAL, "SG_F_RULE_FRAGS needs fixed_req_size and mtu");
+    if ((uint64_t)a->mtu + hl0 > a->ring.slot_size) return fail(c, SG_E_INVAL, "mtu %u + %u header bytes does not fit a %u-byte slot", a->mtu, hl0, a->ring.slot_size);
+    const uint64_t per = (a->fixed_req_size + a->mtu - 1) / a->mtu;
+    if (per * a->n_req != a->n_frags) return fail(c, SG_E_INVAL, "%u requests of %llu bytes at mtu %u are %llu fragments, not %u", a->n_req, (unsigned long long)a->fixed_req_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frags);
+    if (a->fixed_req_size > 0xffffffffull || (app.n_tensors == 0 ? a->fixed_req_size > app.cap : a->fixed_req_size > max_req_bytes))
+      return fail(c, SG_E_INVAL, "request size %llu does not fit its destination", (unsigned long long)a->fixed_req_size);
+    GatherRuleArgs ga;
+    memset(&ga, 0, sizeof ga);
+    ga.ring = static_cast<const uint8_t *>(a->ring.base);
+    ga.frag_slot = a->frag_slot;
+    ga.dst = app.n_tensors == 0 ? app.arena : app.tensor_base[0];
+    ga.cursor_in = c->cursors + 0 + c->parity[0];
+    ga.cursor_out = c->cursors + 0 + (c->parity[0] ^ 1u);
+    if (app.n_tensors == 0) c->parity[0] ^= 1u;
+    ga.size = a->fixed_req_size;
+    ga.cap = app.n_tensors == 0 ? app.cap : 0;
+    ga.n_items = a->n_frags;
+    ga.per_req = (uint32_t)per;
+    ga.mtu = a->mtu;
+    ga.slot_size = a->ring.slot_size;
+    ga.hl = hl0;
+    ga.n_slots = a->ring.n_slots;
+    ga.n_req = a->n_req;
+    ga.frag_len = a->frag_len;
+    ga.first = a->req_first;
+    ga.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
+    ga.status = c->status;
+    ga.app = app;
+    uint32_t grid, remap;
+    geometry(a->n_frags, kGatherPerWave, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
+    ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
+              ((app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_req_size <= app.cap) ? kOptSingleWrap : 0u) |
+              (app.n_tensors > 1 ? kOptMultiTensor : 0u);
+    rc = prof_begin(c, 1);
+    if (rc != SG_OK) return rc;
+    k_gather_rule<<<grid, kBlock, 0, c->stream>>>(ga);
+    rc = prof_end(c);
+    if (rc != SG_OK) return rc;
+    return finish(c, a->flags);
+  }
+
   PrepArgs p;
   memset(&p, 0, sizeof p);
   p.mode = 0;
@@ -921,7 +1274,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.status = c->status;
     ga.app = app;
     uint32_t grid;
-    geometry(a->n_frags, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
+    geometry(a->n_frags, kGatherPerWave, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
     k_gather<<<grid, kBlock, 0, c->stream>>>(ga);
@@ -952,6 +1305,51 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   rc = check_app(c, a->app, &app, &max_req_bytes);
   if (rc != SG_OK) return rc;
   DeviceGuard g(c->device);
+
+  const bool fused = a->resp_size == nullptr && !(a->flags & SG_F_NO_FUSE);
+  if (fused) {
+    if (a->fixed_resp_size == 0 || a->fixed_resp_size > 0xffffffffull)
+      return fail(c, SG_E_INVAL, "fixed response size %llu out of range", (unsigned long long)a->fixed_resp_size);
+    const uint64_t per = (a->fixed_resp_size + a->mtu - 1) / a->mtu;
+    if (per * a->n_req != a->n_frames) return fail(c, SG_E_INVAL, "%u responses of %llu bytes at mtu %u are %llu frames, not %u", a->n_req, (unsigned long long)a->fixed_resp_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frames);
+    if (app.n_tensors == 0 ? a->fixed_resp_size > app.cap : a->fixed_resp_size > max_req_bytes)
+      return fail(c, SG_E_INVAL, "response size %llu does not fit its source", (unsigned long long)a->fixed_resp_size);
+    ScatterArgs sa;
+    memset(&sa, 0, sizeof sa);
+    sa.hdr_src_slot = a->hdr_src_slot;
+    sa.rx = static_cast<const uint8_t *>(a->rx.base);
+    sa.rx_slot_size = a->rx.slot_size;
+    sa.rx_n_slots = a->rx.n_slots;
+    sa.tx = static_cast<uint8_t *>(a->tx.base);
+    sa.tx_slot_size = a->tx.slot_size;
+    sa.hl = hl;
+    sa.ref64 = a->tx.hdr_profile == SG_HDR_REF64;
+    sa.flags = a->flags & 0xfu;
+    sa.n_items = a->n_frames;
+    sa.status = c->status;
+    sa.app = app;
+    sa.rule.item_slot = a->tx_slot;
+    sa.rule.first = a->resp_first;
+    sa.rule.size = a->fixed_resp_size;
+    sa.rule.mtu = a->mtu;
+    sa.rule.per_req = (uint32_t)per;
+    sa.rule.n_req = a->n_req;
+    sa.rule.n_slots = a->tx.n_slots;
+    sa.rule.single_wrap = app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_resp_size <= app.cap;
+    sa.rule.cursor_in = c->cursors + 2 + c->parity[1];
+    sa.rule.cursor_out = c->cursors + 2 + (c->parity[1] ^ 1u);
+    if (app.n_tensors == 0) c->parity[1] ^= 1u;
+    sa.rule.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
+    uint32_t grid;
+    geometry(a->n_frames, 1, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    rc = prof_begin(c, 2);
+    if (rc != SG_OK) return rc;
+    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, true><<<grid, kBlock, 0, c->stream>>>(sa);
+    else k_scatter<false, true><<<grid, kBlock, 0, c->stream>>>(sa);
+    rc = prof_end(c);
+    if (rc != SG_OK) return rc;
+    return finish(c, a->flags);
+  }
 
   PrepArgs p;
   memset(&p, 0, sizeof p);
@@ -1000,11 +1398,11 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.status = c->status;
     sa.app = app;
     uint32_t grid;
-    geometry(a->n_frames, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry(a->n_frames, 1, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true><<<grid, kBlock, 0, c->stream>>>(sa);
-    else k_scatter<false><<<grid, kBlock, 0, c->stream>>>(sa);
+    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, false><<<grid, kBlock, 0, c->stream>>>(sa);
+    else k_scatter<false, false><<<grid, kBlock, 0, c->stream>>>(sa);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }

@@ -126,7 +126,7 @@ class SgContext:
     def gather_args(ring: RingRef, frag_slot: torch.Tensor, frag_len: Optional[torch.Tensor],
                     req_first: torch.Tensor, n_req: int, n_frags: int, app: AppRef,
                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0,
-                    fixed_req_size: int = 0) -> capi.GatherArgs:
+                    fixed_req_size: int = 0, mtu: int = 0) -> capi.GatherArgs:
         a = capi.GatherArgs()
         a.ring = ring.desc()
         a.frag_slot = frag_slot.data_ptr()
@@ -138,6 +138,7 @@ class SgContext:
         a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
         a.flags = flags
         a.fixed_req_size = int(fixed_req_size)
+        a.mtu = int(mtu)
         return a
 
     def gather_batch(self, *args, **kw) -> None:
@@ -286,10 +287,12 @@ class DeviceWorkload:
         return outs
 
     def gather(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False,
-               fixed: bool = True) -> None:
+               fixed: bool = True, rule: bool = False) -> None:
         """``fixed``: declare the common request size when all requests have one
-        (offsets are then multiples of it instead of a prefix scan)."""
-        key = ("g", use_frag_len, fixed)
+        (offsets are then multiples of it instead of a prefix scan).  ``rule``:
+        also state that fragments follow the fragmenting rule, which lets the
+        copy kernel work without a descriptor pass."""
+        key = ("g", use_frag_len, fixed, rule)
         a = self._args.get(key)
         if a is None:
             need_len = use_frag_len or self.w.profile != 0
@@ -297,12 +300,15 @@ class DeviceWorkload:
             fx = int(sizes[0]) if fixed and len(sizes) and bool((sizes == sizes[0]).all()) else 0
             a = ctx.gather_args(self.rx, self.frag_slot, self.frag_len if need_len else None,
                                 self.req_first, self.n_req, self.n_frags, self.req_app,
-                                self.req_offsets, 0, fixed_req_size=fx)
+                                self.req_offsets, 0, fixed_req_size=fx, mtu=self.w.mtu)
+            a._base_flags = capi.F_RULE_FRAGS if (rule and fx) else 0
             self._args[key] = a
-        a.flags = flags
+        a.flags = flags | a._base_flags
         ctx.gather_batch_raw(a)
 
-    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True) -> None:
+    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True) -> None:
+        if not fuse:
+            flags |= capi.F_NO_FUSE
         key = ("s", fixed)
         a = self._args.get(key)
         if a is None:

@@ -14,17 +14,28 @@ pytestmark = pytest.mark.gpu
 CASES = [(1, None), (2, None), (3, None), (4, None), (5, None), (2, 1), (4, 7), (5, 2)]
 
 
-@pytest.mark.parametrize("fixed", [True, False], ids=["fixed", "scan"])
+MODES = {
+    # request offsets by prefix scan, descriptor pass for gather and scatter
+    "scan": dict(fixed=False, rule=False, fuse=False),
+    # one declared size: offsets are multiples, descriptor pass still runs
+    "fixed": dict(fixed=True, rule=False, fuse=False),
+    # one declared size + fragmenting rule: copy kernels derive the descriptors
+    "rule": dict(fixed=True, rule=True, fuse=True),
+}
+
+
+@pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("cfg,n_req", CASES)
-def test_gather_scatter_bit_exact(ctx, cfg, n_req, fixed):
+def test_gather_scatter_bit_exact(ctx, cfg, n_req, mode):
+    fixed, rule, fuse = MODES[mode]["fixed"], MODES[mode]["rule"], MODES[mode]["fuse"]
     w = synth.make_workload(cfg, n_req)
-    print(f"case cfg={cfg} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} fixed={fixed}",
+    print(f"case cfg={cfg} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} mode={mode}",
           flush=True)
     dw = DeviceWorkload(w)
     ctx.set_cursor(0, 0)
     ctx.set_cursor(1, 0)
 
-    dw.gather(ctx, fixed=fixed)
+    dw.gather(ctx, fixed=fixed, rule=rule)
     if w.in_tensor_sizes:
         exp, _, _ = expected_gather(w)
         for t, e in zip(dw.in_tensors, exp):
@@ -39,7 +50,7 @@ def test_gather_scatter_bit_exact(ctx, cfg, n_req, fixed):
         assert ctx.get_cursor(0) == cur
         gathered = exp
 
-    dw.scatter(ctx, fixed=fixed)
+    dw.scatter(ctx, fixed=fixed, fuse=fuse)
     exp_tx, offs, cur = expected_scatter(w, gathered, resp_cap=dw.resp_app.cap if not w.out_tensor_sizes else None)
     got_tx = dw.tx_ring.cpu().numpy()
     assert np.array_equal(got_tx, exp_tx), first_diff(got_tx, exp_tx)
