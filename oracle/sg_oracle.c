@@ -464,7 +464,9 @@ int64_t sgo_gather_batch(const sgo_ring *ring, const uint32_t *frag_slot, const 
   }
   for (uint32_t r = 0; r < n_req; r++) {
     uint32_t f0 = req_first[r], f1 = req_first[r + 1];
-    if (f1 - f0 > SGO_MAX_BI_SIZE) { runs = -1; break; }
+    /* the run table has room for 1023 lengths (p2p_bufs.h:37): a 1024th run
+     * would overwrite num_items in the reference.  Refused here. */
+    if (f1 - f0 > SGO_MAX_BI_SIZE - 1) { runs = -1; break; }
     uint64_t total = 0;
     bufs->num_items = (uint16_t)(f1 - f0);
     for (uint32_t f = f0; f < f1; f++) {
@@ -524,7 +526,7 @@ int64_t sgo_scatter_batch(const sgo_ring *rx, const sgo_ring *tx, const uint32_t
     uint64_t size = resp_size ? resp_size[r] : fixed_resp_size;
     uint32_t f0 = resp_first[r], f1 = resp_first[r + 1];
     uint32_t nf = f1 - f0;
-    if (nf > SGO_MAX_BI_SIZE || nf != sgo_num_frames(size, mtu)) { frames = -1; break; }
+    if (nf > SGO_MAX_BI_SIZE - 1 || nf != sgo_num_frames(size, mtu)) { frames = -1; break; }
     uint64_t base_off = 0;
     if (app->n_tensors == 0) {
       base_off = nf ? sgo_tring_get_next(&tr, size) : tr.prev_offset;

@@ -208,7 +208,7 @@ def _assemble(name: str, cfg: int, seed: int, rng: np.random.Generator, profile:
     assert hl + mtu <= slot_size
     sizes = np.array([len(p) for p in payloads], dtype=np.uint64)
     nfr = np.array([num_frames(int(s), mtu) for s in sizes], dtype=np.uint32)
-    assert nfr.max(initial=0) <= 1024, "a request spans at most MAX_BI_SIZE fragments"
+    assert nfr.max(initial=0) <= 1023, "a reference run table describes at most 1023 runs"
     first = np.zeros(n_req + 1, dtype=np.int64)
     np.cumsum(nfr, out=first[1:])
     n_frags = int(first[-1])

@@ -1,0 +1,381 @@
+"""Edge cases of the HIP path through the C ABI: every alignment phase, the
+per-request entry points, the reference's own 64-byte header profile, ragged
+and empty tables, wrap-around arenas, refused input, and size-independent
+properties at the benchmark's full sizes.  Bit-exact against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from splitrpc_amd import capi, synth
+from splitrpc_amd.engine import AppRef, DeviceWorkload, RingRef, SgContext, SgError, to_dev
+
+from helpers import expected_gather, expected_scatter, first_diff
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev_u8(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+# ---------------------------------------------------------------- per-request entry points
+
+def test_copy_runs_every_phase_and_length(ctx):
+    """sg_hip_gather / sg_hip_scatter: host-built run tables, all 16 x 16
+    source/destination phases, lengths around every chunk boundary."""
+    rng = np.random.default_rng(100)
+    src_h = rng.integers(0, 256, 1 << 20, dtype=np.uint8)
+    src = dev_u8(src_h)
+    dst = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+    want = np.zeros(1 << 20, np.uint8)
+    lens = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 112, 1007, 1008, 1009, 1400, 2016, 2017, 2032,
+            4095, 8800]
+    runs, so, do = [], 64, 64
+    for sp in range(16):
+        for dp in range(16):
+            ln = lens[(sp * 16 + dp) % len(lens)]
+            s = (so + 15) // 16 * 16 + sp
+            d = (do + 15) // 16 * 16 + dp
+            runs.append((s, d, ln))
+            want[d:d + ln] = src_h[s:s + ln]
+            so, do = s + ln + 40, d + ln + 40
+    print(f"case copy_runs: {len(runs)} runs", flush=True)
+    for scatter in (False, True):
+        dst.zero_()
+        for k in range(0, len(runs), 500):
+            part = runs[k:k + 500]
+            ctx.copy_runs([src.data_ptr() + s for s, _, _ in part], [dst.data_ptr() + d for _, d, _ in part],
+                          [n for _, _, n in part], scatter=scatter)
+        got = dst.cpu().numpy()
+        assert np.array_equal(got, want), first_diff(got, want)
+
+
+def test_copy_runs_long_run_is_cut(ctx):
+    rng = np.random.default_rng(101)
+    n = 3_000_003
+    src_h = rng.integers(0, 256, n + 64, dtype=np.uint8)
+    src, dst = dev_u8(src_h), torch.zeros(n + 64, dtype=torch.uint8, device=DEV)
+    ctx.copy_runs([src.data_ptr() + 3], [dst.data_ptr() + 9], [n])
+    got = dst.cpu().numpy()
+    assert np.array_equal(got[9:9 + n], src_h[3:3 + n]) and not got[:9].any() and not got[9 + n:].any()
+
+
+def test_run_table_overflow_is_refused(ctx):
+    skb = capi.SkBuf()
+    skb.num_items = 1024  # len[] holds 1023 (src/p2p_bufs.h:37)
+    rc = ctx.lib.sg_hip_gather(ctx.h, C.byref(skb))
+    assert rc == capi.SG_E_INVAL
+
+
+@pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64])
+@pytest.mark.parametrize("flags", [0, synth.F_UDP_CSUM_PSEUDO, synth.F_UDP_CSUM_PSEUDO | synth.F_REF_QUIRKS,
+                                   synth.F_IPV4_CSUM | synth.F_UDP_CSUM_PSEUDO])
+def test_swap_hdrs_in_place(ctx, profile, flags):
+    """sg_hip_swap_hdrs against swap + routing + lengths + sums of the oracle."""
+    rng = np.random.default_rng(102 + flags)
+    n, slot = 37, 256
+    hl = synth.hdr_len(profile)
+    buf = rng.integers(0, 256, n * slot, dtype=np.uint8)
+    buf.reshape(n, slot)[:, 14] = 0x45
+    dev = dev_u8(buf)
+    payload_size, mtu = 36 * 1400 + 333, 1400
+    ctx.swap_hdrs([dev.data_ptr() + i * slot for i in range(n)], profile, payload_size, mtu, flags)
+    want = buf.copy().reshape(n, slot)
+    L = oracle.lib()
+    for i in range(n):
+        h = want[i, :64].copy()
+        L.sgo_rewrite_resp_hdr(h.ctypes.data_as(C.c_void_p), profile, flags, i, n,
+                               L.sgo_frame_len(payload_size, mtu, i))
+        want[i, :hl] = h[:hl]
+    got = dev.cpu().numpy().reshape(n, slot)
+    assert np.array_equal(got, want), first_diff(got.reshape(-1), want.reshape(-1))
+
+
+# ---------------------------------------------------------------- header profiles, flags
+
+@pytest.mark.parametrize("cfg,n", [(1, 9), (2, 2), (5, 1)])
+@pytest.mark.parametrize("extra", [0, synth.F_REF_QUIRKS, synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL])
+def test_ref64_profile(ctx, cfg, n, extra):
+    """The reference's own p2p_rpc_hdr: 64 bytes, lengths from the NIC table."""
+    w = synth.make_workload(cfg, n, profile=synth.HDR_REF64)
+    w.flags |= extra
+    print(f"case ref64 cfg={cfg} n={n} flags={w.flags}", flush=True)
+    dw = DeviceWorkload(w)
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    dw.gather(ctx, use_frag_len=True)
+    exp, offs, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    assert np.array_equal(dw.req_arena.cpu().numpy(), exp)
+    dw.scatter(ctx)
+    exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
+    got = dw.tx_ring.cpu().numpy()
+    assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
+
+
+def test_ref64_without_length_table_is_refused(ctx):
+    w = synth.make_workload(1, 2, profile=synth.HDR_REF64)
+    dw = DeviceWorkload(w)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app)
+    assert e.value.code == capi.SG_E_INVAL
+
+
+@pytest.mark.parametrize("flags", [0, 1, 2, 3, 4, 5, 6, 7, 10, 15])
+def test_every_checksum_flag_combination(ctx, flags):
+    w = synth.make_custom([5000, 77, 1400, 1401, 9], [3000, 1, 1400, 2801, 4200], seed=40 + flags, flags=flags)
+    dw = DeviceWorkload(w)
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    dw.gather(ctx)
+    exp, _, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    assert np.array_equal(dw.req_arena.cpu().numpy(), exp)
+    dw.scatter(ctx)
+    exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
+    got = dw.tx_ring.cpu().numpy()
+    assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
+
+
+# ---------------------------------------------------------------- ragged, empty, large
+
+def test_ragged_sizes_one_byte_to_many_fragments(ctx):
+    # last: 1023 fragments, what a reference run table can describe (len[] has 1023 entries)
+    sizes = [1, 2, 15, 16, 17, 57, 58, 59, 1399, 1400, 1401, 2799, 2800, 2801, 70000, 3, 1432200]
+    resp = [s // 3 + 1 for s in sizes]
+    w = synth.make_custom(sizes, resp, seed=7, flags=synth.F_UDP_CSUM_PSEUDO | synth.F_IPV4_CSUM)
+    assert int((w.req_first[1:] - w.req_first[:-1]).max()) == 1023
+    print(f"case ragged frags={w.n_frags}", flush=True)
+    dw = DeviceWorkload(w)
+    for fixed in (False, True):
+        ctx.set_cursor(0, 0)
+        ctx.set_cursor(1, 0)
+        dw.req_arena.zero_()
+        dw.gather(ctx, fixed=fixed)
+        exp, offs, cur = expected_gather(w, arena_cap=dw.req_app.cap)
+        got = dw.req_arena.cpu().numpy()
+        assert np.array_equal(got, exp), first_diff(got, exp)
+        assert np.array_equal(dw.req_offsets.cpu().numpy().view(np.uint64), offs)
+        dw.scatter(ctx, fixed=fixed)
+        exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
+        assert np.array_equal(dw.tx_ring.cpu().numpy(), exp_tx)
+
+
+def test_empty_requests_and_empty_batch(ctx):
+    """Requests without fragments move nothing and take no arena space."""
+    w = synth.make_custom([3000, 100, 4500], [10, 10, 10], seed=9)
+    dw = DeviceWorkload(w)
+    # CSR with empty requests interleaved: [r0, -, r1, -, -, r2, -]
+    f = w.req_first.astype(np.uint32)
+    first = np.array([f[0], f[1], f[1], f[2], f[2], f[2], f[3], f[3]], np.uint32)
+    n_req = len(first) - 1
+    offs = torch.zeros(n_req + 1, dtype=torch.int64, device=DEV)
+    ctx.set_cursor(0, 0)
+    ctx.gather_batch(dw.rx, dw.frag_slot, None, to_dev(first, DEV), n_req, dw.n_frags, dw.req_app, offs)
+    exp, _, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    assert np.array_equal(dw.req_arena.cpu().numpy(), exp)
+    o = offs.cpu().numpy().view(np.uint64).tolist()
+    s0, s1, s2 = (int(x) for x in w.req_sizes)  # batch order is completion order
+    end = (s0 + s1 + s2) % dw.req_app.cap
+    assert o == [0, s0, s0, s0 + s1, s0 + s1, s0 + s1, end, end]
+    # n_req == 0 is a no-op
+    ctx.gather_batch(dw.rx, dw.frag_slot, None, to_dev(first, DEV), 0, 0, dw.req_app)
+
+
+# ---------------------------------------------------------------- arena wrap, cursor persistence
+
+@pytest.mark.parametrize("mode", ["scan", "rule"])
+def test_arena_wrap_and_cursor_persistence(ctx, mode):
+    """Two calls in a row continue the bump ring; a request that crosses the end
+    of an arena mapped once is split byte-exactly."""
+    rule = mode == "rule"
+    sizes = [4200] * 5 if rule else [3000, 5000, 700, 4100, 2222]
+    w = synth.make_custom(sizes, [64] * 5, seed=10)
+    total = int(sum(sizes))
+    cap = total - 1000  # the batch wraps
+    dw = DeviceWorkload(w)
+    arena = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+    app = AppRef(arena=arena, cap=cap)
+    offs = torch.zeros(w.n_req + 1, dtype=torch.int64, device=DEV)
+    ctx.set_cursor(0, 777)
+    cur = 777
+    want = np.zeros(cap, np.uint8)
+    for call in range(3):
+        flags = capi.F_RULE_FRAGS if rule else 0
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, app, offs,
+                         flags=flags, fixed_req_size=sizes[0] if rule else 0, mtu=w.mtu)
+        exp, eoffs, ecur = oracle.gather(w, arena_cap=cap, cursor=cur, out=want)
+        got = arena.cpu().numpy()
+        assert np.array_equal(got, exp), f"call {call}: " + first_diff(got, exp)
+        assert np.array_equal(offs.cpu().numpy().view(np.uint64), eoffs)
+        assert ctx.get_cursor(0) == ecur
+        cur = ecur
+
+
+def test_odd_arena_base_and_tensor_major_split(ctx):
+    """Destination phases other than the allocator's: arena and tensors at odd
+    byte offsets; a fragment that straddles the tensor boundary is split."""
+    w = synth.make_workload(3, 33)
+    dw = DeviceWorkload(w)
+    for shift in (1, 7, 8, 13):
+        backing = [torch.zeros(w.n_req * s + 64, dtype=torch.uint8, device=DEV) for s in w.in_tensor_sizes]
+        tensors = [b[shift:shift + w.n_req * s] for b, s in zip(backing, w.in_tensor_sizes)]
+        app = AppRef(tensors=tensors, sizes=w.in_tensor_sizes)
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, app)
+        exp, _, _ = expected_gather(w)
+        for t, e, b in zip(tensors, exp, backing):
+            assert np.array_equal(t.cpu().numpy(), e)
+            bb = b.cpu().numpy()
+            assert not bb[:shift].any() and not bb[shift + e.size:].any()  # nothing written outside
+
+
+# ---------------------------------------------------------------- refused input
+
+def test_bad_slot_index_refuses_the_whole_batch(ctx):
+    w = synth.make_workload(1, 4)
+    dw = DeviceWorkload(w)
+    bad = w.frag_slot.copy()
+    bad[5] = w.n_slots + 3
+    dw.req_arena.fill_(0xAB)
+    ctx.set_cursor(0, 0)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(dw.rx, to_dev(bad, DEV), None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app,
+                         dw.req_offsets)
+    assert e.value.code == capi.SG_E_DATA
+    assert bool((dw.req_arena == 0xAB).all()), "a refused batch must move nothing"
+    # the context is usable again afterwards
+    ctx.set_cursor(0, 0)
+    dw.gather(ctx)
+    exp, _, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    assert np.array_equal(dw.req_arena.cpu().numpy(), exp)
+
+
+def test_bad_tables_and_sizes_are_refused(ctx):
+    w = synth.make_workload(1, 4)
+    dw = DeviceWorkload(w)
+    first = w.req_first.copy()
+    first[2] = first[3] + 1  # not monotone
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, to_dev(first, DEV), dw.n_req, dw.n_frags, dw.req_app)
+    assert e.value.code == capi.SG_E_DATA
+    # a header that claims more payload than a slot holds
+    ring = w.ring.copy().reshape(w.n_slots, w.slot_size)
+    ring[int(w.frag_slot[1]), 54:58] = np.frombuffer((5000).to_bytes(4, "little"), np.uint8)
+    rx = RingRef(dev_u8(ring.reshape(-1)), w.n_slots, w.slot_size, w.profile)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app)
+    assert e.value.code == capi.SG_E_DATA
+    # declared fragmenting rule that the ring does not follow
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app,
+                         flags=capi.F_RULE_FRAGS, fixed_req_size=3136, mtu=1400)
+    assert e.value.code == capi.SG_E_DATA
+    # sizes beyond what the context was created for
+    small = SgContext(0, max_reqs=2, max_frames=4)
+    with pytest.raises(SgError) as e:
+        small.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app)
+    assert e.value.code == capi.SG_E_INVAL
+    small.close()
+    # response frame count that disagrees with size / mtu
+    with pytest.raises(SgError) as e:
+        ctx.scatter_batch(dw.rx, dw.tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first,
+                          to_dev(np.full(w.n_req, 5000, np.uint64), DEV), 0, dw.n_req, dw.n_frames, w.mtu,
+                          dw.resp_app, flags=capi.F_NO_FUSE)
+    assert e.value.code == capi.SG_E_DATA
+
+
+# ---------------------------------------------------------------- properties at full size
+
+def be_sum_rows(rows: np.ndarray) -> np.ndarray:
+    a = rows.astype(np.uint64)
+    if a.shape[1] & 1:
+        a = np.concatenate([a, np.zeros((a.shape[0], 1), np.uint64)], axis=1)
+    s = ((a[:, 0::2] << 8) | a[:, 1::2]).sum(axis=1)
+    for _ in range(4):
+        s = (s & 0xFFFF) + (s >> 16)
+    return s
+
+
+def test_full_size_jumbo_checksums_verify(ctx):
+    """Workload 5 at full size: every response frame's IPv4 and UDP checksum
+    verifies to 0xffff the way a receiver would check it (RFC 1071 / 768), and
+    payload bytes round-trip."""
+    w = synth.make_workload(5)
+    dw = DeviceWorkload(w)
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    dw.gather(ctx, rule=True)
+    assert np.array_equal(dw.req_arena.cpu().numpy(), w.req_payload)
+    dw.scatter(ctx)
+    tx = dw.tx_ring.cpu().numpy().reshape(w.tx_n_slots, w.slot_size)
+    frames = tx[w.tx_slot]
+    assert bool((be_sum_rows(frames[:, 14:34]) == 0xFFFF).all())
+    lens = np.concatenate([synth.frame_lens(int(s), w.mtu) for s in w.resp_sizes])
+    for ln in np.unique(lens):
+        sel = frames[lens == ln]
+        ulen = 8 + 16 + int(ln)
+        psd = np.concatenate([sel[:, 26:34], np.zeros((len(sel), 1), np.uint8), sel[:, 23:24],
+                              np.full((len(sel), 1), ulen >> 8, np.uint8),
+                              np.full((len(sel), 1), ulen & 0xFF, np.uint8)], axis=1)
+        seg = sel[:, 34:34 + ulen]
+        both = np.concatenate([psd, seg], axis=1)
+        assert bool((be_sum_rows(both) == 0xFFFF).all()), f"UDP checksum of {ln}-byte frames"
+    # payload of the responses, frame by frame
+    off = 0
+    for r in range(w.n_req):
+        for i, ln in enumerate(synth.frame_lens(int(w.resp_sizes[r]), w.mtu)):
+            f = int(w.resp_first[r]) + i
+            if i in (0, 57, 119):
+                assert np.array_equal(tx[w.tx_slot[f], 58:58 + ln], w.resp_payload[off:off + ln])
+            off += int(ln)
+
+
+def test_full_size_mixed_echo_round_trip(ctx):
+    """Workload 4 at full size: gather, echo in place, gather again -- the same
+    bytes and the same offsets; requests answered to their senders."""
+    w = synth.make_workload(4)
+    dw = DeviceWorkload(w)
+    before = w.ring.reshape(w.n_slots, w.slot_size)
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    dw.gather(ctx)
+    first = dw.req_arena.cpu().numpy().copy()
+    assert np.array_equal(first, w.req_payload)
+    offs = dw.req_offsets.cpu().numpy().view(np.uint64)
+    assert np.array_equal(offs[:-1], np.concatenate([[0], np.cumsum(w.req_sizes)[:-1]]).astype(np.uint64))
+    dw.scatter(ctx)
+    after = dw.ring.cpu().numpy().reshape(w.n_slots, w.slot_size)
+    used = w.frag_slot
+    assert np.array_equal(after[used, 0:6], before[used, 6:12])      # MACs swapped
+    assert np.array_equal(after[used, 26:30], before[used, 30:34])    # IPs swapped
+    assert np.array_equal(after[used, 58:], before[used, 58:])        # payload echoed
+    dw.req_arena.zero_()
+    ctx.set_cursor(0, 0)
+    dw.gather(ctx)
+    assert np.array_equal(dw.req_arena.cpu().numpy(), first)
+
+
+def test_many_batches_per_call_equal_one_batch_each(ctx):
+    """Laying several batches side by side in one call gives every batch the
+    bytes it gets alone (what the benchmark's batches-per-launch relies on)."""
+    w = synth.make_workload(2, 3)
+    one = DeviceWorkload(w)
+    many = DeviceWorkload(w, copies=5)
+    big = SgContext(0, max_reqs=64, max_frames=1 << 16)
+    big.set_cursor(0, 0)
+    big.set_cursor(1, 0)
+    one.gather(big, rule=True)
+    one.scatter(big)
+    big.set_cursor(0, 0)
+    big.set_cursor(1, 0)
+    many.gather(big, rule=True)
+    many.scatter(big)
+    a = one.req_arena.cpu().numpy()
+    b = many.req_arena.cpu().numpy().reshape(5, -1)
+    assert all(np.array_equal(a, b[k]) for k in range(5))
+    ta = one.tx_ring.cpu().numpy()
+    tb = many.tx_ring.cpu().numpy().reshape(5, -1)
+    assert all(np.array_equal(ta, tb[k]) for k in range(5))
+    big.close()
