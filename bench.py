@@ -29,6 +29,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the dominant kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this file scaled by a plain 512 MiB copy in the same runs (FETCH_SIZE x 2.000,
+# WRITE_SIZE x 1.000): 340.2 MB read + 308.3 MB written.  Known for the default call only.
+MEASURED_TRAFFIC = {(2, 32, "k_gather"): 648.5e6}
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 
@@ -46,6 +50,9 @@ def parse():
     ap.add_argument("--no-sweep", action="store_true", help="skip requests/s of the other workloads")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-remap", action="store_true", help="disable the XCD-aware launch order")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 512 MiB device copy a few times (a kernel of known "
+                         "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     ap.add_argument("--general", action="store_true",
                     help="always run the descriptor pass (do not declare the fragmenting rule)")
     return ap.parse_args()
@@ -167,6 +174,14 @@ def main() -> int:
     ctx = SgContext(0, max_reqs=max(4096, w.n_req * bpl), max_frames=max(65536, max(w.n_frags, w.n_resp_frames) * bpl))
     pool = Pool(w, bpl, a.rotate_mb, extra, rule=not a.general)
 
+    if a.calib_copy:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     sec = timed(ctx, pool, a.steps, a.warmup)
     kt = kernel_times(ctx, pool, min(a.steps, 100))
     total_bytes = pool.gather_bytes + pool.scatter_bytes
@@ -234,7 +249,9 @@ def main() -> int:
         "requests_per_sec": rps,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None if a.general else MEASURED_TRAFFIC.get((a.workload, bpl, dom)),
+                     "traffic_unit": "HBM bytes per launch (rocprofv3 --pmc, see profiles/)",
                      "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3)},
         "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in kt.items()},
         "single_batch_call": single,
