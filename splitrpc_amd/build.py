@@ -43,9 +43,10 @@ def build_host() -> str:
     src = os.path.join(HERE, "host", "host_shim.cpp")
     if not os.path.exists(src):
         return ""
-    _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+    _run([HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+          "-Wno-unused-function", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
           "-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "host"),
-          "-o", HOST_LIB, src, "-L", HERE, "-lsg_hip", "-Wl,-rpath,$ORIGIN"])
+          "-o", HOST_LIB, src, "-L", HERE, "-lsg_hip", "-lpthread", "-Wl,-rpath,$ORIGIN"])
     return HOST_LIB
 
 

@@ -1,0 +1,301 @@
+// host_shim.cpp -- C entry points over the C++ host layer, for the tests and
+// for callers that cannot include C++ headers.  Built into libsg_host.so next
+// to libsg_hip.so.  Functions whose name ends in _gpu touch the device; the
+// others are pure host logic.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#include "sg_app_rr.h"
+#include "sg_engine.h"
+#include "sg_rr.h"
+#include "sg_tables.h"
+#include "sg_wire.h"
+
+extern "C" {
+
+// Layout facts, numbered like the reference probe's table (tests compare the two).
+uint64_t sgh_layout(int what)
+{
+  switch (what) {
+    case 0: return sizeof(p2p_hbufs);
+    case 1: return sizeof(p2p_bufs);
+    case 2: return sizeof(p2p_sk_buf);
+    case 3: return sizeof(g_params);
+    case 4: return sizeof(g_params_v2);
+    case 5: return sizeof(eth_hdr);
+    case 6: return sizeof(ipv4_hdr);
+    case 7: return sizeof(udp_hdr);
+    case 8: return UDP_HEADER_LEN;
+    case 9: return MAX_BI_SIZE;
+    case 10: return offsetof(p2p_hbufs, num_items);
+    case 11: return offsetof(p2p_bufs, item_size);
+    case 12: return offsetof(p2p_bufs, num_items);
+    case 13: return offsetof(p2p_sk_buf, o_buf);
+    case 14: return offsetof(p2p_sk_buf, len);
+    case 15: return offsetof(p2p_sk_buf, num_items);
+    case 16: return offsetof(g_params, resp);
+    case 17: return offsetof(g_params_v2, outputs);
+    case 18: return offsetof(g_params_v2, input_tensor_size);
+    case 19: return offsetof(g_params_v2, output_tensor_size);
+    case 20: return offsetof(ipv4_hdr, tot_len);
+    case 21: return offsetof(ipv4_hdr, check);
+    case 22: return offsetof(ipv4_hdr, src_ip);
+    case 23: return offsetof(ipv4_hdr, dst_ip);
+    case 24: return offsetof(udp_hdr, len);
+    case 25: return offsetof(udp_hdr, check);
+    case 26: return offsetof(ipv4_hdr, protocol);
+    case 27: return sizeof(p2p_rpc_hdr);
+    case 28: return offsetof(p2p_rpc_hdr, req_token);
+    case 29: return offsetof(p2p_rpc_hdr, sock_perf_header);
+    case 30: return offsetof(p2p_rpc_hdr, seq_num);
+    default: return ~0ull;
+  }
+}
+
+// gather_skbs / scatter_skbs on a caller-supplied fragment table.
+uint64_t sgh_skbs(int scatter, const uint64_t *ptrs, const uint64_t *sizes, uint32_t n, uint64_t app_buf,
+                  uint64_t *i_out, uint64_t *o_out, uint64_t *len_out)
+{
+  p2p_bufs *b = new p2p_bufs;
+  p2p_sk_buf *s = new p2p_sk_buf;
+  for (uint32_t i = 0; i < n && i < MAX_BI_SIZE; i++) {
+    b->burst_items[i] = ptrs[i];
+    b->item_size[i] = sizes[i];
+  }
+  if (n == 0) {  // entry 0 is read even then
+    b->burst_items[0] = ptrs[0];
+    b->item_size[0] = sizes[0];
+  }
+  b->num_items = (uint16_t)n;
+  if (scatter) scatter_skbs(s, b, (uint8_t *)app_buf);
+  else gather_skbs(s, b, (uint8_t *)app_buf);
+  const uint64_t k = s->num_items;
+  for (uint64_t i = 0; i < k; i++) {
+    i_out[i] = s->i_buf[i];
+    o_out[i] = s->o_buf[i];
+    len_out[i] = s->len[i];
+  }
+  delete b;
+  delete s;
+  return k;
+}
+
+void sgh_tring_replay(uint64_t base, uint64_t capacity, const uint64_t *sizes, uint32_t n, uint64_t *out)
+{
+  P2pRpcTring t((void *)base, capacity);
+  for (uint32_t i = 0; i < n; i++) out[i] = (uint64_t)(uintptr_t)t.get_next(sizes[i]);
+}
+
+// Feed `n` ring slots, in arrival order, through P2pRpcRRPool::append_to_rr the
+// way the receive loop does (src/transport/dpdk_transport_ng.h:221-252), then
+// drain the rx-ready ring and emit the completed requests' tables.  `ring` is a
+// host image of the packet ring; payload pointers are formed on `dev_base`
+// (only their arithmetic matters here).  Returns completed requests or -1.
+int64_t sgh_pool_replay(const uint8_t *ring, uint32_t n_slots, uint32_t slot_size, uint32_t profile,
+                        uint64_t dev_base, const uint32_t *arrivals, uint32_t n, const uint32_t *len_nic,
+                        uint64_t req_size, int pool_size, uint32_t *frag_slot_out, uint32_t *frag_len_out,
+                        uint32_t *req_first_out, uint64_t *req_token_out, uint64_t *leftover_out)
+{
+  const uint32_t hl = rpc_header_len(profile);
+  P2pRpcRRPool pool(pool_size, profile);
+  p2p_rpc_conn_info *srv = initialize_src_conn_info("b8:ce:f6:cc:6a:52,192.168.25.1,50051");
+  pool.setup_and_init_rr_pool(srv, req_size);
+  release_conn_info(srv);
+  SgRingView view{sg_ring_desc{(void *)dev_base, n_slots, slot_size, profile, 0}};
+  for (uint32_t a = 0; a < n; a++) {
+    const uint32_t s = arrivals[a];
+    if (s >= n_slots) return -1;
+    uint8_t hdr[64];
+    std::memcpy(hdr, ring + (size_t)s * slot_size, sizeof hdr);
+    p2p_rpc_hdr *h = reinterpret_cast<p2p_rpc_hdr *>(hdr);
+    if (h->req_token == 0) continue;  // dropped, as the reference does (:231,247)
+    const size_t len = len_nic ? len_nic[s] : reinterpret_cast<bl58_rpc_hdr *>(hdr)->payload_len;
+    const uintptr_t slot_addr = (uintptr_t)dev_base + (uintptr_t)s * slot_size;
+    pool.append_to_rr(h, slot_addr, slot_addr, slot_addr + hl, len);
+  }
+  int64_t done = 0;
+  uint32_t f = 0;
+  req_first_out[0] = 0;
+  P2pRpcRr *rr;
+  while (pool.get_next_rx_ready_rr(&rr)) {
+    req_token_out[done] = rr->req_token;
+    for (int i = 0; i < rr->payload_bufs->num_items; i++, f++) {
+      const int64_t s = view.slot_of_payload(rr->payload_bufs->burst_items[i]);
+      if (s < 0) return -1;
+      frag_slot_out[f] = (uint32_t)s;
+      frag_len_out[f] = (uint32_t)rr->payload_bufs->item_size[i];
+    }
+    done++;
+    req_first_out[done] = f;
+    pool.reap_rr(rr);
+  }
+  if (leftover_out) *leftover_out = pool.in_flight();
+  return done;
+}
+
+// Pool exhaustion: more concurrent requests than rrs grows the pool, as the
+// reference does.  Returns the container size afterwards.
+uint64_t sgh_pool_exhaust(int pool_size, uint32_t n_tokens)
+{
+  P2pRpcRRPool pool(pool_size, SG_HDR_REF64);
+  p2p_rpc_conn_info *srv = initialize_src_conn_info("b8:ce:f6:cc:6a:52,192.168.25.1,50051");
+  pool.setup_and_init_rr_pool(srv, 1 << 20);
+  release_conn_info(srv);
+  p2p_rpc_hdr h;
+  std::memset(&h, 0, sizeof h);
+  for (uint32_t t = 1; t <= n_tokens; t++) {
+    h.req_token = t;
+    h.seq_num = 0;
+    pool.append_to_rr(&h, 0, 0, 0x1000, 16);
+  }
+  return pool.get_rr_pool_container().size();
+}
+
+// Several producers and consumers hammer one SgPtrRing; returns 1 when every
+// value came out exactly once.
+int sgh_ring_stress(uint32_t n_threads, uint32_t per_thread, uint32_t capacity)
+{
+  SgPtrRing ring(capacity);
+  std::vector<std::atomic<uint32_t>> seen(n_threads * per_thread);
+  for (auto &s : seen) s.store(0);
+  std::atomic<uint32_t> consumed{0};
+  const uint32_t total = n_threads * per_thread;
+  std::vector<std::thread> th;
+  for (uint32_t t = 0; t < n_threads; t++) {
+    th.emplace_back([&, t] {
+      for (uint32_t i = 0; i < per_thread; i++) {
+        void *p = (void *)(uintptr_t)(t * per_thread + i + 1);
+        while (ring.enqueue(p) != 0) std::this_thread::yield();
+      }
+    });
+    th.emplace_back([&] {
+      while (consumed.load() < total) {
+        void *p;
+        if (ring.dequeue(&p) == 0) {
+          seen[(uintptr_t)p - 1].fetch_add(1);
+          consumed.fetch_add(1);
+        } else {
+          std::this_thread::yield();
+        }
+      }
+    });
+  }
+  for (auto &x : th) x.join();
+  for (auto &s : seen)
+    if (s.load() != 1) return 0;
+  void *p;
+  return ring.dequeue(&p) == -ENOENT ? 1 : 0;
+}
+
+// The shunter's work for one burst (src/splitrpc_server/p2p_rpc_dpdk_server.cc:
+// 117-189) on one GPU: file the arrivals under their requests, take a slot of
+// the application ring per ready request, gather, and -- for the responses the
+// caller describes -- set up the response buffers, rewrite their headers and
+// scatter.  per_request != 0 uses the reference's one-request calls, else the
+// batched gather.  The request arena (n_done * req_size bytes) and the TX ring
+// are copied back for inspection.  Fixed-size requests (req_size) as in the
+// reference.  Returns completed requests or a negative error.
+int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots, uint32_t slot_size,
+                      uint32_t profile, const uint32_t *arrivals, uint32_t n_arr, const uint32_t *len_nic,
+                      uint64_t req_size, uint64_t resp_size, uint32_t mtu, uint32_t flags, int per_request,
+                      int want_mirror, const uint8_t *resp_host, uint8_t *tx_ring_host, uint32_t tx_n_slots,
+                      const uint32_t *tx_slot, const uint32_t *hdr_src_slot, uint8_t *req_out,
+                      int *mirrored_out)
+{
+  if (hipSetDevice(device_id) != hipSuccess) return -1;
+  const uint32_t hl = rpc_header_len(profile);
+  const size_t ring_bytes = (size_t)n_slots * slot_size, tx_bytes = (size_t)tx_n_slots * slot_size;
+  uint8_t *d_ring = nullptr, *d_tx = nullptr;
+  if (hipMalloc(&d_ring, ring_bytes) != hipSuccess || hipMalloc(&d_tx, tx_bytes) != hipSuccess) return -2;
+  (void)hipMemcpy(d_ring, ring_host, ring_bytes, hipMemcpyHostToDevice);
+  (void)hipMemcpy(d_tx, tx_ring_host, tx_bytes, hipMemcpyHostToDevice);
+
+  int64_t done = 0;
+  {
+    P2pRpcRRPool pool(-1, profile);
+    p2p_rpc_conn_info *srv = initialize_src_conn_info("b8:ce:f6:cc:6a:52,192.168.25.1,50051");
+    pool.setup_and_init_rr_pool(srv, req_size);
+    release_conn_info(srv);
+    for (uint32_t a = 0; a < n_arr; a++) {
+      const uint32_t s = arrivals[a];
+      uint8_t hdr[64];
+      std::memcpy(hdr, ring_host + (size_t)s * slot_size, sizeof hdr);
+      p2p_rpc_hdr *h = reinterpret_cast<p2p_rpc_hdr *>(hdr);
+      if (h->req_token == 0) continue;
+      const size_t len = len_nic ? len_nic[s] : reinterpret_cast<bl58_rpc_hdr *>(hdr)->payload_len;
+      const uintptr_t slot_addr = (uintptr_t)d_ring + (uintptr_t)s * slot_size;
+      pool.append_to_rr(h, slot_addr, slot_addr, slot_addr + hl, len);
+    }
+    std::vector<P2pRpcRr *> ready;
+    P2pRpcRr *rr;
+    while (pool.get_next_rx_ready_rr(&rr)) ready.push_back(rr);
+    done = (int64_t)ready.size();
+    const int n_app = (int)ready.size() + 3;  // the application ring wraps after a few slots
+    P2pRpcAppRrPool app_pool(n_app, device_id, req_size, resp_size, want_mirror != 0);
+    if (mirrored_out) *mirrored_out = app_pool.rr_mem_pool->mirrored() ? 1 : 0;
+    P2pRpcSgHipEngine engine(device_id);
+    std::vector<P2pRpcAppRr *> slots;
+    for (size_t k = 0; k < ready.size(); k++) slots.push_back(app_pool.get_next());
+
+    // ---- RX half: gather ----
+    if (per_request) {
+      for (size_t k = 0; k < ready.size(); k++) {
+        engine.gather(ready[k], slots[k]->h_stub);
+        if (engine.last_rc != SG_OK) return -10;
+        *slots[k]->h_state = RX_COMPLETE;
+      }
+    } else if (!ready.empty()) {
+      SgRingView view{sg_ring_desc{d_ring, n_slots, slot_size, profile, 0}};
+      sg_app_desc app;
+      std::memset(&app, 0, sizeof app);
+      app.arena = app_pool.rr_mem_pool->get_req_addr_range();
+      app.arena_cap = app_pool.rr_mem_pool->get_req_addr_pool_size();
+      app.arena_mirrored = app_pool.rr_mem_pool->mirrored();
+      if (engine.gather_batch(ready.data(), (uint32_t)ready.size(), view, app, nullptr, req_size,
+                              len_nic ? 0 : mtu, 0) != SG_OK)
+        return -11;
+      for (auto *s : slots) *s->h_state = RX_COMPLETE;
+    }
+    for (size_t k = 0; k < ready.size(); k++)
+      (void)hipMemcpy(req_out + k * req_size, slots[k]->h_stub->req, req_size, hipMemcpyDeviceToHost);
+
+    // ---- the model: responses land in the slots' resp buffers ----
+    for (size_t k = 0; k < ready.size(); k++) {
+      (void)hipMemcpy(slots[k]->h_stub->resp, resp_host + k * resp_size, resp_size, hipMemcpyHostToDevice);
+      *slots[k]->h_state = WORK_COMPLETE;
+    }
+
+    // ---- TX half: response buffers, headers, scatter ----
+    const uint32_t per = (uint32_t)((resp_size + mtu - 1) / mtu);
+    for (size_t k = 0; k < ready.size(); k++) {
+      P2pRpcRr *r = ready[k];
+      r->transport_mbufs->num_items = r->hdr_bufs->num_items = r->payload_bufs->num_items = 0;
+      r->payload_size = 0;
+      size_t rem = resp_size;
+      for (uint32_t i = 0; i < per; i++) {
+        const uint32_t f = (uint32_t)k * per + i;
+        uint8_t *slot = d_tx + (size_t)tx_slot[f] * slot_size;
+        // the response buffer starts out holding the request header it answers
+        (void)hipMemcpy(slot, d_ring + (size_t)hdr_src_slot[f] * slot_size, hl, hipMemcpyDeviceToDevice);
+        const size_t cur = rem <= mtu ? rem : mtu;
+        rem -= cur;
+        r->rr_append_mbuf((uintptr_t)slot, (uintptr_t)slot, (uintptr_t)(slot + hl), cur);
+      }
+      engine.swap_hdrs(r, profile, resp_size, mtu, flags & ~SG_F_UDP_CSUM_FULL);
+      if (engine.last_rc != SG_OK) return -12;
+      engine.scatter(r, slots[k]->h_stub);
+      if (engine.last_rc != SG_OK) return -13;
+      *slots[k]->h_state = FREE;
+      pool.reap_rr(r);
+    }
+    (void)hipMemcpy(tx_ring_host, d_tx, tx_bytes, hipMemcpyDeviceToHost);
+  }
+  (void)hipFree(d_ring);
+  (void)hipFree(d_tx);
+  return done;
+}
+
+}  // extern "C"

@@ -1,0 +1,244 @@
+// sg_engine.h -- the copy-engine interface of the reference
+// (src/p2p_rpc_sg_engine.h) with a HIP engine for gfx950 behind it.
+//
+//   gather_skbs / scatter_skbs   host-side run-table builders (:19-73)
+//   P2pRpcSgEngine               the abstract engine a server selects (:75-105)
+//   P2pRpcSgZcEngine             zero-copy: hands out the first payload pointer (:109-134)
+//   P2pRpcSgHipEngine            stands where P2pRpcSgGpuEngine stood (:185-308):
+//                                the same four calls, synchronous, plus batched
+//                                calls that move every ready request at once
+//
+// There is no CPU copy engine here: the reference's P2pRpcSgCpuEngine exists in
+// this repository only as the test oracle.
+#pragma once
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "sg_hip.h"
+#include "sg_rr.h"
+#include "sg_tables.h"
+
+// Fragment table (in seq order) -> run list into app_buf.  o_buf is the running
+// sum of the fragment sizes; a fragment extends the current run exactly when
+// it starts where the previous fragment ended.
+static inline void gather_skbs(p2p_sk_buf *skb, p2p_bufs *buf_ptrs, uint8_t *app_buf)
+{
+  uintptr_t app_addr = (uintptr_t)app_buf;
+  size_t run = 0;
+  uintptr_t prev_end = 0;
+  // entry 0 is written even for an empty table, as the reference does
+  const int n = buf_ptrs->num_items;
+  for (int i = 0; i < (n > 0 ? n : 1); i++) {
+    const uintptr_t p = buf_ptrs->burst_items[i];
+    const size_t sz = buf_ptrs->item_size[i];
+    if (i > 0 && p == prev_end) {
+      skb->len[run] += sz;
+    } else {
+      if (i > 0) run++;
+      skb->i_buf[run] = p;
+      skb->o_buf[run] = app_addr;
+      skb->len[run] = sz;
+    }
+    prev_end = p + sz;
+    app_addr += sz;
+  }
+  skb->num_items = run + 1;
+}
+
+// Mirror image: i_buf walks the app buffer, o_buf points at the packets.
+static inline void scatter_skbs(p2p_sk_buf *skb, p2p_bufs *buf_ptrs, uint8_t *app_buf)
+{
+  uintptr_t app_addr = (uintptr_t)app_buf;
+  size_t run = 0;
+  uintptr_t prev_end = 0;
+  const int n = buf_ptrs->num_items;
+  for (int i = 0; i < (n > 0 ? n : 1); i++) {
+    const uintptr_t p = buf_ptrs->burst_items[i];
+    const size_t sz = buf_ptrs->item_size[i];
+    if (i > 0 && p == prev_end) {
+      skb->len[run] += sz;
+    } else {
+      if (i > 0) run++;
+      skb->i_buf[run] = app_addr;
+      skb->o_buf[run] = p;
+      skb->len[run] = sz;
+    }
+    prev_end = p + sz;
+    app_addr += sz;
+  }
+  skb->num_items = run + 1;
+}
+
+class P2pRpcSgEngine {
+ public:
+  int num_instances = 1;         // parallel instances of the copy engine
+  int device_id = 0;
+  uint16_t app_queue_length = 1; // queue length of each instance
+  virtual ~P2pRpcSgEngine() {}
+
+  // API v0
+  virtual void gather(P2pRpcRr *, uint8_t *) = 0;
+  virtual void scatter(P2pRpcRr *, uint8_t *) = 0;
+  // API v1
+  virtual void gather(P2pRpcRr *, g_params *) = 0;
+  virtual void scatter(P2pRpcRr *, g_params *) = 0;
+};
+
+class P2pRpcSgZcEngine : public P2pRpcSgEngine {
+ public:
+  inline void gather(P2pRpcRr *rpc_rr, g_params *app_stub) override
+  {
+    app_stub->req = (uint8_t *)rpc_rr->payload_bufs->burst_items[0];
+    app_stub->resp = (uint8_t *)rpc_rr->payload_bufs->burst_items[0];
+    std::atomic_thread_fence(std::memory_order_release);
+  }
+  inline void scatter(P2pRpcRr *, g_params *) override {}
+  inline void gather(P2pRpcRr *, uint8_t *) override {}
+  inline void scatter(P2pRpcRr *, uint8_t *) override {}
+};
+
+// Where the packet buffers of a transport live, for the batched calls: a
+// P2pRpcRr holds payload POINTERS; the batched kernels want slot indices.
+struct SgRingView {
+  sg_ring_desc desc;
+  uintptr_t base() const { return (uintptr_t)desc.base; }
+  uint32_t hdr_len() const { return desc.hdr_profile == SG_HDR_REF64 ? 64u : 58u; }
+  // slot index of a payload pointer, or -1 if it is not a payload start of this ring
+  int64_t slot_of_payload(uintptr_t payload) const
+  {
+    const uintptr_t off = payload - base() - hdr_len();
+    if (payload < base() + hdr_len() || off % desc.slot_size) return -1;
+    const uintptr_t s = off / desc.slot_size;
+    return s < desc.n_slots ? (int64_t)s : -1;
+  }
+};
+
+class P2pRpcSgHipEngine : public P2pRpcSgEngine {
+  sg_hip_ctx *ctx;
+  // pinned staging + device copies of the CSR tables of the batched calls
+  uint32_t *h_tab = nullptr, *d_tab = nullptr;
+  size_t tab_cap = 0;
+  uint32_t max_reqs, max_frames;
+
+  void fail(const char *what, int rc) const
+  {
+    // the reference's engines report and go on (src/p2p_rpc_sg_engine.h:283-298)
+    std::printf("P2pRpcSgHipEngine: %s failed (%d): %s\n", what, rc, sg_hip_last_error(ctx));
+  }
+
+  bool tables(size_t words)
+  {
+    if (words <= tab_cap) return true;
+    if (h_tab) (void)hipHostFree(h_tab);
+    if (d_tab) (void)hipFree(d_tab);
+    tab_cap = 0;
+    if (hipHostMalloc((void **)&h_tab, words * 4, hipHostMallocDefault) != hipSuccess) return false;
+    if (hipMalloc((void **)&d_tab, words * 4) != hipSuccess) return false;
+    tab_cap = words;
+    return true;
+  }
+
+ public:
+  int last_rc = SG_OK;  // result of the most recent call (the virtuals return nothing)
+
+  explicit P2pRpcSgHipEngine(int _device_id, uint32_t _max_reqs = 4096, uint32_t _max_frames = 65536,
+                             void *stream = nullptr)
+      : max_reqs(_max_reqs), max_frames(_max_frames)
+  {
+    device_id = _device_id;
+    sg_hip_cfg cfg{sizeof(sg_hip_cfg), max_reqs, max_frames, 0, stream};
+    ctx = sg_hip_create(device_id, &cfg);
+    if (!ctx) {
+      // nothing can be moved without the device: say so and stop, as checkCudaErrors did
+      std::printf("P2pRpcSgHipEngine: cannot start on device %d: %s\n", device_id, sg_hip_last_error(nullptr));
+      std::exit(1);
+    }
+  }
+
+  ~P2pRpcSgHipEngine() override
+  {
+    if (h_tab) (void)hipHostFree(h_tab);
+    if (d_tab) (void)hipFree(d_tab);
+    sg_hip_destroy(ctx);
+  }
+
+  sg_hip_ctx *context() { return ctx; }
+
+  // ---- the reference's four calls: one request, synchronous ----
+  inline void gather(P2pRpcRr *rpc_rr, g_params *app_stub) override { gather(rpc_rr, app_stub->req); }
+  inline void scatter(P2pRpcRr *rpc_rr, g_params *app_stub) override { scatter(rpc_rr, app_stub->resp); }
+
+  inline void gather(P2pRpcRr *rpc_rr, uint8_t *payload) override
+  {
+    gather_skbs(rpc_rr->payload_sk_bufs, rpc_rr->payload_bufs, payload);
+    last_rc = sg_hip_gather(ctx, reinterpret_cast<const sg_sk_buf *>(rpc_rr->payload_sk_bufs));
+    if (last_rc != SG_OK) fail("gather", last_rc);
+  }
+
+  inline void scatter(P2pRpcRr *rpc_rr, uint8_t *payload) override
+  {
+    scatter_skbs(rpc_rr->payload_sk_bufs, rpc_rr->payload_bufs, payload);
+    last_rc = sg_hip_scatter(ctx, reinterpret_cast<const sg_sk_buf *>(rpc_rr->payload_sk_bufs));
+    if (last_rc != SG_OK) fail("scatter", last_rc);
+  }
+
+  // Header rewrite of one response on the GPU (rr_swap_hdr with device memory,
+  // src/transport/dpdk_transport_ng.h:157-159, left unimplemented there).
+  inline void swap_hdrs(P2pRpcRr *rpc_rr, uint32_t hdr_profile, size_t payload_size, uint32_t mtu, uint32_t flags)
+  {
+    last_rc = sg_hip_swap_hdrs(ctx, reinterpret_cast<const sg_hbufs *>(rpc_rr->hdr_bufs), hdr_profile,
+                               payload_size, mtu, flags);
+    if (last_rc != SG_OK) fail("swap_hdrs", last_rc);
+  }
+
+  // ---- batched: every ready request in one call ----
+  // Gathers n requests whose payload pointers lie in `ring` into `app`
+  // (consecutive bump-ring positions or tensor-major buffers), in the order
+  // given.  fixed_req_size / rule_mtu as in sg_gather_args.  Returns SG_OK or
+  // the error; `flags` may carry SG_F_ASYNC.
+  int gather_batch(P2pRpcRr *const *rrs, uint32_t n, const SgRingView &ring, const sg_app_desc &app,
+                   uint64_t *offsets_out_dev, uint64_t fixed_req_size, uint32_t rule_mtu, uint32_t flags)
+  {
+    size_t n_frags = 0;
+    for (uint32_t r = 0; r < n; r++) n_frags += rrs[r]->payload_bufs->num_items;
+    if (n > max_reqs || n_frags > max_frames) return last_rc = SG_E_INVAL;
+    // the staging tables are reused: what the previous call enqueued must have read them
+    if ((last_rc = sg_hip_sync(ctx)) != SG_OK) return last_rc;
+    const size_t words = 2 * n_frags + n + 1;
+    if (!tables(words)) return last_rc = SG_E_NOMEM;
+    uint32_t *slot = h_tab, *len = h_tab + n_frags, *first = h_tab + 2 * n_frags;
+    size_t f = 0;
+    for (uint32_t r = 0; r < n; r++) {
+      const p2p_bufs *b = rrs[r]->payload_bufs;
+      first[r] = (uint32_t)f;
+      for (int i = 0; i < b->num_items; i++, f++) {
+        const int64_t s = ring.slot_of_payload(b->burst_items[i]);
+        if (s < 0) return last_rc = SG_E_INVAL;
+        slot[f] = (uint32_t)s;
+        len[f] = (uint32_t)b->item_size[i];
+      }
+    }
+    first[n] = (uint32_t)f;
+    hipStream_t st = static_cast<hipStream_t>(sg_hip_stream(ctx));
+    if (hipMemcpyAsync(d_tab, h_tab, words * 4, hipMemcpyHostToDevice, st) != hipSuccess) return last_rc = SG_E_HIP;
+    sg_gather_args a;
+    std::memset(&a, 0, sizeof a);
+    a.ring = ring.desc;
+    a.frag_slot = d_tab;
+    a.frag_len = d_tab + n_frags;
+    a.req_first = d_tab + 2 * n_frags;
+    a.n_req = n;
+    a.n_frags = (uint32_t)n_frags;
+    a.app = app;
+    a.offsets_out = offsets_out_dev;
+    a.flags = flags | (rule_mtu && fixed_req_size ? SG_F_RULE_FRAGS : 0u);
+    a.mtu = rule_mtu;
+    a.fixed_req_size = fixed_req_size;
+    last_rc = sg_hip_gather_batch(ctx, &a);
+    if (last_rc != SG_OK) fail("gather_batch", last_rc);
+    return last_rc;
+  }
+};

@@ -1,0 +1,150 @@
+"""The C++ host layer (splitrpc_amd/host/*.h: the reference's P2pRpcRr /
+P2pRpcRRPool / P2pRpcTring / gather_skbs interfaces) through its C shim,
+against the CPU oracle and the compiled reference headers.  No GPU needed."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from splitrpc_amd import build, synth
+
+L = oracle.lib()
+REF = oracle.ref()
+
+
+@pytest.fixture(scope="module")
+def host():
+    assert os.path.exists(build.HOST_LIB), "build first: python -m splitrpc_amd.build"
+    h = C.CDLL(build.HOST_LIB)
+    h.sgh_layout.restype = C.c_uint64
+    h.sgh_skbs.restype = C.c_uint64
+    h.sgh_skbs.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint64, C.c_void_p, C.c_void_p, C.c_void_p]
+    h.sgh_tring_replay.argtypes = [C.c_uint64, C.c_uint64, C.c_void_p, C.c_uint32, C.c_void_p]
+    h.sgh_pool_replay.restype = C.c_int64
+    h.sgh_pool_replay.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint64, C.c_void_p, C.c_uint32,
+                                  C.c_void_p, C.c_uint64, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                  C.c_void_p]
+    h.sgh_pool_exhaust.restype = C.c_uint64
+    h.sgh_pool_exhaust.argtypes = [C.c_int, C.c_uint32]
+    h.sgh_ring_stress.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32]
+    return h
+
+
+def p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def test_layouts(host):
+    want = [8194, 16386, 24576, 16, 128, 14, 20, 8, 42, 1024, 8192, 8192, 16384, 8192, 16384, 24568, 8, 32, 64, 96,
+            2, 10, 12, 16, 4, 6, 9]
+    got = [host.sgh_layout(i) for i in range(27)]
+    assert got == want
+    if REF is not None:  # the numbers above are the compiled reference's
+        assert got == [REF.ref_layout(i) for i in range(27)]
+    # p2p_rpc_hdr: 64 bytes, token @42, sock_perf_header @50, seq_num @58 (src/p2p_rpc.h:10-17)
+    assert [host.sgh_layout(i) for i in range(27, 31)] == [64, 42, 50, 58]
+
+
+def test_run_table_builders_match_the_oracle(host):
+    rng = np.random.default_rng(31)
+    for trial in range(300):
+        n = int(rng.integers(0, 60)) if trial else 0
+        m = max(n, 1)
+        sizes = rng.integers(1, 3000, m).astype(np.uint64)
+        ptrs = np.zeros(m, np.uint64)
+        cur = 1 << 22
+        for i in range(m):
+            if i and rng.random() < 0.5:
+                cur = int(ptrs[i - 1] + sizes[i - 1])
+            else:
+                cur += int(rng.integers(4000, 9000))
+            ptrs[i] = cur
+        for scatter in (0, 1):
+            io, oo, lo = np.zeros(1024, np.uint64), np.zeros(1024, np.uint64), np.zeros(1024, np.uint64)
+            k = host.sgh_skbs(scatter, p(ptrs), p(sizes), n, 0x5000, p(io), p(oo), p(lo))
+            b, skb = oracle.Bufs(), oracle.SkBuf()
+            for i in range(m):
+                b.burst_items[i], b.item_size[i] = int(ptrs[i]), int(sizes[i])
+            b.num_items = n
+            (L.sgo_scatter_skbs if scatter else L.sgo_gather_skbs)(C.byref(skb), C.byref(b), 0x5000)
+            assert k == skb.num_items
+            assert io[:k].tolist() == [skb.i_buf[i] for i in range(k)]
+            assert oo[:k].tolist() == [skb.o_buf[i] for i in range(k)]
+            assert lo[:k].tolist() == [skb.len[i] for i in range(k)]
+
+
+def test_tring(host):
+    rng = np.random.default_rng(32)
+    sizes = rng.integers(1, 5000, 300).astype(np.uint64)
+    out = np.zeros(300, np.uint64)
+    host.sgh_tring_replay(1 << 32, 77777, p(sizes), 300, p(out))
+    t = oracle.Tring()
+    L.sgo_tring_init(C.byref(t), 1 << 32, 77777)
+    assert out.tolist() == [L.sgo_tring_get_next(C.byref(t), int(s)) for s in sizes]
+    if REF is not None:
+        ref_out = np.zeros(300, np.uint64)
+        REF.ref_tring_replay(1 << 32, 77777, p(sizes), 300, p(ref_out))
+        assert np.array_equal(out, ref_out)
+
+
+def _pool_replay(host, w, arrivals, len_nic=None, req_size=0, pool_size=-1):
+    n = len(arrivals)
+    fs, fl = np.zeros(n + 1, np.uint32), np.zeros(n + 1, np.uint32)
+    rf, tok = np.zeros(n + 2, np.uint32), np.zeros(n + 1, np.uint64)
+    left = np.zeros(1, np.uint64)
+    arr = np.ascontiguousarray(arrivals, dtype=np.uint32)
+    done = host.sgh_pool_replay(p(w.ring), w.n_slots, w.slot_size, w.profile, 0x7F0000000000, p(arr), n,
+                                p(len_nic), req_size, pool_size, p(fs), p(fl), p(rf), p(tok), p(left))
+    assert done >= 0
+    nf = int(rf[done])
+    return fs[:nf], fl[:nf], rf[:done + 1], tok[:done], int(left[0])
+
+
+@pytest.mark.parametrize("cfg,n", [(1, 10), (2, 2), (3, 50), (4, 80), (5, 2)])
+def test_pool_reassembly_matches_the_oracle(host, cfg, n):
+    w = synth.make_workload(cfg, n)
+    got = _pool_replay(host, w, w.arrivals)
+    want = oracle.reassemble(w)
+    for g, e in zip(got[:4], want):
+        assert np.array_equal(g, e)
+    assert got[4] == 0
+    # and with the arrivals shuffled
+    arr = np.random.default_rng(cfg).permutation(w.arrivals)
+    got = _pool_replay(host, w, arr)
+    want = oracle.reassemble(w, arrivals=arr)
+    for g, e in zip(got[:4], want):
+        assert np.array_equal(g, e)
+
+
+def test_pool_reassembly_ref64_by_request_size(host):
+    """The reference's own readiness rule: payload_size == max_payload_size."""
+    w = synth.make_workload(2, 3, profile=synth.HDR_REF64)
+    len_nic = np.zeros(w.n_slots, np.uint32)
+    len_nic[w.frag_slot] = w.frag_len
+    size = int(w.req_sizes[0])
+    got = _pool_replay(host, w, w.arrivals, len_nic=len_nic, req_size=size)
+    want = oracle.reassemble(w, req_size=size, frag_len_nic=len_nic)
+    for g, e in zip(got[:4], want):
+        assert np.array_equal(g, e)
+    assert np.array_equal(got[0], w.frag_slot)
+
+
+def test_lost_fragment_parks_the_request(host):
+    """A lost fragment leaves its request in the cache for good
+    (src/p2p_rpc_rr_pool_ng.h:57-64): nothing is handed over for it."""
+    w = synth.make_workload(1, 6)
+    arr = np.delete(w.arrivals, 4)
+    fs, fl, rf, tok, left = _pool_replay(host, w, arr)
+    assert len(tok) == 5 and left == 1
+
+
+def test_pool_grows_when_exhausted(host):
+    assert host.sgh_pool_exhaust(4, 3) == 3      # pool_size - 1 rrs, all taken
+    assert host.sgh_pool_exhaust(4, 10) == 10    # seven more were allocated
+
+
+def test_pointer_ring_multi_producer_multi_consumer(host):
+    assert host.sgh_ring_stress(4, 20000, 64) == 1
+    assert host.sgh_ring_stress(2, 1000, 2) == 1
