@@ -239,8 +239,11 @@ __global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
 
 // Scan of the request totals through the bump ring (one workgroup):
 //   ret = base + off; off = (off + size) % capacity   (src/p2p_rpc_tring.h:27-33)
+// Each thread owns kScanPerThread consecutive requests (read and written as
+// 16-byte pairs), so one pass of the workgroup covers 16384 requests.
 constexpr int kScanBlock = 1024;
-constexpr int kScanPerThread = 4;
+constexpr int kScanPerThread = 16;
+typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
 __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
@@ -249,21 +252,32 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
     const uint32_t q0 = base + threadIdx.x * kScanPerThread;
     uint64_t sz[kScanPerThread];
     uint64_t mine = 0;
+    if (q0 + kScanPerThread <= a.n_req) {
 #pragma unroll
-    for (int k = 0; k < kScanPerThread; k++) {
-      sz[k] = (q0 + k < a.n_req) ? a.req_size[q0 + k] : 0;
-      mine += sz[k];
+      for (int k = 0; k < kScanPerThread; k += 2) {
+        const u64x2 v = *reinterpret_cast<const u64x2 *>(a.req_size + q0 + k);  // q0 is a multiple of 16
+        sz[k] = v[0];
+        sz[k + 1] = v[1];
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kScanPerThread; k++) sz[k] = (q0 + k < a.n_req) ? a.req_size[q0 + k] : 0;
     }
+#pragma unroll
+    for (int k = 0; k < kScanPerThread; k++) mine += sz[k];
     uint64_t tot;
     uint64_t ex = block_exclusive_scan<kScanBlock>(mine, wave_tot, &tot);
+    // offsets stay below 2 * capacity between reductions: run < cap and every
+    // prefix of one pass is reduced as it grows
+    uint64_t off = (run + ex) % a.cap;
 #pragma unroll
     for (int k = 0; k < kScanPerThread; k++) {
       if (q0 + k < a.n_req) {
-        const uint64_t off = (run + ex) % a.cap;
         a.req_off[q0 + k] = off;
         if (a.offsets_out) a.offsets_out[q0 + k] = off;
       }
-      ex += sz[k];
+      off += sz[k];  // sz <= cap (checked by the descriptor pass), so one subtraction reduces
+      if (off >= a.cap) off = a.cap ? off % a.cap : 0;
     }
     run = (run + tot) % a.cap;
   }
@@ -321,6 +335,7 @@ struct GatherArgs {
   uint32_t hl;
   uint32_t n_items;
   uint32_t remap;
+  uint32_t pieces;  // wavefronts per fragment
   uint32_t *status;
   AppDev app;
 };
@@ -448,77 +463,54 @@ __device__ __forceinline__ bool plain_target(const AppDev &app, uint64_t req_off
   return false;
 }
 
-// A gather wavefront takes kGatherPerWave consecutive fragment runs and has the
-// loads of all of them in flight before it stores the first.  Measured on
-// 1400-byte fragments, one run per wavefront is fastest (two cost 2 %, three
-// 13 %): the wavefront count, not the bytes in flight per wavefront, is what
-// covers the HBM latency here.
-#ifndef SG_GATHER_PER_WAVE
-#define SG_GATHER_PER_WAVE 1
-#endif
-constexpr uint32_t kGatherPerWave = SG_GATHER_PER_WAVE;
-
-struct GatherItem {
-  bool live;    // there is something to move
-  bool plain;   // one contiguous destination piece: begin/end path
-  uint8_t *pkt; // payload in the slot
-  uint8_t *to;
-  uint32_t len, off, r;
-  uint64_t ro;
-};
-
-// Gather from descriptors written by the descriptor pass.
+// Gather from descriptors written by the descriptor pass.  One wavefront per
+// fragment piece: a fragment longer than kPieceChunks chunks is spread over
+// `pieces` consecutive wavefronts.  (Several fragments per wavefront were
+// measured too: two cost 2 %, three 13 % on 1400-byte fragments -- the number
+// of wavefronts in flight is what covers the HBM latency.)
+template <bool LONG>
 __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
 {
   const u32x4 *desc = a.desc;
   const uint64_t *req_off = a.req_off;
   const uint8_t *ring = a.ring;
   const uint32_t slot_size = a.slot_size, hl = a.hl, n_items = a.n_items, remap = a.remap;
+  const uint32_t pieces = a.pieces;
   const uint32_t *status = a.status;
   SG_PIN(desc); SG_PIN(req_off); SG_PIN(ring); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_items);
-  SG_PIN(remap); SG_PIN(status);
-  const uint32_t item0 = item_of_wave(remap != 0) * kGatherPerWave;
-  if (item0 >= n_items) return;
+  SG_PIN(remap); SG_PIN(status); SG_PIN(pieces);
+  const uint32_t w = item_of_wave(remap != 0);
+  const uint32_t item = LONG ? w / pieces : w;
+  const uint32_t piece = LONG ? w - item * pieces : 0;
+  if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   if (sload(status)) return;  // the descriptor pass refused the batch: move nothing
-
-  GatherItem it[kGatherPerWave];
-  RunState rs[kGatherPerWave];
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++) {
-    const bool in = item0 + k < n_items;
-    const u32x4 d = sload(desc + (in ? item0 + k : item0));
-    it[k].live = in && d[1] != 0 && d[3] != kInvalidReq;
-    it[k].len = d[1];
-    it[k].off = d[2];
-    it[k].r = d[3];
-    it[k].ro = 0;
-    it[k].plain = false;
-    it[k].pkt = const_cast<uint8_t *>(ring) + (size_t)d[0] * slot_size + hl;
-    if (it[k].live) {
-      if (a.app.n_tensors == 0) it[k].ro = sload(req_off + d[3]);
-      it[k].plain = plain_target(a.app, it[k].ro, d[3], d[2], d[1], &it[k].to);
+  const u32x4 d = sload(desc + item);
+  if (d[1] == 0 || d[3] == kInvalidReq) return;
+  const uint64_t ro = a.app.n_tensors == 0 ? sload(req_off + d[3]) : 0;
+  uint8_t *pkt = const_cast<uint8_t *>(ring) + (size_t)d[0] * slot_size + hl;
+  uint8_t *to;
+  if (plain_target(a.app, ro, d[3], d[2], d[1], &to)) {
+    if (LONG) {
+      PieceState ps;
+      piece_begin(ps, pkt, to, d[1], lane, piece * kPieceChunks, kPieceChunks);
+      piece_end<false>(ps, lane);
+    } else {
+      copy_run<false>(pkt, to, d[1], lane);
     }
-  }
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++)
-    if (it[k].live && it[k].plain) run_begin(rs[k], it[k].pkt, it[k].to, it[k].len, lane);
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++) {
-    if (!it[k].live) continue;
-    if (it[k].plain) run_end<false>(rs[k], lane);
-    else move_run<true, false>(a.app, it[k].ro, it[k].r, it[k].off, it[k].pkt, it[k].len, lane);
+  } else if (piece == 0) {
+    move_run<true, false>(a.app, ro, d[3], d[2], pkt, d[1], lane);
   }
 }
 
 // Gather without a descriptor pass: all requests have `size` bytes cut by the
-// fragmenting rule, so a wavefront derives its descriptors from its item
-// numbers (item f belongs to request f / per_req, is its fragment f % per_req,
+// fragmenting rule, so a wavefront derives its descriptor from its item
+// number (item f belongs to request f / per_req, is its fragment f % per_req,
 // carries min(remaining, mtu) bytes and starts i * mtu bytes into the request;
-// request r starts at cursor + r * size in the bump ring) and holds every
+// request r starts at cursor + r * size in the bump ring) and holds the
 // fragment's real length against the rule.
 struct GatherRuleArgs {
-  // hot: what a wavefront needs before its first payload load (64 bytes)
+  // hot: what a wavefront needs before its first payload load
   const uint8_t *ring;
   const uint32_t *frag_slot;
   uint8_t *dst;               // arena (packed) or the tensor (one tensor-major buffer)
@@ -529,11 +521,12 @@ struct GatherRuleArgs {
   uint32_t per_req;
   uint32_t mtu;
   uint32_t slot_size;
-  // warm
   uint32_t hl;
   uint32_t n_slots;
-  uint32_t n_req;
+  uint32_t pieces;            // wavefronts per fragment
   uint32_t opts;  // kOptRemap | kOptMirrored | kOptSingleWrap | kOptMultiTensor
+  // warm
+  uint32_t n_req;
   const uint32_t *frag_len;
   const uint32_t *first;
   uint64_t *offsets_out;
@@ -543,17 +536,7 @@ struct GatherRuleArgs {
 };
 constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptSingleWrap = 4u, kOptMultiTensor = 8u;
 
-// Does the payload_len of a BL58 header (u32 at byte 54) equal `len`?  Read as
-// the two aligned dwords around it through the scalar cache and compared half
-// by half (a combined value would be fetched with one misaligned vector load).
-// For kernels that only read the ring.
-__device__ __forceinline__ bool bl58_len_is(const uint8_t *slot, uint32_t len)
-{
-  const uint32_t w0 = sload(reinterpret_cast<const uint32_t *>(slot + 52));
-  const uint32_t w1 = sload(reinterpret_cast<const uint32_t *>(slot + 56));
-  return ((w0 >> 16) == (len & 0xffffu)) & ((w1 & 0xffffu) == (len >> 16));
-}
-
+template <bool LONG>
 __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
 {
   const uint8_t *ring = a.ring;
@@ -562,94 +545,89 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint64_t *cursor_in = a.cursor_in;
   const uint64_t size = a.size, cap = a.cap;
   const uint32_t n_items = a.n_items, per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
-  const uint32_t hl = a.hl, n_slots = a.n_slots, opts = a.opts;
+  const uint32_t hl = a.hl, n_slots = a.n_slots, pieces = a.pieces, opts = a.opts;
   SG_PIN(ring); SG_PIN(frag_slot); SG_PIN(dst); SG_PIN(cursor_in); SG_PIN(size); SG_PIN(cap);
   SG_PIN(n_items); SG_PIN(per_req); SG_PIN(mtu); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_slots);
-  SG_PIN(opts);
+  SG_PIN(pieces); SG_PIN(opts);
 
-  const uint32_t item0 = item_of_wave((opts & kOptRemap) != 0) * kGatherPerWave;
-  if (item0 >= n_items) return;
+  const uint32_t w = item_of_wave((opts & kOptRemap) != 0);
+  const uint32_t item = LONG ? w / pieces : w;
+  const uint32_t piece = LONG ? w - item * pieces : 0;
+  if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  uint32_t slot[kGatherPerWave];
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++)
-    slot[k] = sload(frag_slot + (item0 + k < n_items ? item0 + k : item0));
+  const uint32_t slot = sload(frag_slot + item);
   uint64_t c0 = cap ? sload(cursor_in) : 0;
-  if (c0 >= cap && cap) c0 %= cap;  // only after a set_cursor beyond the capacity
+  const uint32_t r = item / per_req;
+  const uint32_t i = item - r * per_req;
+  const uint32_t off = i * mtu;
+  const uint64_t rem = size - off;
+  const uint32_t len = (uint32_t)(rem <= mtu ? rem : mtu);
+  if (slot >= n_slots) {
+    if (lane == 0 && piece == 0) atomicOr(a.status, kStBadSlot);
+    return;
+  }
+  uint8_t *pkt = const_cast<uint8_t *>(ring) + (size_t)slot * slot_size;
 
-  GatherItem it[kGatherPerWave];
-  RunState rs[kGatherPerWave];
-  uint32_t idx[kGatherPerWave];
-  uint32_t bad = 0;
-  const uint32_t r0 = item0 / per_req;
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++) {
-    const uint32_t item = item0 + k;
-    // items of one wavefront are consecutive: at most one request boundary apart
-    uint32_t r = r0, i = item - r0 * per_req;
-    if (i >= per_req) { r += 1; i -= per_req; }
-    idx[k] = i;
-    it[k].live = item < n_items;
-    it[k].r = r;
-    it[k].off = i * mtu;
-    const uint64_t rem = size - it[k].off;
-    it[k].len = (uint32_t)(rem <= mtu ? rem : mtu);
-    if (it[k].live && slot[k] >= n_slots) {
-      bad |= kStBadSlot;
-      it[k].live = false;
-    }
-    it[k].pkt = const_cast<uint8_t *>(ring) + (size_t)slot[k] * slot_size;
-    it[k].ro = 0;
-    it[k].plain = !(opts & kOptMultiTensor);
-    it[k].to = nullptr;
-    if (!it[k].live) continue;
-    if (cap) {
-      // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
-      uint64_t ro = c0 + (uint64_t)r * size;
-      if (opts & kOptSingleWrap) ro = ro >= cap ? ro - cap : ro;  // n_req * size <= capacity
-      else ro %= cap;
-      it[k].ro = ro;
-      if (lane == 0) {
-        if (i == 0 && a.offsets_out) a.offsets_out[r] = ro;
-        if (item == n_items - 1) {
-          uint64_t end = ro + size;  // size <= capacity
-          end = end >= cap ? end - cap : end;
-          *a.cursor_out = end;
-          if (a.offsets_out) a.offsets_out[a.n_req] = end;
-        }
+  uint64_t ro = 0;
+  bool plain = !(opts & kOptMultiTensor);
+  uint8_t *to = nullptr;
+  if (cap) {
+    // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
+    if (c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
+    ro = c0 + (uint64_t)r * size;
+    if (opts & kOptSingleWrap) ro = ro >= cap ? ro - cap : ro;  // n_req * size <= capacity
+    else ro %= cap;
+    if (lane == 0 && piece == 0) {
+      if (i == 0 && a.offsets_out) a.offsets_out[r] = ro;
+      if (item == n_items - 1) {
+        uint64_t end = ro + size;  // size <= capacity
+        end = end >= cap ? end - cap : end;
+        *a.cursor_out = end;
+        if (a.offsets_out) a.offsets_out[a.n_req] = end;
       }
-      if (it[k].plain) {
-        uint64_t o = ro + it[k].off;  // < 2 * capacity
-        if (!(opts & kOptMirrored)) {
-          if (o >= cap) o -= cap;
-          else if (o + it[k].len > cap) it[k].plain = false;  // crosses the end of an arena mapped once
-        }
-        it[k].to = dst + o;
-      }
-    } else if (it[k].plain) {
-      it[k].to = dst + (uint64_t)r * size + it[k].off;
     }
+    uint64_t o = ro + off;  // < 2 * capacity
+    if (!(opts & kOptMirrored)) {
+      if (o >= cap) o -= cap;
+      else if (o + len > cap) plain = false;  // crosses the end of an arena mapped once
+    }
+    to = dst + o;
+  } else {
+    to = dst + (uint64_t)r * size + off;
+  }
+  // The header words that hold the fragment's real length are fetched together
+  // with the payload, so that checking them does not lengthen the wavefront's
+  // life by another memory round trip.
+  const bool check_hdr = piece == 0 && a.frag_len == nullptr;
+  uint32_t w0 = 0, w1 = 0;
+  if (check_hdr) {
+    w0 = sload(reinterpret_cast<const uint32_t *>(pkt + 52));
+    w1 = sload(reinterpret_cast<const uint32_t *>(pkt + 56));
   }
   // copying the ruled length stays inside the slot whatever the header says
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++)
-    if (it[k].live && it[k].plain) run_begin(rs[k], it[k].pkt + hl, it[k].to, it[k].len, lane);
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++) {
-    if (!it[k].live) continue;
-    if (it[k].plain) run_end<false>(rs[k], lane);
-    else move_run<true, false>(a.app, it[k].ro, it[k].r, it[k].off, it[k].pkt + hl, it[k].len, lane);
+  RunState rs;
+  PieceState ps;
+  if (plain) {
+    if (LONG) piece_begin(ps, pkt + hl, to, len, lane, piece * kPieceChunks, kPieceChunks);
+    else run_begin(rs, pkt + hl, to, len, lane);
   }
-#pragma unroll
-  for (uint32_t k = 0; k < kGatherPerWave; k++) {
-    if (!it[k].live) continue;
-    const uint32_t item = item0 + k;
-    const bool as_ruled = a.frag_len ? sload(a.frag_len + item) == it[k].len
-                                     : bl58_len_is(it[k].pkt, it[k].len);
+  SG_PIN(w0);
+  SG_PIN(w1);
+  if (plain) {
+    if (LONG) piece_end<false>(ps, lane);
+    else run_end<false>(rs, lane);
+  } else if (piece == 0) {
+    move_run<true, false>(a.app, ro, r, off, pkt + hl, len, lane);
+  }
+  if (piece == 0) {
+    uint32_t bad = 0;
+    // payload_len is the u32 at byte 54: the upper half of w0 and the lower half of w1
+    const bool as_ruled = check_hdr ? (((w0 >> 16) == (len & 0xffffu)) & ((w1 & 0xffffu) == (len >> 16)))
+                                    : sload(a.frag_len + item) == len;
     if (!as_ruled) bad |= kStNotRule;
-    if (idx[k] == 0 && sload(a.first + it[k].r) != item) bad |= kStBadTable;
+    if (i == 0 && sload(a.first + r) != item) bad |= kStBadTable;
+    if (bad && lane == 0) atomicOr(a.status, bad);
   }
-  if (bad && lane == 0) atomicOr(a.status, bad);
 }
 
 struct ScatterArgs {
@@ -667,15 +645,22 @@ struct ScatterArgs {
   uint32_t flags;
   uint32_t n_items;
   uint32_t remap;
+  uint32_t pieces;  // wavefronts per frame (1 when the payload is summed: one wavefront owns the sum)
   uint32_t *status;
   RuleArgs rule;
   AppDev app;
 };
 
-template <bool FULL_CSUM, bool FUSED>
+// LONG: frames longer than kPieceChunks chunks are spread over a.pieces
+// wavefronts (never when the payload is summed: one wavefront owns the sum).
+template <bool FULL_CSUM, bool FUSED, bool LONG>
 __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
-  const uint32_t item = item_of_wave(a.remap != 0);
+  static_assert(!(FULL_CSUM && LONG), "a summed frame belongs to one wavefront");
+  const uint32_t w = item_of_wave(a.remap != 0);
+  const uint32_t pieces = LONG ? a.pieces : 1u;
+  const uint32_t item = LONG ? w / pieces : w;
+  const uint32_t piece = LONG ? w - item * pieces : 0;
   if (item >= a.n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   u32x4 d;
@@ -691,21 +676,32 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     ro = a.app.n_tensors == 0 ? a.req_off[r] : 0;
   } else {
     uint32_t slot_i, len, off, i;
-    const uint32_t bad = rule_desc(a.rule, a.app, item, a.n_items, lane, &slot_i, &len, &off, &r, &i, &ro);
+    const uint32_t bad = rule_desc(a.rule, a.app, item, a.n_items, piece == 0 ? lane : 1u, &slot_i, &len,
+                                   &off, &r, &i, &ro);
     if (bad) {
-      if (lane == 0) atomicOr(a.status, bad);
+      if (lane == 0 && piece == 0) atomicOr(a.status, bad);
       return;
     }
     d = (u32x4){slot_i, len, off, r};
     f0 = item - i;
     nf = a.rule.per_req;
   }
+  uint8_t *slot = a.tx + (size_t)d[0] * a.tx_slot_size;
+  if (LONG && piece != 0) {
+    // a later piece of a long frame: payload only
+    uint8_t *from;
+    if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
+      PieceState ps;
+      piece_begin(ps, from, slot + a.hl, d[1], lane, piece * kPieceChunks, kPieceChunks);
+      piece_end<false>(ps, lane);
+    }
+    return;
+  }
   uint32_t hs = a.hdr_src_slot[item];
   if (hs >= a.rx_n_slots) {
     if (lane == 0) atomicOr(a.status, kStBadSlot);
     return;
   }
-  uint8_t *slot = a.tx + (size_t)d[0] * a.tx_slot_size;
 
   // read the request header before anything of this slot is overwritten
   // (the TX slot may be the very slot the header comes from)
@@ -715,7 +711,14 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   if (!FULL_CSUM) hb = hdr_rewrite(hin, lane, hf, 0);
 
   uint32_t acc = 0;
-  if (d[1]) acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
+  uint8_t *from;
+  if (LONG && d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
+    PieceState ps;
+    piece_begin(ps, from, slot + a.hl, d[1], lane, 0, kPieceChunks);
+    piece_end<false>(ps, lane);
+  } else if (d[1]) {
+    acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
+  }
   if (FULL_CSUM) {
     // the payload copy wrote past the header only, so in place the request
     // header is still intact here
@@ -872,10 +875,9 @@ int check_app(sg_hip_ctx *c, const sg_app_desc &a, AppDev *out, uint64_t *max_re
 
 // Launch geometry for one wavefront per item; with the XCD-aware order the
 // grid is padded to whole rounds of kXcds * kXcdRun workgroups.
-void geometry(uint32_t n_items, uint32_t per_wave, bool want_remap, uint32_t *grid, uint32_t *remap)
+void geometry(uint64_t n_waves, bool want_remap, uint32_t *grid, uint32_t *remap)
 {
-  const uint32_t per_group = kWavesPerBlock * per_wave;
-  const uint32_t groups = (n_items + per_group - 1) / per_group;
+  const uint32_t groups = (uint32_t)((n_waves + kWavesPerBlock - 1) / kWavesPerBlock);
   const uint32_t round = kXcds * kXcdRun;
   if (want_remap && groups >= 2 * round) {
     *grid = (groups + round - 1) / round * round;
@@ -1221,14 +1223,16 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
     ga.status = c->status;
     ga.app = app;
+    ga.pieces = pieces_for(a->mtu);
     uint32_t grid, remap;
-    geometry(a->n_frags, kGatherPerWave, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
+    geometry((uint64_t)a->n_frags * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
               ((app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_req_size <= app.cap) ? kOptSingleWrap : 0u) |
               (app.n_tensors > 1 ? kOptMultiTensor : 0u);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    k_gather_rule<<<grid, kBlock, 0, c->stream>>>(ga);
+    if (ga.pieces > 1) k_gather_rule<true><<<grid, kBlock, 0, c->stream>>>(ga);
+    else k_gather_rule<false><<<grid, kBlock, 0, c->stream>>>(ga);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
     return finish(c, a->flags);
@@ -1273,11 +1277,13 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.n_items = a->n_frags;
     ga.status = c->status;
     ga.app = app;
+    ga.pieces = pieces_for(p.slot_size - p.hl);
     uint32_t grid;
-    geometry(a->n_frags, kGatherPerWave, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
+    geometry((uint64_t)a->n_frags * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    k_gather<<<grid, kBlock, 0, c->stream>>>(ga);
+    if (ga.pieces > 1) k_gather<true><<<grid, kBlock, 0, c->stream>>>(ga);
+    else k_gather<false><<<grid, kBlock, 0, c->stream>>>(ga);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }
@@ -1340,12 +1346,14 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.rule.cursor_out = c->cursors + 2 + (c->parity[1] ^ 1u);
     if (app.n_tensors == 0) c->parity[1] ^= 1u;
     sa.rule.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
+    sa.pieces = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : pieces_for(a->mtu);
     uint32_t grid;
-    geometry(a->n_frames, 1, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry((uint64_t)a->n_frames * sa.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, true><<<grid, kBlock, 0, c->stream>>>(sa);
-    else k_scatter<false, true><<<grid, kBlock, 0, c->stream>>>(sa);
+    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, true, false><<<grid, kBlock, 0, c->stream>>>(sa);
+    else if (sa.pieces > 1) k_scatter<false, true, true><<<grid, kBlock, 0, c->stream>>>(sa);
+    else k_scatter<false, true, false><<<grid, kBlock, 0, c->stream>>>(sa);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
     return finish(c, a->flags);
@@ -1397,12 +1405,14 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.n_items = a->n_frames;
     sa.status = c->status;
     sa.app = app;
+    sa.pieces = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : pieces_for(a->mtu);
     uint32_t grid;
-    geometry(a->n_frames, 1, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry((uint64_t)a->n_frames * sa.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, false><<<grid, kBlock, 0, c->stream>>>(sa);
-    else k_scatter<false, false><<<grid, kBlock, 0, c->stream>>>(sa);
+    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, false, false><<<grid, kBlock, 0, c->stream>>>(sa);
+    else if (sa.pieces > 1) k_scatter<false, false, true><<<grid, kBlock, 0, c->stream>>>(sa);
+    else k_scatter<false, false, false><<<grid, kBlock, 0, c->stream>>>(sa);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }
