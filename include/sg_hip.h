@@ -171,6 +171,31 @@ typedef struct sg_scatter_args {
   uint64_t *offsets_out; /* device, n_req + 1, or NULL */
 } sg_scatter_args;
 
+/* One burst of arrivals to sort into requests on the device.  Replaces the
+ * per-packet work of the receive thread: get_rr / rr_emplace_mbuf /
+ * is_rr_ready / mark_rx_ready_rr (src/p2p_rpc_rr_pool_ng.h:97-119,149-155;
+ * src/transport/dpdk_transport_ng.h:221-252).  A request is complete when
+ * num_frags fragments are in (BL58) or when its payload bytes reach req_size
+ * (REF64, src/p2p_rpc_rr_ng.h:107-110).  Completed requests come out in
+ * completion order -- the order in which their last fragment arrived, which
+ * is the order of the reference's rx-ready ring -- as the CSR tables
+ * sg_hip_gather_batch takes.  Packets with token 0 are dropped (:231);
+ * arrivals of requests that do not complete within this burst are left out
+ * and counted.  As in the reference, duplicate fragments are not detected. */
+typedef struct sg_reassemble_args {
+  sg_ring_desc ring;
+  const uint32_t *arrivals; /* device, n_arrivals: ring slots in arrival order */
+  const uint32_t *len_nic;  /* device, n_slots: payload bytes of each slot as the NIC reports
+                               them (required for REF64; NULL for BL58: read from the header) */
+  uint32_t n_arrivals;
+  uint32_t reserved;
+  uint64_t req_size;        /* REF64: the server-wide request size */
+  uint32_t *frag_slot;      /* device out, n_arrivals */
+  uint32_t *frag_len;       /* device out, n_arrivals */
+  uint32_t *req_first;      /* device out, max_reqs + 1 of the context */
+  uint64_t *req_token;      /* device out, max_reqs, or NULL */
+} sg_reassemble_args;
+
 /* ---- lifetime -------------------------------------------------------------
  * Replaces P2pRpcSgGpuEngine's constructor/destructor work
  * (src/p2p_rpc_sg_engine.h:261-307: stubs, doorbells, streams, persistent
@@ -213,6 +238,13 @@ int sg_hip_swap_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, uint32_t hdr_profile
 int sg_hip_gather_batch(sg_hip_ctx *ctx, const sg_gather_args *args);
 int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
 
+/* Sorts a burst of arrivals into requests (see sg_reassemble_args).
+ * Synchronous: the counts come back to the host because the caller sizes the
+ * gather call with them.  n_left: arrivals that belong to no completed
+ * request. */
+int sg_hip_reassemble(sg_hip_ctx *ctx, const sg_reassemble_args *args, uint32_t *n_req_out,
+                      uint32_t *n_frags_out, uint32_t *n_left_out);
+
 /* Device-resident bump-ring cursors (P2pRpcTring::prev_offset,
  * src/p2p_rpc_tring.h:14-16), one for the request arena (which = 0) and one
  * for the response arena (which = 1).  Both calls synchronize. */
@@ -224,7 +256,7 @@ int sg_hip_get_cursor(sg_hip_ctx *ctx, int which, uint64_t *value);
  * context's stream (the PROFILE_MODE GDelay/SDelay vectors of the reference,
  * src/p2p_rpc_sg_engine.h:83-92, at kernel granularity).  which: 0 descriptor
  * build, 1 gather copy, 2 scatter copy + header rewrite, 3 per-request run
- * copy, 4 header-only rewrite.  sg_hip_kernel_time synchronizes, returns the
+ * copy, 4 header-only rewrite, 5 reassembly (its six small kernels together).  sg_hip_kernel_time synchronizes, returns the
  * accumulated milliseconds and launch count since profiling was switched on,
  * and leaves the accumulators running. */
 int sg_hip_set_profiling(sg_hip_ctx *ctx, int on);

@@ -37,7 +37,7 @@ MAX_TENSORS = 4
 SYMBOLS = [
     "sg_hip_create", "sg_hip_destroy", "sg_hip_last_error", "sg_hip_abi_version", "sg_hip_stream",
     "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_gather_batch",
-    "sg_hip_scatter_batch", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
+    "sg_hip_scatter_batch", "sg_hip_reassemble", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
     "sg_hip_kernel_time",
 ]
 
@@ -84,6 +84,13 @@ class ScatterArgs(C.Structure):
                 ("offsets_out", C.c_void_p)]
 
 
+class ReassembleArgs(C.Structure):
+    _fields_ = [("ring", RingDesc), ("arrivals", C.c_void_p), ("len_nic", C.c_void_p),
+                ("n_arrivals", C.c_uint32), ("reserved", C.c_uint32), ("req_size", C.c_uint64),
+                ("frag_slot", C.c_void_p), ("frag_len", C.c_void_p), ("req_first", C.c_void_p),
+                ("req_token", C.c_void_p)]
+
+
 _lib = None
 
 
@@ -116,6 +123,8 @@ def load() -> C.CDLL:
     lib.sg_hip_swap_hdrs.argtypes = [P, C.POINTER(HBufs), C.c_uint32, C.c_uint64, C.c_uint32, C.c_uint32]
     lib.sg_hip_gather_batch.argtypes = [P, C.POINTER(GatherArgs)]
     lib.sg_hip_scatter_batch.argtypes = [P, C.POINTER(ScatterArgs)]
+    lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32),
+                                      C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
     lib.sg_hip_set_cursor.argtypes = [P, C.c_int, C.c_uint64]
     lib.sg_hip_get_cursor.argtypes = [P, C.c_int, C.POINTER(C.c_uint64)]
     lib.sg_hip_set_profiling.argtypes = [P, C.c_int]

@@ -763,6 +763,212 @@ __global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, 
   if (lane < hl) h[lane] = (uint8_t)b;
 }
 
+// ---------------------------------------------------------------------------
+// request reassembly on the device
+// ---------------------------------------------------------------------------
+// What the receive thread of the reference does per packet -- look the request
+// up by token (get_rr), file the fragment at its sequence number
+// (rr_emplace_mbuf), hand the request over once complete (is_rr_ready,
+// mark_rx_ready_rr) -- done for a whole burst of arrivals at once:
+//   k_ra_insert  one thread per arrival: open-addressing insert of the token
+//                into a hash table (atomicCAS on the key, linear probing over a
+//                table at least twice the arrivals: every probe makes progress,
+//                nothing waits), fragment count / byte total / last arrival
+//                position per request by atomics
+//   k_ra_flag    the thread of a complete request's LAST arrival flags that
+//                position with the request's fragment count; workgroup-local
+//                scan of the packed (requests, fragments) flags
+//   k_ra_scan    one workgroup scans the workgroup totals
+//   k_ra_assign  batch index = number of requests completed before (completion
+//                order, the order of the rx-ready ring); first fragment index
+//   k_ra_emit    every arrival of a complete request writes its table entry at
+//                first + seq_num, and wipes its hash cell for the next call
+
+struct RaArgs {
+  const uint8_t *ring;
+  uint32_t n_slots, slot_size, ref64, n;
+  const uint32_t *arrivals;
+  const uint32_t *len_nic;
+  uint64_t req_size;  // REF64 readiness: bytes == req_size; BL58: fragments == num_frags
+  uint32_t hmask;     // table size - 1
+  uint32_t max_req;
+  // hash table
+  unsigned long long *keys;
+  uint32_t *cnt, *last, *want, *cell_first, *cell_rank;
+  unsigned long long *bytes;
+  // per arrival
+  uint32_t *arr_cell, *arr_len, *arr_fidx;
+  unsigned long long *arr_pack;  // (1 << 32 | fragments) at the completing arrival, else 0; then its local scan
+  unsigned long long *blk;       // workgroup totals, then their scan; blk[n_blocks] = grand total
+  uint32_t n_blocks;
+  // outputs
+  uint32_t *frag_slot, *frag_len, *req_first;
+  uint64_t *req_token;
+  uint32_t *counts;  // [0] requests, [1] fragments, [2] arrivals left out
+  uint32_t *status;
+};
+
+constexpr uint32_t kRaNoCell = 0xffffffffu;
+constexpr int kRaBlock = 1024;
+
+__device__ __forceinline__ uint32_t ra_hash(unsigned long long k)
+{
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 33;
+  return (uint32_t)k;
+}
+
+__global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
+{
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.n) return;
+  const uint32_t slot = a.arrivals[i];
+  uint32_t cell = kRaNoCell, len = 0, fidx = 0;
+  if (slot >= a.n_slots) {
+    atomicOr(a.status, kStBadSlot);
+  } else {
+    const uint8_t *h = a.ring + (size_t)slot * a.slot_size;
+    const uint32_t t0 = load32_any(h + 42), t1 = load32_any(h + 46);
+    const unsigned long long token = ((unsigned long long)t1 << 32) | t0;
+    uint32_t want = 0;
+    if (a.ref64) {
+      fidx = load32_any(h + 58) & 0xffffu;
+      len = a.len_nic[slot];
+    } else {
+      const uint32_t w = load32_any(h + 50);
+      fidx = w & 0xffffu;
+      want = w >> 16;
+      len = a.len_nic ? a.len_nic[slot] : load32_any(h + 54);
+    }
+    const uint32_t hl = a.ref64 ? 64u : 58u;
+    if (len > a.slot_size - hl) {
+      atomicOr(a.status, kStBadLen);
+    } else if (token != 0) {  // token 0: dropped (src/transport/dpdk_transport_ng.h:231)
+      uint32_t c = ra_hash(token) & a.hmask;
+      for (uint32_t probe = 0; probe <= a.hmask; probe++) {
+        const unsigned long long old = atomicCAS(&a.keys[c], 0ull, token);
+        if (old == 0ull || old == token) {
+          cell = c;
+          break;
+        }
+        c = (c + 1) & a.hmask;
+      }
+      if (cell != kRaNoCell) {
+        atomicAdd(&a.cnt[cell], 1u);
+        atomicAdd(&a.bytes[cell], (unsigned long long)len);
+        atomicMax(&a.last[cell], i);
+        if (!a.ref64) a.want[cell] = want;  // every fragment of a request says the same
+      }
+    }
+  }
+  a.arr_cell[i] = cell;
+  a.arr_len[i] = len;
+  a.arr_fidx[i] = fidx;
+}
+
+__device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell)
+{
+  return a.ref64 ? a.bytes[cell] == a.req_size : a.cnt[cell] == a.want[cell];
+}
+
+__global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
+{
+  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  const uint32_t i = blockIdx.x * kRaBlock + threadIdx.x;
+  unsigned long long pack = 0;
+  if (i < a.n) {
+    const uint32_t cell = a.arr_cell[i];
+    if (cell != kRaNoCell && a.last[cell] == i && ra_complete(a, cell))
+      pack = (1ull << 32) | a.cnt[cell];
+  }
+  uint64_t tot;
+  const uint64_t ex = block_exclusive_scan<kRaBlock>(pack, wave_tot, &tot);
+  if (i < a.n) a.arr_pack[i] = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
+  if (threadIdx.x == 0) a.blk[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
+{
+  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  uint64_t run = 0;
+  for (uint32_t base = 0; base < a.n_blocks; base += kRaBlock) {
+    const uint32_t b = base + threadIdx.x;
+    const uint64_t v = b < a.n_blocks ? a.blk[b] : 0;
+    uint64_t tot;
+    const uint64_t ex = block_exclusive_scan<kRaBlock>(v, wave_tot, &tot);
+    if (b < a.n_blocks) a.blk[b] = run + ex;
+    run += tot;
+  }
+  if (threadIdx.x == 0) {
+    a.blk[a.n_blocks] = run;
+    const uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
+    a.counts[0] = n_req;
+    a.counts[1] = n_frag;
+    if (n_req <= a.max_req) a.req_first[n_req] = n_frag;
+    else atomicOr(a.status, kStBadTable);
+  }
+}
+
+__global__ __launch_bounds__(256) void k_ra_assign(RaArgs a)
+{
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.n) return;
+  const unsigned long long p = a.arr_pack[i];
+  if (!(p >> 63)) return;
+  const unsigned long long v = (p & ~(1ull << 63)) + a.blk[i / kRaBlock];
+  const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v;
+  if (r >= a.max_req) return;  // refused by k_ra_scan
+  const uint32_t cell = a.arr_cell[i];
+  a.cell_rank[cell] = r;
+  a.cell_first[cell] = first;
+  a.req_first[r] = first;
+  if (a.req_token) a.req_token[r] = a.keys[cell];
+}
+
+__global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
+{
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.n) return;
+  const uint32_t cell = a.arr_cell[i];
+  if (cell == kRaNoCell) {
+    atomicAdd(&a.counts[2], 1u);
+    return;
+  }
+  // completeness was decided on the counters; they are read here before any
+  // thread of this kernel wipes them only through the flag the assign pass left:
+  // a complete request's cell carries its rank in cell_rank, an incomplete one kRaNoCell
+  const uint32_t rank = a.cell_rank[cell];
+  if (rank != kRaNoCell && rank < a.max_req) {
+    const uint32_t first = a.cell_first[cell];
+    const uint32_t n = a.req_first[rank + 1] - first;
+    const uint32_t fidx = a.arr_fidx[i];
+    if (fidx < n) {
+      a.frag_slot[first + fidx] = a.arrivals[i];
+      a.frag_len[first + fidx] = a.arr_len[i];
+    } else {
+      atomicOr(a.status, kStBadTable);  // a sequence number beyond the request's fragments
+    }
+  } else {
+    atomicAdd(&a.counts[2], 1u);  // its request did not complete among these arrivals
+  }
+}
+
+// Wipes the cells this call used, so that the table is empty for the next one.
+__global__ __launch_bounds__(256) void k_ra_wipe(RaArgs a)
+{
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.n) return;
+  const uint32_t cell = a.arr_cell[i];
+  if (cell == kRaNoCell) return;
+  a.keys[cell] = 0;
+  a.cnt[cell] = 0;
+  a.bytes[cell] = 0;
+  a.last[cell] = 0;
+  a.want[cell] = 0;
+  a.cell_rank[cell] = kRaNoCell;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -796,8 +1002,12 @@ struct sg_hip_ctx {
   // profiling
   bool profiling = false;
   std::vector<EvPair> ev_used, ev_free;
-  double prof_ms[5] = {0, 0, 0, 0, 0};
-  uint64_t prof_n[5] = {0, 0, 0, 0, 0};
+  double prof_ms[6] = {0, 0, 0, 0, 0, 0};
+  uint64_t prof_n[6] = {0, 0, 0, 0, 0, 0};
+  // reassembly scratch, allocated by the first sg_hip_reassemble call
+  void *ra_mem = nullptr;
+  uint32_t ra_cells = 0;  // hash table size (power of two >= 2 * max_frames)
+  uint32_t *h_counts = nullptr;  // pinned: requests, fragments, arrivals left out
   char err[512] = {0};
 };
 
@@ -1034,6 +1244,8 @@ void sg_hip_destroy(sg_hip_ctx *c)
   if (c->h_runs) (void)hipHostFree(c->h_runs);
   if (c->h_ptrs) (void)hipHostFree(c->h_ptrs);
   if (c->h_status) (void)hipHostFree(c->h_status);
+  if (c->h_counts) (void)hipHostFree(c->h_counts);
+  (void)hipFree(c->ra_mem);
   if (c->own_stream && c->stream) (void)hipStreamDestroy(c->stream);
   delete c;
 }
@@ -1084,13 +1296,13 @@ int sg_hip_set_profiling(sg_hip_ctx *c, int on)
   if (!c) return SG_E_INVAL;
   int rc = sg_hip_sync(c);
   c->profiling = on != 0;
-  for (int i = 0; i < 5; i++) { c->prof_ms[i] = 0; c->prof_n[i] = 0; }
+  for (int i = 0; i < 6; i++) { c->prof_ms[i] = 0; c->prof_n[i] = 0; }
   return rc;
 }
 
 int sg_hip_kernel_time(sg_hip_ctx *c, int which, double *total_ms, uint64_t *launches)
 {
-  if (!c || which < 0 || which > 4) return fail(c, SG_E_INVAL, "kernel index %d", which);
+  if (!c || which < 0 || which > 5) return fail(c, SG_E_INVAL, "kernel index %d", which);
   int rc = sg_hip_sync(c);
   if (total_ms) *total_ms = c->prof_ms[which];
   if (launches) *launches = c->prof_n[which];
@@ -1417,6 +1629,99 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     if (rc != SG_OK) return rc;
   }
   return finish(c, a->flags);
+}
+
+// ---- reassembly ----------------------------------------------------------------
+
+int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_req_out, uint32_t *n_frags_out,
+                      uint32_t *n_left_out)
+{
+  if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
+  int rc = check_ring(c, a->ring, "rx");
+  if (rc != SG_OK) return rc;
+  if (n_req_out) *n_req_out = 0;
+  if (n_frags_out) *n_frags_out = 0;
+  if (n_left_out) *n_left_out = 0;
+  if (a->n_arrivals == 0) return SG_OK;
+  if (a->n_arrivals > c->max_frames) return fail(c, SG_E_INVAL, "n_arrivals %u > max_frames %u of this context", a->n_arrivals, c->max_frames);
+  if (!a->arrivals || !a->frag_slot || !a->frag_len || !a->req_first) return fail(c, SG_E_INVAL, "null tables");
+  const bool ref64 = a->ring.hdr_profile == SG_HDR_REF64;
+  if (ref64 && (!a->len_nic || !a->req_size)) return fail(c, SG_E_INVAL, "REF64 headers need len_nic and the server-wide request size");
+  DeviceGuard g(c->device);
+
+  const uint32_t n_max = c->max_frames;
+  if (!c->ra_mem) {
+    uint32_t cells = 2;
+    while (cells < 2 * n_max) cells <<= 1;
+    // keys u64, bytes u64, cnt/last/want/cell_first/cell_rank u32 per cell;
+    // arr_cell/arr_len/arr_fidx u32 + arr_pack u64 per arrival; blk u64 per workgroup
+    const size_t n_blk = (n_max + kRaBlock - 1) / kRaBlock + 1;
+    const size_t bytes = (size_t)cells * (8 + 8 + 5 * 4) + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 64;
+    HIP_TRY(c, hipMalloc(&c->ra_mem, bytes));
+    HIP_TRY(c, hipMemsetAsync(c->ra_mem, 0, bytes, c->stream));
+    c->ra_cells = cells;
+    // cell_rank starts as "no request"
+    uint8_t *base = static_cast<uint8_t *>(c->ra_mem);
+    uint32_t *cell_rank = reinterpret_cast<uint32_t *>(base + (size_t)cells * (8 + 8 + 4 * 4));
+    HIP_TRY(c, hipMemsetAsync(cell_rank, 0xff, (size_t)cells * 4, c->stream));
+    HIP_TRY(c, hipHostMalloc((void **)&c->h_counts, 4 * sizeof(uint32_t), hipHostMallocDefault));
+  }
+  RaArgs r;
+  memset(&r, 0, sizeof r);
+  r.ring = static_cast<const uint8_t *>(a->ring.base);
+  r.n_slots = a->ring.n_slots;
+  r.slot_size = a->ring.slot_size;
+  r.ref64 = ref64;
+  r.n = a->n_arrivals;
+  r.arrivals = a->arrivals;
+  r.len_nic = a->len_nic;
+  r.req_size = a->req_size;
+  // a table at least twice the arrivals of THIS call keeps probes short and the touched memory small
+  uint32_t cells = 2;
+  while (cells < 2 * a->n_arrivals) cells <<= 1;
+  r.hmask = cells - 1;
+  r.max_req = c->max_reqs;
+  const size_t C = c->ra_cells;
+  uint8_t *m = static_cast<uint8_t *>(c->ra_mem);
+  r.keys = reinterpret_cast<unsigned long long *>(m); m += C * 8;
+  r.bytes = reinterpret_cast<unsigned long long *>(m); m += C * 8;
+  r.cnt = reinterpret_cast<uint32_t *>(m); m += C * 4;
+  r.last = reinterpret_cast<uint32_t *>(m); m += C * 4;
+  r.want = reinterpret_cast<uint32_t *>(m); m += C * 4;
+  r.cell_first = reinterpret_cast<uint32_t *>(m); m += C * 4;
+  r.cell_rank = reinterpret_cast<uint32_t *>(m); m += C * 4;
+  r.arr_pack = reinterpret_cast<unsigned long long *>(m); m += (size_t)n_max * 8;
+  r.blk = reinterpret_cast<unsigned long long *>(m); m += ((n_max + kRaBlock - 1) / kRaBlock + 1) * 8;
+  r.arr_cell = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
+  r.arr_len = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
+  r.arr_fidx = reinterpret_cast<uint32_t *>(m);
+  r.n_blocks = (a->n_arrivals + kRaBlock - 1) / kRaBlock;
+  r.frag_slot = a->frag_slot;
+  r.frag_len = a->frag_len;
+  r.req_first = a->req_first;
+  r.req_token = a->req_token;
+  r.counts = reinterpret_cast<uint32_t *>(c->req_size);  // the descriptor pass's scratch is idle here
+  r.status = c->status;
+
+  const uint32_t g256 = (a->n_arrivals + 255) / 256;
+  rc = prof_begin(c, 5);
+  if (rc != SG_OK) return rc;
+  HIP_TRY(c, hipMemsetAsync(r.counts, 0, 4 * sizeof(uint32_t), c->stream));
+  k_ra_insert<<<g256, 256, 0, c->stream>>>(r);
+  k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
+  k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);
+  k_ra_assign<<<g256, 256, 0, c->stream>>>(r);
+  k_ra_emit<<<g256, 256, 0, c->stream>>>(r);
+  k_ra_wipe<<<g256, 256, 0, c->stream>>>(r);
+  rc = prof_end(c);
+  if (rc != SG_OK) return rc;
+  HIP_TRY(c, hipMemcpyAsync(c->h_counts, r.counts, 3 * sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
+  rc = finish(c, 0);
+  if (rc != SG_OK) return rc;
+  if (n_req_out) *n_req_out = c->h_counts[0];
+  if (n_frags_out) *n_frags_out = c->h_counts[1];
+  if (n_left_out) *n_left_out = c->h_counts[2];
+  return SG_OK;
 }
 
 }  // extern "C"

@@ -179,6 +179,26 @@ class SgContext:
         if rc != capi.SG_OK:
             self._check(rc)
 
+    def reassemble(self, ring: RingRef, arrivals: torch.Tensor, n_arrivals: int, frag_slot: torch.Tensor,
+                   frag_len: torch.Tensor, req_first: torch.Tensor, req_token: Optional[torch.Tensor] = None,
+                   len_nic: Optional[torch.Tensor] = None, req_size: int = 0):
+        """Sort a burst of arrivals into requests on the device; returns
+        (requests, fragments, arrivals left out)."""
+        a = capi.ReassembleArgs()
+        a.ring = ring.desc()
+        a.arrivals = arrivals.data_ptr()
+        a.len_nic = len_nic.data_ptr() if len_nic is not None else None
+        a.n_arrivals = n_arrivals
+        a.req_size = int(req_size)
+        a.frag_slot = frag_slot.data_ptr()
+        a.frag_len = frag_len.data_ptr()
+        a.req_first = req_first.data_ptr()
+        a.req_token = req_token.data_ptr() if req_token is not None else None
+        n_req, n_frag, n_left = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+        self._check(self.lib.sg_hip_reassemble(self.h, C.byref(a), C.byref(n_req), C.byref(n_frag),
+                                               C.byref(n_left)))
+        return int(n_req.value), int(n_frag.value), int(n_left.value)
+
     # -- per request ---------------------------------------------------------
     def copy_runs(self, src: Sequence[int], dst: Sequence[int], lens: Sequence[int],
                   scatter: bool = False) -> None:
@@ -230,6 +250,7 @@ class DeviceWorkload:
             body = [first[:-1].astype(np.uint32) + np.uint32(i * int(first[-1])) for i in range(k)]
             return np.concatenate(body + [np.array([int(first[-1]) * k], dtype=np.uint32)])
 
+        self.arrivals = to_dev(tile_slots(w.arrivals, w.n_slots), dev)
         self.frag_slot = to_dev(tile_slots(w.frag_slot, w.n_slots), dev)
         self.frag_len = to_dev(np.tile(w.frag_len, k), dev)
         self.req_first = to_dev(tile_csr(w.req_first), dev)
