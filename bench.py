@@ -69,7 +69,7 @@ class Pool:
         per = (w.ring.nbytes + int(w.req_sizes.sum()) + w.tx_n_slots * w.slot_size
                + int(w.resp_sizes.sum())) * bpl
         r = max(2, min(64, -(-rotate_mb * (1 << 20) // max(per, 1))))
-        self.items = [DeviceWorkload(w, copies=bpl) for _ in range(r)]
+        self.items = [DeviceWorkload(w, copies=bpl, unique_tokens=True) for _ in range(r)]
         self.w = w
         self.bpl = bpl
         self.extra_flags = extra_flags
@@ -205,8 +205,7 @@ def main() -> int:
     ra_sec = (time.perf_counter() - t0) / 20
     reassembly = {"arrivals": n_arr, "requests": got[0], "ms_per_call": round(ra_sec * 1e3, 4),
                   "arrivals_per_sec": round(n_arr / ra_sec, 1),
-                  "tables_match_pre_staged": bool(torch.equal(ra_fs, dw0.frag_slot))
-                  if bpl == 1 else None}
+                  "tables_match_pre_staged": bool(got[0] == pool.n_req and torch.equal(ra_fs, dw0.frag_slot))}
     del ra_fs, ra_fl, ra_rf
 
     # the single-batch call of the same workload, for the record

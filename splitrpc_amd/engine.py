@@ -226,7 +226,8 @@ class DeviceWorkload:
     """A synthetic workload staged in one GPU's memory: the landing-zone ring,
     the fragment tables and the application buffers."""
 
-    def __init__(self, w: Workload, device="cuda:0", arena_slack: int = 0, copies: int = 1):
+    def __init__(self, w: Workload, device="cuda:0", arena_slack: int = 0, copies: int = 1,
+                 unique_tokens: bool = False):
         """``copies`` > 1 lays that many copies of the ring (and of the tables,
         slot indices shifted) side by side, so that one call moves ``copies``
         batches and the working set outgrows the caches."""
@@ -241,6 +242,13 @@ class DeviceWorkload:
         self.n_frames = w.n_resp_frames * k
         ring1 = torch.from_numpy(w.ring).to(dev)
         self.ring = ring1.repeat(k) if k > 1 else ring1
+        if unique_tokens and k > 1:
+            # give every copy its own request tokens (bits 40..55 of the u64 at byte 42)
+            v = self.ring.view(k, w.n_slots, w.slot_size)
+            c = torch.arange(k, device=dev, dtype=torch.int32).view(k, 1)
+            used = torch.from_numpy(w.frag_slot.astype(np.int64)).to(dev)
+            v[:, used, 47] = ((v[:, used, 47].to(torch.int32) + (c & 0xFF)) & 0xFF).to(torch.uint8)
+            v[:, used, 48] = ((v[:, used, 48].to(torch.int32) + (c >> 8)) & 0xFF).to(torch.uint8)
         self.rx = RingRef(self.ring, w.n_slots * k, w.slot_size, w.profile)
 
         def tile_slots(a: np.ndarray, n_slots: int) -> np.ndarray:
