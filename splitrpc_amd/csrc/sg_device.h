@@ -408,14 +408,23 @@ __device__ __forceinline__ uint32_t hdr_src_index(uint32_t j)
   return j;
 }
 
-// Returns the final value of header byte `lane` (garbage on lanes >= hl).
-__device__ __forceinline__ uint32_t hdr_rewrite(const uint8_t *__restrict__ in, uint32_t lane,
-                                                const HdrFields &f, uint32_t payload_sum)
+// The byte lane `lane` starts from: the incoming header's byte at the swapped
+// position.  Split from hdr_finish so that a kernel can have this load in
+// flight together with its payload loads.
+__device__ __forceinline__ uint32_t hdr_fetch(const uint8_t *__restrict__ in, uint32_t lane, uint32_t hl)
+{
+  uint32_t b = 0;
+  if (lane < hl) b = in[hdr_src_index(lane)];
+  return b;
+}
+
+// Returns the final value of header byte `lane` (garbage on lanes >= hl) from
+// the fetched byte.
+__device__ __forceinline__ uint32_t hdr_finish(uint32_t b, uint32_t lane, const HdrFields &f,
+                                               uint32_t payload_sum)
 {
   const uint32_t j = lane;
   const bool live = j < f.hl;
-  uint32_t b = 0;
-  if (live) b = in[hdr_src_index(j)];
 
   const uint32_t L = (f.hl - 42u) + f.payload_len;
   const uint32_t tot = (28u + L) & 0xffffu;
@@ -468,6 +477,12 @@ __device__ __forceinline__ uint32_t hdr_rewrite(const uint8_t *__restrict__ in, 
     }
   }
   return b;
+}
+
+__device__ __forceinline__ uint32_t hdr_rewrite(const uint8_t *__restrict__ in, uint32_t lane,
+                                                const HdrFields &f, uint32_t payload_sum)
+{
+  return hdr_finish(hdr_fetch(in, lane, f.hl), lane, f, payload_sum);
 }
 
 }  // namespace sg

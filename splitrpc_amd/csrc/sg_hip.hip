@@ -237,54 +237,96 @@ __global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
   if (lane == 0) prep_finish(a, r, carry, bad);
 }
 
-// Scan of the request totals through the bump ring (one workgroup):
+// Scan of the request totals through the bump ring:
 //   ret = base + off; off = (off + size) % capacity   (src/p2p_rpc_tring.h:27-33)
-// Each thread owns kScanPerThread consecutive requests (read and written as
-// 16-byte pairs), so one pass of the workgroup covers 16384 requests.
+// Up to kScanTile requests: one workgroup does it all (k_req_scan).  Beyond:
+// one workgroup per tile scans locally (k_req_scan_local), one workgroup
+// scans the tile totals from the cursor (k_req_scan_tiles), and the tiles add
+// their base (k_req_scan_add).
 constexpr int kScanBlock = 1024;
-constexpr int kScanPerThread = 16;
-typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+constexpr int kScanPerThread = 4;
+constexpr uint32_t kScanTile = kScanBlock * kScanPerThread;
+
+// Exclusive scan of one tile; returns this thread's prefix for its first
+// request and leaves its requests' sizes in sz[].
+__device__ __forceinline__ uint64_t scan_tile(const PrepArgs &a, uint32_t q0, uint64_t *sz,
+                                              uint64_t *wave_tot, uint64_t *tot)
+{
+  uint64_t mine = 0;
+#pragma unroll
+  for (int k = 0; k < kScanPerThread; k++) {
+    sz[k] = (q0 + k < a.n_req) ? a.req_size[q0 + k] : 0;
+    mine += sz[k];
+  }
+  return block_exclusive_scan<kScanBlock>(mine, wave_tot, tot);
+}
+
+__device__ __forceinline__ void scan_emit(const PrepArgs &a, uint32_t q0, const uint64_t *sz, uint64_t off)
+{
+  // off < capacity on entry; every size <= capacity (checked by the descriptor pass)
+#pragma unroll
+  for (int k = 0; k < kScanPerThread; k++) {
+    if (q0 + k < a.n_req) {
+      a.req_off[q0 + k] = off;
+      if (a.offsets_out) a.offsets_out[q0 + k] = off;
+    }
+    off += sz[k];
+    if (off >= a.cap) off %= a.cap;
+  }
+}
+
 __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
   uint64_t run = *a.cursor_in % a.cap;
-  for (uint32_t base = 0; base < a.n_req; base += kScanBlock * kScanPerThread) {
+  for (uint32_t base = 0; base < a.n_req; base += kScanTile) {
     const uint32_t q0 = base + threadIdx.x * kScanPerThread;
-    uint64_t sz[kScanPerThread];
-    uint64_t mine = 0;
-    if (q0 + kScanPerThread <= a.n_req) {
-#pragma unroll
-      for (int k = 0; k < kScanPerThread; k += 2) {
-        const u64x2 v = *reinterpret_cast<const u64x2 *>(a.req_size + q0 + k);  // q0 is a multiple of 16
-        sz[k] = v[0];
-        sz[k + 1] = v[1];
-      }
-    } else {
-#pragma unroll
-      for (int k = 0; k < kScanPerThread; k++) sz[k] = (q0 + k < a.n_req) ? a.req_size[q0 + k] : 0;
-    }
-#pragma unroll
-    for (int k = 0; k < kScanPerThread; k++) mine += sz[k];
-    uint64_t tot;
-    uint64_t ex = block_exclusive_scan<kScanBlock>(mine, wave_tot, &tot);
-    // offsets stay below 2 * capacity between reductions: run < cap and every
-    // prefix of one pass is reduced as it grows
-    uint64_t off = (run + ex) % a.cap;
-#pragma unroll
-    for (int k = 0; k < kScanPerThread; k++) {
-      if (q0 + k < a.n_req) {
-        a.req_off[q0 + k] = off;
-        if (a.offsets_out) a.offsets_out[q0 + k] = off;
-      }
-      off += sz[k];  // sz <= cap (checked by the descriptor pass), so one subtraction reduces
-      if (off >= a.cap) off = a.cap ? off % a.cap : 0;
-    }
+    uint64_t sz[kScanPerThread], tot;
+    const uint64_t ex = scan_tile(a, q0, sz, wave_tot, &tot);
+    scan_emit(a, q0, sz, (run + ex) % a.cap);
     run = (run + tot) % a.cap;
   }
   if (threadIdx.x == 0) {
     *a.cursor_out = run;
     if (a.offsets_out) a.offsets_out[a.n_req] = run;
   }
+}
+
+// tile totals go to tile_tot[blockIdx.x]; the local prefixes are recomputed by k_req_scan_add
+__global__ __launch_bounds__(kScanBlock) void k_req_scan_local(PrepArgs a, uint64_t *tile_tot)
+{
+  __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  const uint32_t q0 = blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
+  uint64_t sz[kScanPerThread], tot;
+  (void)scan_tile(a, q0, sz, wave_tot, &tot);
+  if (threadIdx.x == 0) tile_tot[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(kScanBlock) void k_req_scan_tiles(PrepArgs a, uint64_t *tile_tot, uint32_t n_tiles)
+{
+  __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  uint64_t run = *a.cursor_in % a.cap;
+  for (uint32_t base = 0; base < n_tiles; base += kScanBlock) {
+    const uint32_t t = base + threadIdx.x;
+    const uint64_t v = t < n_tiles ? tile_tot[t] % a.cap : 0;
+    uint64_t tot;
+    const uint64_t ex = block_exclusive_scan<kScanBlock>(v, wave_tot, &tot);
+    if (t < n_tiles) tile_tot[t] = (run + ex % a.cap) % a.cap;
+    run = (run + tot % a.cap) % a.cap;
+  }
+  if (threadIdx.x == 0) {
+    *a.cursor_out = run;
+    if (a.offsets_out) a.offsets_out[a.n_req] = run;
+  }
+}
+
+__global__ __launch_bounds__(kScanBlock) void k_req_scan_add(PrepArgs a, const uint64_t *tile_base)
+{
+  __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  const uint32_t q0 = blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
+  uint64_t sz[kScanPerThread], tot;
+  const uint64_t ex = scan_tile(a, q0, sz, wave_tot, &tot);
+  scan_emit(a, q0, sz, (tile_base[blockIdx.x] + ex % a.cap) % a.cap);
 }
 
 // ---------------------------------------------------------------------------
@@ -658,7 +700,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
   static_assert(!(FULL_CSUM && LONG), "a summed frame belongs to one wavefront");
   const uint32_t w = item_of_wave(a.remap != 0);
-  const uint32_t pieces = LONG ? a.pieces : 1u;
+  const uint32_t pieces = LONG ? a.pieces : 1u;  // FULL_CSUM: a.pieces only says "long frames"
   const uint32_t item = LONG ? w / pieces : w;
   const uint32_t piece = LONG ? w - item * pieces : 0;
   if (item >= a.n_items) return;
@@ -707,24 +749,33 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   // (the TX slot may be the very slot the header comes from)
   const uint8_t *hin = a.rx + (size_t)hs * a.rx_slot_size;
   HdrFields hf{a.hl, a.ref64, a.flags, item - f0, nf, d[1]};
-  uint32_t hb = 0;
-  if (!FULL_CSUM) hb = hdr_rewrite(hin, lane, hf, 0);
-
-  uint32_t acc = 0;
-  uint8_t *from;
-  if (LONG && d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
-    PieceState ps;
-    piece_begin(ps, from, slot + a.hl, d[1], lane, 0, kPieceChunks);
-    piece_end<false>(ps, lane);
+  // header bytes and payload chunks are fetched together; the header arithmetic
+  // then runs while the payload is still on its way
+  const uint32_t raw = hdr_fetch(hin, lane, a.hl);
+  uint32_t hb = 0, acc = 0;
+  uint8_t *from = nullptr;
+  const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
+  RunState rs;
+  PieceState ps;
+  // a summed frame stays with one wavefront; a long one then walks all its
+  // chunks with the deeper pipeline of the piece copy
+  const bool whole_long = FULL_CSUM && a.pieces > 1;
+  if (plain) {
+    if (LONG) piece_begin(ps, from, slot + a.hl, d[1], lane, 0, kPieceChunks);
+    else if (whole_long) piece_begin(ps, from, slot + a.hl, d[1], lane, 0, kWholeRun);
+    else run_begin(rs, from, slot + a.hl, d[1], lane);
+  }
+  if (!FULL_CSUM) hb = hdr_finish(raw, lane, hf, 0);
+  if (plain) {
+    if (LONG) acc = piece_end<false>(ps, lane);
+    else if (whole_long) acc = piece_end<FULL_CSUM>(ps, lane);
+    else acc = run_end<FULL_CSUM>(rs, lane);
   } else if (d[1]) {
     acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
   }
-  if (FULL_CSUM) {
-    // the payload copy wrote past the header only, so in place the request
-    // header is still intact here
-    const uint32_t psum = wave_sum(acc);
-    hb = hdr_rewrite(hin, lane, hf, psum);
-  }
+  if (FULL_CSUM) hb = hdr_finish(raw, lane, hf, wave_sum(acc));
+  // the payload went past the header only, so a TX slot that is the header's own
+  // source still held the request header when it was fetched above
   if (lane < a.hl) slot[lane] = (uint8_t)hb;
 }
 
@@ -989,6 +1040,7 @@ struct sg_hip_ctx {
   u32x4 *desc = nullptr;
   uint64_t *req_size = nullptr;
   uint64_t *req_off = nullptr;
+  uint64_t *tile_tot = nullptr;  // one total per 4096 requests, for the tiled request scan
   // bump-ring cursors: request arena at [0 + parity], response arena at
   // [2 + parity]; a launch reads one parity and writes the other
   uint64_t *cursors = nullptr;
@@ -1149,7 +1201,17 @@ int launch_prep(sg_hip_ctx *c, const PrepArgs &p)
   } else {
     k_prep_block<1024><<<p.n_req, 1024, 0, c->stream>>>(p);
   }
-  if (p.packed && !p.fixed_offsets) k_req_scan<<<1, kScanBlock, 0, c->stream>>>(p);
+  if (p.packed && !p.fixed_offsets) {
+    if (p.n_req <= 2 * kScanTile) {
+      k_req_scan<<<1, kScanBlock, 0, c->stream>>>(p);
+    } else {
+      const uint32_t n_tiles = (p.n_req + kScanTile - 1) / kScanTile;
+      uint64_t *tile_tot = c->tile_tot;
+      k_req_scan_local<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot);
+      k_req_scan_tiles<<<1, kScanBlock, 0, c->stream>>>(p, tile_tot, n_tiles);
+      k_req_scan_add<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot);
+    }
+  }
   return prof_end(c);
 }
 
@@ -1198,6 +1260,7 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMalloc(&c->desc, sizeof(u32x4) * (size_t)c->max_frames));
   HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
+  HIP_TRY(nullptr, hipMalloc(&c->tile_tot, sizeof(uint64_t) * ((size_t)c->max_reqs / kScanTile + 2)));
   HIP_TRY(nullptr, hipMalloc(&c->cursors, 4 * sizeof(uint64_t)));
   HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
   HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 4 * sizeof(uint64_t), c->stream));
@@ -1239,6 +1302,7 @@ void sg_hip_destroy(sg_hip_ctx *c)
   (void)hipFree(c->desc);
   (void)hipFree(c->req_size);
   (void)hipFree(c->req_off);
+  (void)hipFree(c->tile_tot);
   (void)hipFree(c->cursors);
   (void)hipFree(c->status);
   if (c->h_runs) (void)hipHostFree(c->h_runs);
@@ -1558,9 +1622,10 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.rule.cursor_out = c->cursors + 2 + (c->parity[1] ^ 1u);
     if (app.n_tensors == 0) c->parity[1] ^= 1u;
     sa.rule.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
-    sa.pieces = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : pieces_for(a->mtu);
+    sa.pieces = pieces_for(a->mtu);
+    const uint32_t waves_per_frame = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces;
     uint32_t grid;
-    geometry((uint64_t)a->n_frames * sa.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry((uint64_t)a->n_frames * waves_per_frame, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
     if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, true, false><<<grid, kBlock, 0, c->stream>>>(sa);
@@ -1617,9 +1682,10 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.n_items = a->n_frames;
     sa.status = c->status;
     sa.app = app;
-    sa.pieces = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : pieces_for(a->mtu);
+    sa.pieces = pieces_for(a->mtu);
+    const uint32_t waves_per_frame = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces;
     uint32_t grid;
-    geometry((uint64_t)a->n_frames * sa.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry((uint64_t)a->n_frames * waves_per_frame, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
     if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, false, false><<<grid, kBlock, 0, c->stream>>>(sa);

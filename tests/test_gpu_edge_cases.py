@@ -379,3 +379,31 @@ def test_many_batches_per_call_equal_one_batch_each(ctx):
     tb = many.tx_ring.cpu().numpy().reshape(5, -1)
     assert all(np.array_equal(ta, tb[k]) for k in range(5))
     big.close()
+
+
+def test_tiled_request_scan_beyond_8192_requests():
+    """More requests than one workgroup scans in two passes: the tiled scan of
+    the request totals gives the same offsets as the sequential bump ring."""
+    w = synth.make_workload(4, 3000)
+    k = 3
+    big = SgContext(0, max_reqs=3000 * k, max_frames=1 << 17)
+    dw = DeviceWorkload(w, copies=k)
+    total = int(w.req_sizes.sum())
+    for cursor, cap_extra in ((0, 0), (12345, 777)):
+        cap = total * k + cap_extra
+        arena = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+        offs = torch.zeros(dw.n_req + 1, dtype=torch.int64, device=DEV)
+        big.set_cursor(0, cursor)
+        big.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags,
+                         AppRef(arena=arena, cap=cap), offs)
+        sizes = np.tile(w.req_sizes, k).astype(np.uint64)
+        want = (cursor + np.concatenate([[0], np.cumsum(sizes)])) % cap
+        assert np.array_equal(offs.cpu().numpy().view(np.uint64), want.astype(np.uint64))
+        assert big.get_cursor(0) == int(want[-1])
+        got = arena.cpu().numpy()
+        exp = np.zeros(cap, np.uint8)
+        pay = np.tile(w.req_payload, k)
+        idx = (cursor + np.arange(pay.size, dtype=np.int64)) % cap
+        exp[idx] = pay
+        assert np.array_equal(got, exp), first_diff(got, exp)
+    big.close()
