@@ -235,128 +235,54 @@ __device__ __forceinline__ uint32_t copy_run(const uint8_t *__restrict__ src,
   return run_end<CSUM>(r, lane);
 }
 
-// A LONG run (jumbo frames) in the hands of several wavefronts: a wavefront
-// covers the destination chunks [c_begin, c_end) of the run, kPieceChunks at a
-// time; the one that covers chunk 0 also moves the head bytes, the one that
-// covers the last chunk the tail bytes.  Same copy scheme as RunState above.
-// Kept apart from it because the extra range arithmetic costs the short-run
-// kernels 5-10 % when it sits on their path.
+// A LONG run (jumbo frames) is cut into sub-runs of kPieceChunks destination
+// chunks that different wavefronts (or one wavefront, two at a time) copy with
+// the functions above: sub-run 0 is the head bytes plus the first
+// kPieceChunks aligned chunks, every later one starts on a 16-byte destination
+// boundary, the last one takes the tail bytes.  A sub-run's aligned source
+// loads may reach into its neighbours' bytes -- which are bytes of the same run.
 constexpr uint32_t kPieceChunks = 126;
-constexpr uint32_t kWholeRun = 0xffffffffu;
+constexpr uint32_t kPieceBytes = kPieceChunks * 16;
 
-struct PieceState {
-  const uint8_t *src;
-  uint8_t *dst;
-  const uint8_t *sa;  // source of the first aligned store, rounded down to 16
-  uint8_t *d;         // first aligned store
-  uint32_t c_begin;   // destination chunks this wavefront stores: [c_begin, c_end)
-  uint32_t c_end;
-  uint32_t lim;       // last source chunk that may be loaded
-  uint32_t p;         // source phase
-  uint32_t eoff;      // this lane's edge byte, if any
-  uint32_t eb;
-  bool edge;
-  u32x4 v0, v1;
-};
-
-// `first` / `count`: the destination chunks asked of this wavefront
-// (0 / kWholeRun: the whole run).
-__device__ __forceinline__ void piece_begin(PieceState &r, const uint8_t *__restrict__ src,
-                                          uint8_t *__restrict__ dst, uint32_t len, uint32_t lane,
-                                          uint32_t first = 0, uint32_t count = kWholeRun)
-{
-  uint32_t head = (uint32_t)(-(uintptr_t)dst) & 15u;
-  head = head < len ? head : len;
-  const uint32_t body = (len - head) >> 4;
-  const uint32_t tail = (len - head) & 15u;
-  r.src = src;
-  r.dst = dst;
-  r.c_begin = first < body ? first : body;
-  r.c_end = (count == kWholeRun || first + count > body) ? body : first + count;
-  if (r.c_end < r.c_begin) r.c_end = r.c_begin;
-  // head bytes go with chunk 0, tail bytes with the last chunk (with chunk 0's
-  // wavefront when there is no chunk at all)
-  const bool has_head = first == 0;
-  const bool has_tail = body == 0 ? first == 0 : (r.c_begin < body && r.c_end == body);
-  r.edge = false;
-  r.eoff = 0;
-  if (lane < 16) {
-    r.edge = has_head && lane < head;
-    r.eoff = lane;
-  } else if (lane < 32) {
-    r.edge = has_tail && (lane - 16) < tail;
-    r.eoff = head + (body << 4) + (lane - 16);
-  }
-  r.eb = 0;
-  if (r.edge) r.eb = src[r.eoff];
-  const uint8_t *s = src + head;
-  r.d = dst + head;
-  r.p = (uint32_t)(uintptr_t)s & 15u;
-  r.sa = s - r.p;
-  // the chunk after the last stored one is loaded for its neighbour's sake; it
-  // exists (holds bytes of the run) unless the phase is zero and the run ends there
-  r.lim = r.p ? r.c_end : (r.c_end < body ? r.c_end : r.c_end - 1);
-  r.v0 = (u32x4){0, 0, 0, 0};
-  r.v1 = (u32x4){0, 0, 0, 0};
-  if (r.c_begin < r.c_end) {
-    const uint32_t c0 = r.c_begin + lane, c1 = r.c_begin + 63u + lane;
-    if (c0 <= r.lim) r.v0 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c0 << 4));
-    if (c1 <= r.lim) r.v1 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c1 << 4));
-  }
-}
-
-// With CSUM returns this lane's share of the sum of the 16-bit little-endian
-// words the bytes it moved fall into, a byte's position in its word being the
-// parity of its DESTINATION ADDRESS (packet offsets and addresses have the
-// same parity: ring bases, slot sizes and header lengths are even).
-template <bool CSUM>
-__device__ __forceinline__ uint32_t piece_end(PieceState &r, uint32_t lane)
-{
-  uint32_t acc = 0;
-  if (r.c_begin < r.c_end) {
-    const uint32_t c0 = r.c_begin + lane, c1 = r.c_begin + 63u + lane;
-    const u32x4 o0 = realign(r.v0, r.p);
-    const u32x4 o1 = realign(r.v1, r.p);
-    if (lane < 63 && c0 < r.c_end) {
-      store16_aligned(r.d + ((size_t)c0 << 4), o0);
-      if (CSUM) acc += words_sum(o0);
-    }
-    if (lane < 63 && c1 < r.c_end) {
-      store16_aligned(r.d + ((size_t)c1 << 4), o1);
-      if (CSUM) acc += words_sum(o1);
-    }
-  }
-  // what one begin did not cover: four steps (252 chunks) in flight at a time
-  for (uint32_t base = r.c_begin + kPieceChunks; base < r.c_end; base += 2 * kPieceChunks) {
-    u32x4 v[4];
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-      const uint32_t c = base + 63u * k + lane;
-      v[k] = (u32x4){0, 0, 0, 0};
-      if (c <= r.lim) v[k] = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c << 4));
-    }
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-      const uint32_t c = base + 63u * k + lane;
-      const u32x4 q = realign(v[k], r.p);
-      if (lane < 63 && c < r.c_end) {
-        store16_aligned(r.d + ((size_t)c << 4), q);
-        if (CSUM) acc += words_sum(q);
-      }
-    }
-  }
-  if (r.edge) {
-    r.dst[r.eoff] = (uint8_t)r.eb;
-    if (CSUM) acc += ((uintptr_t)(r.dst + r.eoff) & 1u) ? (r.eb << 8) : r.eb;
-  }
-  return acc;
-}
-
-// How many wavefronts a run of at most `max_len` bytes is spread over.
+// How many sub-runs a run of at most `max_len` bytes is cut into.
 __host__ __device__ inline uint32_t pieces_for(uint32_t max_len)
 {
   const uint32_t chunks = (max_len >> 4) + 1;
   return (chunks + kPieceChunks - 1) / kPieceChunks;
+}
+
+// Offset and length of sub-run `piece` of a run of `len` bytes to `dst`;
+// length 0 when the run has no such sub-run.
+__device__ __forceinline__ void sub_run(const uint8_t *dst, uint32_t len, uint32_t piece, uint32_t *off,
+                                        uint32_t *n)
+{
+  uint32_t head = (uint32_t)(-(uintptr_t)dst) & 15u;
+  head = head < len ? head : len;
+  const uint32_t start = piece == 0 ? 0 : head + piece * kPieceBytes;
+  const uint32_t end = head + (piece + 1) * kPieceBytes;
+  *off = start;
+  *n = start >= len ? 0 : (end < len ? end : len) - start;
+}
+
+// Copy a whole long run with one wavefront, two sub-runs in flight at a time.
+template <bool CSUM>
+__device__ __forceinline__ uint32_t copy_long_run(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                  uint32_t len, uint32_t lane)
+{
+  uint32_t acc = 0;
+  for (uint32_t piece = 0;; piece += 2) {
+    uint32_t o0, n0, o1, n1;
+    sub_run(dst, len, piece, &o0, &n0);
+    sub_run(dst, len, piece + 1, &o1, &n1);
+    if (n0 == 0) break;
+    RunState r0, r1;
+    run_begin(r0, src + o0, dst + o0, n0, lane);
+    if (n1) run_begin(r1, src + o1, dst + o1, n1, lane);
+    acc += run_end<CSUM>(r0, lane);
+    if (n1) acc += run_end<CSUM>(r1, lane);
+    else break;
+  }
+  return acc;
 }
 
 // Byte-wise copy into / out of a bump-ring arena that is NOT mirrored, for a

@@ -534,9 +534,9 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   uint8_t *to;
   if (plain_target(a.app, ro, d[3], d[2], d[1], &to)) {
     if (LONG) {
-      PieceState ps;
-      piece_begin(ps, pkt, to, d[1], lane, piece * kPieceChunks, kPieceChunks);
-      piece_end<false>(ps, lane);
+      uint32_t o, n;
+      sub_run(to, d[1], piece, &o, &n);
+      if (n) copy_run<false>(pkt + o, to + o, n, lane);
     } else {
       copy_run<false>(pkt, to, d[1], lane);
     }
@@ -648,16 +648,13 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   }
   // copying the ruled length stays inside the slot whatever the header says
   RunState rs;
-  PieceState ps;
-  if (plain) {
-    if (LONG) piece_begin(ps, pkt + hl, to, len, lane, piece * kPieceChunks, kPieceChunks);
-    else run_begin(rs, pkt + hl, to, len, lane);
-  }
+  uint32_t sub_off = 0, sub_len = len;
+  if (LONG && plain) sub_run(to, len, piece, &sub_off, &sub_len);
+  if (plain && sub_len) run_begin(rs, pkt + hl + sub_off, to + sub_off, sub_len, lane);
   SG_PIN(w0);
   SG_PIN(w1);
   if (plain) {
-    if (LONG) piece_end<false>(ps, lane);
-    else run_end<false>(rs, lane);
+    if (sub_len) run_end<false>(rs, lane);
   } else if (piece == 0) {
     move_run<true, false>(a.app, ro, r, off, pkt + hl, len, lane);
   }
@@ -733,9 +730,9 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     // a later piece of a long frame: payload only
     uint8_t *from;
     if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
-      PieceState ps;
-      piece_begin(ps, from, slot + a.hl, d[1], lane, piece * kPieceChunks, kPieceChunks);
-      piece_end<false>(ps, lane);
+      uint32_t o, n;
+      sub_run(slot + a.hl, d[1], piece, &o, &n);
+      if (n) copy_run<false>(from + o, slot + a.hl + o, n, lane);
     }
     return;
   }
@@ -756,19 +753,18 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   uint8_t *from = nullptr;
   const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
   RunState rs;
-  PieceState ps;
-  // a summed frame stays with one wavefront; a long one then walks all its
-  // chunks with the deeper pipeline of the piece copy
+  // a summed frame stays with one wavefront; a long one is then walked two
+  // sub-runs at a time
   const bool whole_long = FULL_CSUM && a.pieces > 1;
-  if (plain) {
-    if (LONG) piece_begin(ps, from, slot + a.hl, d[1], lane, 0, kPieceChunks);
-    else if (whole_long) piece_begin(ps, from, slot + a.hl, d[1], lane, 0, kWholeRun);
-    else run_begin(rs, from, slot + a.hl, d[1], lane);
+  uint32_t first_len = d[1];
+  if (LONG && plain) {
+    uint32_t o;
+    sub_run(slot + a.hl, d[1], 0, &o, &first_len);
   }
+  if (plain && !whole_long) run_begin(rs, from, slot + a.hl, first_len, lane);
   if (!FULL_CSUM) hb = hdr_finish(raw, lane, hf, 0);
   if (plain) {
-    if (LONG) acc = piece_end<false>(ps, lane);
-    else if (whole_long) acc = piece_end<FULL_CSUM>(ps, lane);
+    if (whole_long) acc = copy_long_run<FULL_CSUM>(from, slot + a.hl, d[1], lane);
     else acc = run_end<FULL_CSUM>(rs, lane);
   } else if (d[1]) {
     acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
