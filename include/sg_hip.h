@@ -169,6 +169,16 @@ typedef struct sg_scatter_args {
   uint32_t flags; /* SG_F_* */
   sg_app_desc app;
   uint64_t *offsets_out; /* device, n_req + 1, or NULL */
+  /* Headers from connection templates instead of from request headers: what
+   * rr_set_hdr does for freshly allocated response buffers
+   * (src/transport/dpdk_transport_ng.h:113-141).  hdr_templates holds one
+   * 64-byte template per request (P2pRpcRr::_client_conn_info.hdr_template,
+   * already pointing at the client: set_conn_info, src/p2p_rpc_conn_info.h:73-84);
+   * frame i of request r gets a copy of template r with token req_token[r]
+   * (the template's own when req_token is NULL), seq_num / frag_idx i,
+   * lengths and sums.  Nothing is swapped and hdr_src_slot is not read. */
+  const uint8_t *hdr_templates; /* device, n_req * 64 bytes, or NULL: swap request headers */
+  const uint64_t *req_token;    /* device, n_req, or NULL */
 } sg_scatter_args;
 
 /* One burst of arrivals to sort into requests on the device.  Replaces the
@@ -227,6 +237,16 @@ int sg_hip_scatter(sg_hip_ctx *ctx, const sg_sk_buf *skb);
  * payload_size.  Synchronous. */
 int sg_hip_swap_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, uint32_t hdr_profile,
                      uint64_t payload_size, uint32_t mtu, uint32_t flags);
+
+/* Replaces rr_set_hdr (src/transport/dpdk_transport_ng.h:113-141): fill the
+ * headers of freshly allocated response buffers from a connection template.
+ * hdr_template is a HOST pointer to the 64 bytes of
+ * p2p_rpc_conn_info::hdr_template (src/p2p_rpc_conn_info.h:21-30); header i
+ * becomes a copy of it with req_token, seq_num / frag_idx i, lengths and the
+ * sums `flags` asks for.  Synchronous. */
+int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_template,
+                    uint64_t req_token, uint32_t hdr_profile, uint64_t payload_size, uint32_t mtu,
+                    uint32_t flags);
 
 /* ---- batched entry points ----------------------------------------------------
  * No counterpart call in the reference (which handles one request per

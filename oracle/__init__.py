@@ -105,7 +105,7 @@ def lib() -> C.CDLL:
         L.sgo_gather_batch.restype = C.c_int64
         L.sgo_scatter_batch.argtypes = [C.POINTER(Ring), C.POINTER(Ring), u32p, u32p, u32p, u64p,
                                         C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32,
-                                        C.POINTER(AppBufs), u64p, u64p]
+                                        C.POINTER(AppBufs), u64p, u64p, u8p, u64p]
         L.sgo_scatter_batch.restype = C.c_int64
         L.sgo_now_sec.restype = C.c_double
         _lib = L
@@ -179,10 +179,13 @@ def gather(w, arena_cap: Optional[int] = None, cursor: int = 0, use_frag_len: bo
 
 
 def scatter(w, rx_ring: np.ndarray, tx_ring: np.ndarray, resp_src, arena_cap: Optional[int] = None,
-            cursor: int = 0, flags: Optional[int] = None, fixed_size: Optional[int] = None):
+            cursor: int = 0, flags: Optional[int] = None, fixed_size: Optional[int] = None,
+            templates: Optional[np.ndarray] = None, tokens: Optional[np.ndarray] = None):
     """Run the CPU scatter composite.  ``tx_ring`` is modified in place (pass
     ``rx_ring`` itself for in-place responses).  ``resp_src`` is the packed
-    arena (uint8 array) or the list of tensor-major output tensors."""
+    arena (uint8 array) or the list of tensor-major output tensors.
+    ``templates`` (n_req x 64 uint8) switches the headers to the template
+    path, with ``tokens`` (n_req uint64) as the request tokens."""
     L = lib()
     rx = _ring(rx_ring, w.n_slots, w.slot_size, w.profile)
     tx = _ring(tx_ring, w.tx_n_slots, w.slot_size, w.profile)
@@ -192,6 +195,9 @@ def scatter(w, rx_ring: np.ndarray, tx_ring: np.ndarray, resp_src, arena_cap: Op
     rs = None if fixed_size is not None else np.ascontiguousarray(w.resp_sizes, dtype=np.uint64)
     cur = np.array([cursor], dtype=np.uint64)
     offs = np.zeros(w.n_req + 1, dtype=np.uint64)
+    tm = None if templates is None else np.ascontiguousarray(templates, dtype=np.uint8)
+    tk = None if tokens is None else np.ascontiguousarray(tokens, dtype=np.uint64)
+    assert tm is None or tm.size == w.n_req * 64
     if w.out_tensor_sizes:
         app = _app(w.out_tensor_sizes, resp_src, None, 0)
     else:
@@ -199,7 +205,8 @@ def scatter(w, rx_ring: np.ndarray, tx_ring: np.ndarray, resp_src, arena_cap: Op
         app = _app([], [], resp_src, cap)
     rc = L.sgo_scatter_batch(C.byref(rx), C.byref(tx), _p(ts), _p(hs), _p(rf), _p(rs),
                              int(fixed_size or 0), w.n_req, w.mtu,
-                             w.flags if flags is None else flags, C.byref(app), _p(cur), _p(offs))
+                             w.flags if flags is None else flags, C.byref(app), _p(cur), _p(offs),
+                             _p(tm), _p(tk))
     assert rc >= 0, "oracle scatter rejected the tables"
     return offs, int(cur[0])
 

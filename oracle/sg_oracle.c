@@ -509,7 +509,8 @@ int64_t sgo_scatter_batch(const sgo_ring *rx, const sgo_ring *tx, const uint32_t
                           const uint32_t *hdr_src_slot, const uint32_t *resp_first,
                           const uint64_t *resp_size, uint64_t fixed_resp_size, uint32_t n_req,
                           uint32_t mtu, uint32_t flags, const sgo_app_bufs *app, uint64_t *cursor,
-                          uint64_t *offsets_out)
+                          uint64_t *offsets_out, const uint8_t *hdr_templates,
+                          const uint64_t *req_token)
 {
   const uint32_t hl = sgo_hdr_len(tx->profile);
   sgo_bufs *bufs = (sgo_bufs *)malloc(sizeof *bufs);
@@ -538,11 +539,18 @@ int64_t sgo_scatter_batch(const sgo_ring *rx, const sgo_ring *tx, const uint32_t
     bufs->num_items = (uint16_t)nf;
     for (uint32_t i = 0; i < nf; i++) {
       uint8_t *slot = tx->base + (uint64_t)tx_slot[f0 + i] * tx->slot_size;
-      const uint8_t *hsrc = rx->base + (uint64_t)hdr_src_slot[f0 + i] * rx->slot_size;
       uint32_t len = sgo_frame_len(size, mtu, i);
       uint8_t h[64];
-      memcpy(h, hsrc, hl);
-      sgo_rewrite_resp_hdr(h, tx->profile, flags, (uint16_t)i, (uint16_t)nf, len);
+      if (hdr_templates) {
+        /* fresh response buffers: rr_set_hdr, transport/dpdk_transport_ng.h:113-141 */
+        const uint8_t *t = hdr_templates + (uint64_t)r * 64;
+        uint64_t tok = req_token ? req_token[r] : rd64(t + 42);
+        sgo_template_resp_hdr(h, t, tx->profile, flags, tok, (uint16_t)i, (uint16_t)nf, len);
+      } else {
+        const uint8_t *hsrc = rx->base + (uint64_t)hdr_src_slot[f0 + i] * rx->slot_size;
+        memcpy(h, hsrc, hl);
+        sgo_rewrite_resp_hdr(h, tx->profile, flags, (uint16_t)i, (uint16_t)nf, len);
+      }
       memcpy(slot, h, hl);
       bufs->burst_items[i] = (uint64_t)(uintptr_t)(slot + hl);
       bufs->item_size[i] = len;

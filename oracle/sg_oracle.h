@@ -174,12 +174,16 @@ int64_t sgo_gather_batch(const sgo_ring *ring, const uint32_t *frag_slot, const 
  * NULL) cut by the fragmenting rule at `mtu`; frame f of the batch goes to
  * tx_slot[f]; its header is rewritten from the request header found in
  * rx ring slot hdr_src_slot[f].  Payload source: packed arena through the
- * bump ring, or tensor-major outputs.  Returns number of frames or -1. */
+ * bump ring, or tensor-major outputs.  With hdr_templates (n_req x 64 bytes)
+ * the header of every frame of response r is built from template r and
+ * req_token[r] instead (rr_set_hdr) and hdr_src_slot is not read.
+ * Returns number of frames or -1. */
 int64_t sgo_scatter_batch(const sgo_ring *rx, const sgo_ring *tx, const uint32_t *tx_slot,
                           const uint32_t *hdr_src_slot, const uint32_t *resp_first,
                           const uint64_t *resp_size, uint64_t fixed_resp_size, uint32_t n_req,
                           uint32_t mtu, uint32_t flags, const sgo_app_bufs *app, uint64_t *cursor,
-                          uint64_t *offsets_out);
+                          uint64_t *offsets_out, const uint8_t *hdr_templates,
+                          const uint64_t *req_token);
 
 /* Single-threaded timing helpers used by the CPU-baseline leg of the
  * benchmark: run the composite `iters` times over `n_rings` rotated copies and

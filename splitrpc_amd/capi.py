@@ -36,7 +36,7 @@ MAX_TENSORS = 4
 # every symbol include/sg_hip.h declares
 SYMBOLS = [
     "sg_hip_create", "sg_hip_destroy", "sg_hip_last_error", "sg_hip_abi_version", "sg_hip_stream",
-    "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_gather_batch",
+    "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_set_hdrs", "sg_hip_gather_batch",
     "sg_hip_scatter_batch", "sg_hip_reassemble", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
     "sg_hip_kernel_time",
 ]
@@ -81,7 +81,7 @@ class ScatterArgs(C.Structure):
                 ("hdr_src_slot", C.c_void_p), ("resp_first", C.c_void_p), ("resp_size", C.c_void_p),
                 ("fixed_resp_size", C.c_uint64), ("n_req", C.c_uint32), ("n_frames", C.c_uint32),
                 ("mtu", C.c_uint32), ("flags", C.c_uint32), ("app", AppDesc),
-                ("offsets_out", C.c_void_p)]
+                ("offsets_out", C.c_void_p), ("hdr_templates", C.c_void_p), ("req_token", C.c_void_p)]
 
 
 class ReassembleArgs(C.Structure):
@@ -121,6 +121,8 @@ def load() -> C.CDLL:
     lib.sg_hip_gather.argtypes = [P, C.POINTER(SkBuf)]
     lib.sg_hip_scatter.argtypes = [P, C.POINTER(SkBuf)]
     lib.sg_hip_swap_hdrs.argtypes = [P, C.POINTER(HBufs), C.c_uint32, C.c_uint64, C.c_uint32, C.c_uint32]
+    lib.sg_hip_set_hdrs.argtypes = [P, C.POINTER(HBufs), C.c_void_p, C.c_uint64, C.c_uint32, C.c_uint64,
+                                    C.c_uint32, C.c_uint32]
     lib.sg_hip_gather_batch.argtypes = [P, C.POINTER(GatherArgs)]
     lib.sg_hip_scatter_batch.argtypes = [P, C.POINTER(ScatterArgs)]
     lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32),

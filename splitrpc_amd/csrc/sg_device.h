@@ -321,6 +321,10 @@ struct HdrFields {
   uint32_t frag_idx;
   uint32_t num_frags;
   uint32_t payload_len;
+  uint32_t from_template;  // bytes come from a connection template: nothing was swapped, and the
+                           // checksum fields keep the template's bytes unless a flag fills them
+  uint32_t set_token;      // write `token` into bytes 42..49
+  uint64_t token;
 };
 
 __device__ __forceinline__ uint32_t hdr_src_index(uint32_t j)
@@ -337,10 +341,11 @@ __device__ __forceinline__ uint32_t hdr_src_index(uint32_t j)
 // The byte lane `lane` starts from: the incoming header's byte at the swapped
 // position.  Split from hdr_finish so that a kernel can have this load in
 // flight together with its payload loads.
-__device__ __forceinline__ uint32_t hdr_fetch(const uint8_t *__restrict__ in, uint32_t lane, uint32_t hl)
+__device__ __forceinline__ uint32_t hdr_fetch(const uint8_t *__restrict__ in, uint32_t lane, uint32_t hl,
+                                              bool swap = true)
 {
   uint32_t b = 0;
-  if (lane < hl) b = in[hdr_src_index(lane)];
+  if (lane < hl) b = in[swap ? hdr_src_index(lane) : lane];
   return b;
 }
 
@@ -359,7 +364,8 @@ __device__ __forceinline__ uint32_t hdr_finish(uint32_t b, uint32_t lane, const 
   if (j == 17) b = tot & 0xffu;
   if (j == 38) b = ulen >> 8;
   if (j == 39) b = ulen & 0xffu;
-  if (j == 24 || j == 25 || j == 40 || j == 41) b = 0;
+  if (!f.from_template && (j == 24 || j == 25 || j == 40 || j == 41)) b = 0;  // swap_eth_hdr zeroes both sums
+  if (f.set_token && j >= 42 && j < 50) b = (uint32_t)(f.token >> (8u * (j - 42u))) & 0xffu;
   if (f.ref64) {
     if (j >= 50 && j < 54) b = 0;                 // sock_perf_header &= 0xFFFFFFFF00000000
     if (j == 58) b = f.frag_idx & 0xffu;
@@ -376,7 +382,7 @@ __device__ __forceinline__ uint32_t hdr_finish(uint32_t b, uint32_t lane, const 
   const uint32_t w = (j & 1u) ? (b << 8) : b;  // contribution to a little-endian word sum
   const uint32_t kAnyCsum = 0x7u;              // IPV4 | PSEUDO | FULL
   if (f.flags & kAnyCsum) {
-    const uint32_t s_ip = wave_sum((j >= 14 && j < 34) ? w : 0u);
+    const uint32_t s_ip = wave_sum((j >= 14 && j < 34 && j != 24 && j != 25) ? w : 0u);
     const uint32_t s_addr = wave_sum((j >= 26 && j < 34) ? w : 0u);
     const uint32_t b14 = __shfl(b, 14, 64);
     const uint32_t proto = __shfl(b, 23, 64);

@@ -674,6 +674,8 @@ struct ScatterArgs {
   const uint64_t *req_off;
   const uint32_t *first;         // resp_first CSR (for frag_idx / num_frags)
   const uint32_t *hdr_src_slot;
+  const uint8_t *hdr_templates;  // non-null: headers from per-request templates, nothing swapped
+  const uint64_t *req_token;
   const uint8_t *rx;
   uint32_t rx_slot_size;
   uint32_t rx_n_slots;
@@ -736,19 +738,29 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     }
     return;
   }
-  uint32_t hs = a.hdr_src_slot[item];
-  if (hs >= a.rx_n_slots) {
-    if (lane == 0) atomicOr(a.status, kStBadSlot);
-    return;
+  const bool from_template = a.hdr_templates != nullptr;
+  const uint8_t *hin;
+  HdrFields hf{a.hl, a.ref64, a.flags, item - f0, nf, d[1], 0, 0, 0};
+  if (from_template) {
+    hin = a.hdr_templates + (size_t)r * 64;
+    hf.from_template = 1;
+    if (a.req_token) {
+      hf.set_token = 1;
+      hf.token = a.req_token[r];
+    }
+  } else {
+    const uint32_t hs = a.hdr_src_slot[item];
+    if (hs >= a.rx_n_slots) {
+      if (lane == 0) atomicOr(a.status, kStBadSlot);
+      return;
+    }
+    // read the request header before anything of this slot is overwritten
+    // (the TX slot may be the very slot the header comes from)
+    hin = a.rx + (size_t)hs * a.rx_slot_size;
   }
-
-  // read the request header before anything of this slot is overwritten
-  // (the TX slot may be the very slot the header comes from)
-  const uint8_t *hin = a.rx + (size_t)hs * a.rx_slot_size;
-  HdrFields hf{a.hl, a.ref64, a.flags, item - f0, nf, d[1]};
   // header bytes and payload chunks are fetched together; the header arithmetic
   // then runs while the payload is still on its way
-  const uint32_t raw = hdr_fetch(hin, lane, a.hl);
+  const uint32_t raw = hdr_fetch(hin, lane, a.hl, !from_template);
   uint32_t hb = 0, acc = 0;
   uint8_t *from = nullptr;
   const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
@@ -795,9 +807,13 @@ __global__ __launch_bounds__(kBlock) void k_copy_runs(const Run *runs, uint32_t 
                   (uint32_t)r.len, lane);
 }
 
+// tmpl == nullptr: swap each header in place; else every header is a copy of
+// the 64-byte template with `token` in it (the two ways the reference fills
+// response headers: rr_swap_hdr and rr_set_hdr).
 __global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, uint32_t n,
                                                       uint32_t hl, uint32_t ref64, uint32_t flags,
-                                                      uint64_t payload_size, uint32_t mtu)
+                                                      uint64_t payload_size, uint32_t mtu,
+                                                      const uint8_t *tmpl, uint64_t token)
 {
   const uint32_t item = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (item >= n) return;
@@ -805,8 +821,9 @@ __global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, 
   uint8_t *h = reinterpret_cast<uint8_t *>(hdr_ptrs[item]);
   const uint64_t taken = (uint64_t)item * mtu;
   const uint64_t rem = taken < payload_size ? payload_size - taken : 0;
-  HdrFields hf{hl, ref64, flags & ~(1u << 2), item, n, (uint32_t)(rem <= mtu ? rem : mtu)};
-  const uint32_t b = hdr_rewrite(h, lane, hf, 0);
+  HdrFields hf{hl, ref64, flags & ~(1u << 2), item, n, (uint32_t)(rem <= mtu ? rem : mtu),
+               tmpl != nullptr, tmpl != nullptr, token};
+  const uint32_t b = hdr_finish(hdr_fetch(tmpl ? tmpl : h, lane, hl, tmpl == nullptr), lane, hf, 0);
   if (lane < hl) h[lane] = (uint8_t)b;
 }
 
@@ -1263,7 +1280,7 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
   c->h_runs_cap = 8192;
   HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
-  HIP_TRY(nullptr, hipHostMalloc(&c->h_ptrs, sizeof(uint64_t) * SG_MAX_BI_SIZE, hipHostMallocDefault));
+  HIP_TRY(nullptr, hipHostMalloc(&c->h_ptrs, sizeof(uint64_t) * (SG_MAX_BI_SIZE + 8), hipHostMallocDefault));
   HIP_TRY(nullptr, hipHostMalloc(&c->h_status, sizeof(uint32_t), hipHostMallocDefault));
   HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
   return SG_OK;
@@ -1420,8 +1437,8 @@ static int copy_skb(sg_hip_ctx *c, const sg_sk_buf *skb)
 int sg_hip_gather(sg_hip_ctx *c, const sg_sk_buf *skb) { return copy_skb(c, skb); }
 int sg_hip_scatter(sg_hip_ctx *c, const sg_sk_buf *skb) { return copy_skb(c, skb); }
 
-int sg_hip_swap_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, uint32_t profile, uint64_t payload_size,
-                     uint32_t mtu, uint32_t flags)
+static int fill_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, const uint8_t *tmpl, uint64_t token,
+                     uint32_t profile, uint64_t payload_size, uint32_t mtu, uint32_t flags)
 {
   if (!c || !hdrs) return fail(c, SG_E_INVAL, "null argument");
   if (profile > SG_HDR_REF64) return fail(c, SG_E_INVAL, "unknown header profile %u", profile);
@@ -1436,13 +1453,33 @@ int sg_hip_swap_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, uint32_t profile, uint
     if (!hdrs->burst_items[i]) return fail(c, SG_E_INVAL, "header %u is null", i);
     c->h_ptrs[i] = hdrs->burst_items[i];
   }
+  // the template rides behind the pointer table in the same pinned block
+  const uint8_t *d_tmpl = nullptr;
+  if (tmpl) {
+    memcpy(c->h_ptrs + SG_MAX_BI_SIZE, tmpl, 64);
+    d_tmpl = reinterpret_cast<const uint8_t *>(c->h_ptrs + SG_MAX_BI_SIZE);
+  }
   int rc = prof_begin(c, 4);
   if (rc != SG_OK) return rc;
   k_swap_hdrs<<<(n + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(
-      c->h_ptrs, n, hdr_len_of(profile), profile == SG_HDR_REF64, flags & 0xfu, payload_size, mtu);
+      c->h_ptrs, n, hdr_len_of(profile), profile == SG_HDR_REF64, flags & 0xfu, payload_size, mtu,
+      d_tmpl, token);
   rc = prof_end(c);
   if (rc != SG_OK) return rc;
   return finish(c, 0);
+}
+
+int sg_hip_swap_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, uint32_t profile, uint64_t payload_size,
+                     uint32_t mtu, uint32_t flags)
+{
+  return fill_hdrs(c, hdrs, nullptr, 0, profile, payload_size, mtu, flags);
+}
+
+int sg_hip_set_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, const uint8_t *hdr_template, uint64_t req_token,
+                    uint32_t profile, uint64_t payload_size, uint32_t mtu, uint32_t flags)
+{
+  if (!hdr_template) return fail(c, SG_E_INVAL, "null header template");
+  return fill_hdrs(c, hdrs, hdr_template, req_token, profile, payload_size, mtu, flags);
 }
 
 // ---- batched ------------------------------------------------------------------
@@ -1573,7 +1610,8 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   if (a->n_req == 0) return SG_OK;
   if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
   if (a->n_frames > c->max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u of this context", a->n_frames, c->max_frames);
-  if (!a->tx_slot || !a->hdr_src_slot || !a->resp_first) return fail(c, SG_E_INVAL, "null frame tables");
+  if (!a->tx_slot || !a->resp_first || (!a->hdr_src_slot && !a->hdr_templates))
+    return fail(c, SG_E_INVAL, "null frame tables");
   const uint32_t hl = hdr_len_of(a->tx.hdr_profile);
   if (a->mtu == 0 || (uint64_t)a->mtu + hl > a->tx.slot_size)
     return fail(c, SG_E_INVAL, "mtu %u + %u header bytes does not fit a %u-byte slot", a->mtu, hl, a->tx.slot_size);
@@ -1595,6 +1633,8 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     ScatterArgs sa;
     memset(&sa, 0, sizeof sa);
     sa.hdr_src_slot = a->hdr_src_slot;
+    sa.hdr_templates = a->hdr_templates;
+    sa.req_token = a->req_token;
     sa.rx = static_cast<const uint8_t *>(a->rx.base);
     sa.rx_slot_size = a->rx.slot_size;
     sa.rx_n_slots = a->rx.n_slots;
@@ -1667,6 +1707,8 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.req_off = c->req_off;
     sa.first = a->resp_first;
     sa.hdr_src_slot = a->hdr_src_slot;
+    sa.hdr_templates = a->hdr_templates;
+    sa.req_token = a->req_token;
     sa.rx = static_cast<const uint8_t *>(a->rx.base);
     sa.rx_slot_size = a->rx.slot_size;
     sa.rx_n_slots = a->rx.n_slots;

@@ -154,7 +154,9 @@ class SgContext:
                      hdr_src_slot: torch.Tensor, resp_first: torch.Tensor,
                      resp_size: Optional[torch.Tensor], fixed_resp_size: int, n_req: int,
                      n_frames: int, mtu: int, app: AppRef,
-                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0) -> capi.ScatterArgs:
+                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0,
+                     hdr_templates: Optional[torch.Tensor] = None,
+                     req_token: Optional[torch.Tensor] = None) -> capi.ScatterArgs:
         a = capi.ScatterArgs()
         a.rx = rx.desc()
         a.tx = tx.desc()
@@ -169,6 +171,8 @@ class SgContext:
         a.flags = flags
         a.app = app.desc()
         a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
+        a.hdr_templates = hdr_templates.data_ptr() if hdr_templates is not None else None
+        a.req_token = req_token.data_ptr() if req_token is not None else None
         return a
 
     def scatter_batch(self, *args, **kw) -> None:
@@ -220,6 +224,16 @@ class SgContext:
             hb.burst_items[i] = p
         hb.num_items = len(hdr_ptrs)
         self._check(self.lib.sg_hip_swap_hdrs(self.h, C.byref(hb), profile, payload_size, mtu, flags))
+
+    def set_hdrs(self, hdr_ptrs: Sequence[int], template: bytes, token: int, profile: int,
+                 payload_size: int, mtu: int, flags: int) -> None:
+        hb = capi.HBufs()
+        for i, p in enumerate(hdr_ptrs):
+            hb.burst_items[i] = p
+        hb.num_items = len(hdr_ptrs)
+        assert len(template) >= 64
+        t = (C.c_uint8 * 64).from_buffer_copy(bytes(template[:64]))
+        self._check(self.lib.sg_hip_set_hdrs(self.h, C.byref(hb), t, token, profile, payload_size, mtu, flags))
 
 
 class DeviceWorkload:
@@ -335,17 +349,23 @@ class DeviceWorkload:
         a.flags = flags | a._base_flags
         ctx.gather_batch_raw(a)
 
-    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True) -> None:
+    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True,
+                templates: Optional[torch.Tensor] = None, tokens: Optional[torch.Tensor] = None) -> None:
+        """``templates`` (n_req x 64 uint8 on the device) takes the frame
+        headers from connection templates instead of request headers."""
         if not fuse:
             flags |= capi.F_NO_FUSE
         key = ("s", fixed)
         a = self._args.get(key)
+        if a is not None:
+            a.hdr_templates = templates.data_ptr() if templates is not None else None
+            a.req_token = tokens.data_ptr() if tokens is not None else None
         if a is None:
             sizes = self.w.resp_sizes
             fx = int(sizes[0]) if fixed and len(sizes) and bool((sizes == sizes[0]).all()) else 0
             a = ctx.scatter_args(self.rx, self.tx, self.tx_slot, self.hdr_src_slot, self.resp_first,
                                  None if fx else self.resp_size, fx, self.n_req, self.n_frames,
-                                 self.w.mtu, self.resp_app, self.resp_offsets, 0)
+                                 self.w.mtu, self.resp_app, self.resp_offsets, 0, templates, tokens)
             self._args[key] = a
         a.flags = self.w.flags | flags
         ctx.scatter_batch_raw(a)

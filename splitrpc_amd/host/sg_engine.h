@@ -194,6 +194,17 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
     if (last_rc != SG_OK) fail("swap_hdrs", last_rc);
   }
 
+  // Headers of a freshly allocated response from the connection template
+  // (rr_set_hdr, src/transport/dpdk_transport_ng.h:113-141), written on the GPU.
+  inline void set_hdrs(const p2p_rpc_conn_info *conn, P2pRpcRr *rpc_rr, uint32_t hdr_profile, size_t payload_size,
+                       uint32_t mtu, uint32_t flags)
+  {
+    last_rc = sg_hip_set_hdrs(ctx, reinterpret_cast<const sg_hbufs *>(rpc_rr->hdr_bufs),
+                              reinterpret_cast<const uint8_t *>(&conn->hdr_template), rpc_rr->req_token,
+                              hdr_profile, payload_size, mtu, flags);
+    if (last_rc != SG_OK) fail("set_hdrs", last_rc);
+  }
+
   // ---- batched: every ready request in one call ----
   // Gathers n requests whose payload pointers lie in `ring` into `app`
   // (consecutive bump-ring positions or tensor-major buffers), in the order

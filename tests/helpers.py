@@ -9,7 +9,7 @@ def expected_gather(w, arena_cap=None, cursor=0):
     return oracle.gather(w, arena_cap=arena_cap, cursor=cursor)
 
 
-def expected_scatter(w, gathered, resp_cap=None, cursor=0, flags=None):
+def expected_scatter(w, gathered, resp_cap=None, cursor=0, flags=None, templates=None, tokens=None):
     """Returns the TX ring bytes after the oracle's scatter (+ offsets, cursor)."""
     if w.tx_in_place:
         tx = w.ring.copy()
@@ -31,7 +31,8 @@ def expected_scatter(w, gathered, resp_cap=None, cursor=0, flags=None):
             src = w.resp_payload if w.resp_payload.size >= 16 else np.concatenate(
                 [w.resp_payload, np.zeros(16 - w.resp_payload.size, np.uint8)])
             cap = max(int(w.resp_payload.size), 16) if resp_cap is None else resp_cap
-    offs, cur = oracle.scatter(w, rx, tx, src, arena_cap=cap, cursor=cursor, flags=flags)
+    offs, cur = oracle.scatter(w, rx, tx, src, arena_cap=cap, cursor=cursor, flags=flags,
+                              templates=templates, tokens=tokens)
     return tx, offs, cur
 
 
@@ -43,3 +44,29 @@ def first_diff(a: np.ndarray, b: np.ndarray) -> str:
         return "equal"
     i = int(idx[0])
     return f"{idx.size} bytes differ, first at {i}: got {a[i]} want {b[i]}"
+
+
+def conn_templates(w, seed=0):
+    """Per-request connection templates the way the reference builds them: a
+    server-side template (gen_*_header_template) pointed at the client by
+    set_conn_info with the request's first packet.  Returns (n_req x 64 uint8,
+    n_req uint64 tokens read from those packets)."""
+    import ctypes as C
+    L = oracle.lib()
+    rng = np.random.default_rng(seed)
+    pp = lambda a: a.ctypes.data_as(C.c_void_p)
+    tm = np.zeros((w.n_req, 64), np.uint8)
+    tk = np.zeros(w.n_req, np.uint64)
+    for r in range(w.n_req):
+        if w.req_first[r + 1] == w.req_first[r]:
+            continue
+        slot = int(w.frag_slot[w.req_first[r]])
+        recv = np.ascontiguousarray(w.ring[slot * w.slot_size: slot * w.slot_size + 64])
+        sm, dm = rng.integers(0, 256, 6, dtype=np.uint8), rng.integers(0, 256, 6, dtype=np.uint8)
+        t = np.zeros(64, np.uint8)
+        L.sgo_gen_hdr_template(pp(t), pp(sm), pp(dm), int(rng.integers(0, 2 ** 32)), int(rng.integers(0, 2 ** 32)),
+                               int(rng.integers(0, 65536)), int(rng.integers(0, 65536)))
+        L.sgo_set_conn_info(pp(t), pp(recv), w.profile)
+        tm[r] = t
+        tk[r] = recv[42:50].view(np.uint64)[0]
+    return tm, tk

@@ -12,7 +12,7 @@ import oracle
 from splitrpc_amd import capi, synth
 from splitrpc_amd.engine import AppRef, DeviceWorkload, RingRef, SgContext, SgError, to_dev
 
-from helpers import expected_gather, expected_scatter, first_diff
+from helpers import conn_templates, expected_gather, expected_scatter, first_diff
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -95,6 +95,33 @@ def test_swap_hdrs_in_place(ctx, profile, flags):
     assert np.array_equal(got, want), first_diff(got.reshape(-1), want.reshape(-1))
 
 
+@pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64])
+@pytest.mark.parametrize("flags", [0, synth.F_UDP_CSUM_PSEUDO | synth.F_REF_QUIRKS,
+                                   synth.F_IPV4_CSUM | synth.F_UDP_CSUM_PSEUDO])
+def test_set_hdrs_from_template(ctx, profile, flags):
+    """sg_hip_set_hdrs against the oracle's rr_set_hdr."""
+    rng = np.random.default_rng(300 + flags)
+    n, slot = 23, 128
+    hl = synth.hdr_len(profile)
+    buf = rng.integers(0, 256, n * slot, dtype=np.uint8)
+    tmpl = rng.integers(0, 256, 64, dtype=np.uint8)
+    tmpl[14] = 0x45
+    token = 0x0123456789abcdef
+    dev = dev_u8(buf)
+    payload_size, mtu = 22 * 1400 + 1, 1400
+    ctx.set_hdrs([dev.data_ptr() + i * slot for i in range(n)], tmpl.tobytes(), token, profile,
+                 payload_size, mtu, flags)
+    want = buf.copy().reshape(n, slot)
+    L = oracle.lib()
+    for i in range(n):
+        h = np.zeros(64, np.uint8)
+        L.sgo_template_resp_hdr(h.ctypes.data_as(C.c_void_p), tmpl.ctypes.data_as(C.c_void_p), profile, flags,
+                                token, i, n, L.sgo_frame_len(payload_size, mtu, i))
+        want[i, :hl] = h[:hl]
+    got = dev.cpu().numpy().reshape(n, slot)
+    assert np.array_equal(got, want), first_diff(got.reshape(-1), want.reshape(-1))
+
+
 # ---------------------------------------------------------------- header profiles, flags
 
 @pytest.mark.parametrize("cfg,n", [(1, 9), (2, 2), (5, 1)])
@@ -114,6 +141,35 @@ def test_ref64_profile(ctx, cfg, n, extra):
     exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
     got = dw.tx_ring.cpu().numpy()
     assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
+
+
+@pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64])
+@pytest.mark.parametrize("flags", [0, synth.F_UDP_CSUM_PSEUDO | synth.F_REF_QUIRKS,
+                                   synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL])
+@pytest.mark.parametrize("with_tokens", [True, False])
+def test_headers_from_connection_templates(ctx, profile, flags, with_tokens):
+    """Fresh response buffers: headers copied from per-request templates."""
+    w = synth.make_custom([5000, 77, 1400, 0, 1401, 60000], [3000, 1, 1400, 0, 2801, 4200], seed=77,
+                          flags=flags, profile=profile)
+    print(f"case templates profile={profile} flags={flags} tokens={with_tokens}", flush=True)
+    dw = DeviceWorkload(w)
+    tm, tk = conn_templates(w, seed=5)
+    if with_tokens:
+        tk = tk ^ np.uint64(0x5a5a00000000a5a5)   # tokens that differ from the templates' own
+    d_tm = to_dev(tm.reshape(-1), "cuda")
+    d_tk = to_dev(tk, "cuda") if with_tokens else None
+    ctx.set_cursor(0, 0)
+    dw.gather(ctx, use_frag_len=profile == synth.HDR_REF64)
+    exp, _, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    for fuse in (True, False):
+        for fixed in (False,):
+            ctx.set_cursor(1, 0)
+            dw.tx_ring.copy_(to_dev(w.ring if w.tx_in_place else w.tx_ring_init, "cuda"))
+            dw.scatter(ctx, fuse=fuse, fixed=fixed, templates=d_tm, tokens=d_tk)
+            exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap, templates=tm,
+                                            tokens=tk if with_tokens else None)
+            got = dw.tx_ring.cpu().numpy()
+            assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
 
 
 def test_ref64_without_length_table_is_refused(ctx):

@@ -185,6 +185,37 @@ def test_sockperf_and_conn_info():
         assert np.array_equal(tmpl[same], t0[same])
 
 
+@pytest.mark.parametrize("prof,hl", [(synth.HDR_BL58, 58), (synth.HDR_REF64, 64)])
+def test_template_header_equals_swapped_header_on_one_connection(prof, hl):
+    """rr_set_hdr (template copy) and rr_swap_hdr (in-place swap) are two ways
+    to the same response header: when the server's template carries the
+    identity the request was sent to, they must agree byte for byte.  A wrong
+    offset in either path, or in set_conn_info, breaks the equality."""
+    rng = np.random.default_rng(31)
+    for it in range(40):
+        cm, sm = rng.integers(0, 256, 6, dtype=np.uint8), rng.integers(0, 256, 6, dtype=np.uint8)
+        cip, sip = int(rng.integers(0, 2 ** 32)), int(rng.integers(0, 2 ** 32))
+        cp, sp = int(rng.integers(0, 65536)), int(rng.integers(0, 65536))
+        req = np.zeros(64, np.uint8)
+        L.sgo_gen_hdr_template(p(req), p(cm), p(sm), cip, sip, cp, sp)       # client -> server
+        req[42:64] = rng.integers(0, 256, 22, dtype=np.uint8)
+        tmpl = np.zeros(64, np.uint8)
+        other = rng.integers(0, 256, 6, dtype=np.uint8)
+        L.sgo_gen_hdr_template(p(tmpl), p(sm), p(other), sip, 0x01020304, sp, 9)  # server -> nobody yet
+        L.sgo_set_conn_info(p(tmpl), p(req), prof)
+        token = int(req[42:50].view(np.uint64)[0])
+        for flags in (0, 1, 2, 3, 10):
+            for idx, n, plen in ((0, 1, 1), (3, 7, 1400), (1022, 1023, 777)):
+                a, b = req.copy(), np.zeros(64, np.uint8)
+                L.sgo_rewrite_resp_hdr(p(a), prof, flags, idx, n, plen)
+                L.sgo_template_resp_hdr(p(b), p(tmpl), prof, flags, token, idx, n, plen)
+                assert np.array_equal(a[:hl], b[:hl]), (it, flags, idx, np.flatnonzero(a[:hl] != b[:hl]))
+        # and the token argument really lands in bytes 42..49
+        b = np.zeros(64, np.uint8)
+        L.sgo_template_resp_hdr(p(b), p(tmpl), prof, 0, 0x1122334455667788, 0, 1, 5)
+        assert bytes(b[42:50]) == (0x1122334455667788).to_bytes(8, "little")
+
+
 @needs_ref
 def test_header_template_matches_compiled_reference():
     rng = np.random.default_rng(2)
