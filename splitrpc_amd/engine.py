@@ -59,6 +59,7 @@ class AppRef:
     mirrored: bool = False
     tensors: Sequence[torch.Tensor] = ()
     sizes: Sequence[int] = ()
+    arena_ptr: int = 0   # raw device address instead of ``arena`` (memory torch does not own)
 
     def desc(self) -> capi.AppDesc:
         d = capi.AppDesc()
@@ -68,6 +69,9 @@ class AppRef:
             d.tensor_size[i] = int(s)
         if self.arena is not None:
             d.arena = self.arena.data_ptr()
+            d.arena_cap = int(self.cap)
+        elif self.arena_ptr:
+            d.arena = self.arena_ptr
             d.arena_cap = int(self.cap)
         d.arena_mirrored = 1 if self.mirrored else 0
         return d

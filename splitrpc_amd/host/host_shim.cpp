@@ -298,4 +298,22 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
   return done;
 }
 
+// A double-mapped arena for callers outside C++ (the tests): the request
+// range of a P2pRpcAppRrMemPool.  Returns a handle, or NULL.
+void *sgh_mempool_create(int device_id, int n, uint64_t req_size, uint64_t resp_size, int want_mirror)
+{
+  if (hipSetDevice(device_id) != hipSuccess) return nullptr;
+  try {
+    return new P2pRpcAppRrMemPool(n, device_id, req_size, resp_size, want_mirror != 0);
+  } catch (...) {
+    return nullptr;
+  }
+}
+void sgh_mempool_destroy(void *p) { delete static_cast<P2pRpcAppRrMemPool *>(p); }
+int sgh_mempool_mirrored(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->mirrored() ? 1 : 0; }
+void *sgh_mempool_req_base(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_req_addr_range(); }
+uint64_t sgh_mempool_req_bytes(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_req_addr_pool_size(); }
+void *sgh_mempool_resp_base(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_resp_addr_range(); }
+uint64_t sgh_mempool_resp_bytes(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_resp_addr_pool_size(); }
+
 }  // extern "C"

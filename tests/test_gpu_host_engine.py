@@ -24,6 +24,16 @@ def host():
                                 C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32, C.c_int, C.c_int,
                                 C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.POINTER(C.c_int)]
+    h.sgh_mempool_create.restype = C.c_void_p
+    h.sgh_mempool_create.argtypes = [C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_int]
+    h.sgh_mempool_destroy.argtypes = [C.c_void_p]
+    h.sgh_mempool_mirrored.argtypes = [C.c_void_p]
+    for f in ("req_base", "resp_base"):
+        getattr(h, "sgh_mempool_" + f).restype = C.c_void_p
+        getattr(h, "sgh_mempool_" + f).argtypes = [C.c_void_p]
+    for f in ("req_bytes", "resp_bytes"):
+        getattr(h, "sgh_mempool_" + f).restype = C.c_uint64
+        getattr(h, "sgh_mempool_" + f).argtypes = [C.c_void_p]
     return h
 
 
@@ -59,3 +69,73 @@ def test_one_burst_of_the_shunter(host, cfg, n, profile, mirror, per_request):
     exp_tx = w.tx_ring_init.copy()
     oracle.scatter(w, w.ring, exp_tx, w.resp_payload, flags=flags)
     assert np.array_equal(tx, exp_tx), first_diff(tx, exp_tx)
+
+
+@pytest.mark.parametrize("mode", ["scan", "rule"])
+def test_batch_across_the_end_of_a_double_mapped_arena(host, ctx, mode):
+    """The request and response arenas of P2pRpcAppRrMemPool are mapped twice
+    back to back (the reference's VMM trick, src/p2p_rpc_app_rr.h:60-143), so a
+    request that crosses the end of the ring is written and read linearly.
+    The oracle wraps byte by byte; both must leave the same bytes."""
+    import torch
+    from splitrpc_amd import capi
+    from splitrpc_amd.engine import AppRef, DeviceWorkload
+    from helpers import expected_scatter
+    rule = mode == "rule"
+    sizes = [70000] * 6 if rule else [70000, 1, 123457, 8, 99999, 70001]
+    resp = [50000] * 6 if rule else [1, 50000, 77, 140001, 4200, 1399]
+    w = synth.make_custom(sizes, resp, seed=21, flags=synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL)
+    dw = DeviceWorkload(w)
+    pool = host.sgh_mempool_create(0, 1, 1 << 21, 1 << 21, 1)
+    assert pool
+    try:
+        assert host.sgh_mempool_mirrored(pool) == 1, "HIP virtual memory management is expected on this GPU"
+        cap = int(host.sgh_mempool_req_bytes(pool))
+        rcap = int(host.sgh_mempool_resp_bytes(pool))
+        req_base, resp_base = host.sgh_mempool_req_base(pool), host.sgh_mempool_resp_base(pool)
+        assert cap == 1 << 21 and rcap == 1 << 21
+        print(f"case mirrored mode={mode} cap={cap}", flush=True)
+        app = AppRef(arena_ptr=req_base, cap=cap, mirrored=True)
+        rapp = AppRef(arena_ptr=resp_base, cap=rcap, mirrored=True)
+        stage = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()   # the context launches on its own stream
+        ctx.copy_runs([stage.data_ptr()], [req_base], [cap])           # clear the arena
+        start = cap - 100000                                           # the second request crosses the end
+        ctx.set_cursor(0, start)
+        offs = torch.zeros(w.n_req + 1, dtype=torch.int64, device="cuda")
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, app, offs,
+                         flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if rule else 0, mtu=w.mtu)
+        exp, eoffs, ecur = oracle.gather(w, arena_cap=cap, cursor=start)
+        ctx.copy_runs([req_base], [stage.data_ptr()], [cap])
+        got = stage.cpu().numpy()
+        assert np.array_equal(got, exp), first_diff(got, exp)
+        assert np.array_equal(offs.cpu().numpy().view(np.uint64), eoffs)
+        assert ctx.get_cursor(0) == ecur
+        # the second mapping shows the same bytes
+        ctx.copy_runs([req_base + cap], [stage.data_ptr()], [cap])
+        assert np.array_equal(stage.cpu().numpy(), exp)
+
+        # responses: lay them out in the response arena the way the oracle's bump ring does
+        rstart = rcap - 60000
+        resp_arena = np.zeros(rcap, np.uint8)
+        pos = rstart
+        for r in range(w.n_req):
+            n = int(w.resp_sizes[r])
+            src = w.resp_payload[sum(int(x) for x in w.resp_sizes[:r]):][:n]
+            idx = (pos + np.arange(n)) % rcap
+            resp_arena[idx] = src
+            pos = (pos + n) % rcap
+        stage.copy_(torch.from_numpy(resp_arena).cuda())
+        torch.cuda.synchronize()
+        ctx.copy_runs([stage.data_ptr()], [resp_base], [rcap])
+        ctx.set_cursor(1, rstart)
+        sz = None if rule else dw.resp_size
+        ctx.scatter_batch(dw.rx, dw.tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first, sz, resp[0] if rule else 0,
+                          dw.n_req, dw.n_frames, w.mtu, rapp, None, w.flags)
+        tx = w.tx_ring_init.copy()
+        oracle.scatter(w, w.ring, tx, resp_arena, arena_cap=rcap, cursor=rstart,
+                       fixed_size=resp[0] if rule else None)
+        got = dw.tx_ring.cpu().numpy()
+        assert np.array_equal(got, tx), first_diff(got, tx)
+    finally:
+        host.sgh_mempool_destroy(pool)
