@@ -883,52 +883,100 @@ __device__ __forceinline__ uint32_t ra_hash(unsigned long long k)
   return (uint32_t)k;
 }
 
+// Find or claim the hash cell of `token`: linear probing from its hash; a plain
+// read first, since nearly every arrival finds its request already present.
+__device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long long token)
+{
+  uint32_t c = ra_hash(token) & a.hmask;
+  for (uint32_t probe = 0; probe <= a.hmask; probe++) {
+    unsigned long long old = __hip_atomic_load(&a.keys[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == 0ull) old = atomicCAS(&a.keys[c], 0ull, token);
+    if (old == 0ull || old == token) return c;
+    c = (c + 1) & a.hmask;
+  }
+  return kRaNoCell;
+}
+
+// Fragments of one request tend to arrive together, so the lanes of a
+// wavefront are first grouped by token: a group's first lane looks the cell up
+// once and adds the group's fragment count, bytes and last position in one
+// atomic each.  After kRaRounds groups the lanes still waiting go one by one
+// (bursts that interleave many requests).
+constexpr int kRaRounds = 4;
+
 __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
 {
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= a.n) return;
-  const uint32_t slot = a.arrivals[i];
-  uint32_t cell = kRaNoCell, len = 0, fidx = 0;
-  if (slot >= a.n_slots) {
-    atomicOr(a.status, kStBadSlot);
-  } else {
-    const uint8_t *h = a.ring + (size_t)slot * a.slot_size;
-    const uint32_t t0 = load32_any(h + 42), t1 = load32_any(h + 46);
-    const unsigned long long token = ((unsigned long long)t1 << 32) | t0;
-    uint32_t want = 0;
-    if (a.ref64) {
-      fidx = load32_any(h + 58) & 0xffffu;
-      len = a.len_nic[slot];
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const bool in_range = i < a.n;
+  uint32_t cell = kRaNoCell, len = 0, fidx = 0, want = 0;
+  unsigned long long token = 0;
+  bool pending = false;
+  if (in_range) {
+    const uint32_t slot = a.arrivals[i];
+    if (slot >= a.n_slots) {
+      atomicOr(a.status, kStBadSlot);
     } else {
-      const uint32_t w = load32_any(h + 50);
-      fidx = w & 0xffffu;
-      want = w >> 16;
-      len = a.len_nic ? a.len_nic[slot] : load32_any(h + 54);
-    }
-    const uint32_t hl = a.ref64 ? 64u : 58u;
-    if (len > a.slot_size - hl) {
-      atomicOr(a.status, kStBadLen);
-    } else if (token != 0) {  // token 0: dropped (src/transport/dpdk_transport_ng.h:231)
-      uint32_t c = ra_hash(token) & a.hmask;
-      for (uint32_t probe = 0; probe <= a.hmask; probe++) {
-        const unsigned long long old = atomicCAS(&a.keys[c], 0ull, token);
-        if (old == 0ull || old == token) {
-          cell = c;
-          break;
-        }
-        c = (c + 1) & a.hmask;
+      const uint8_t *h = a.ring + (size_t)slot * a.slot_size;
+      const uint32_t t0 = load32_any(h + 42), t1 = load32_any(h + 46);
+      token = ((unsigned long long)t1 << 32) | t0;
+      if (a.ref64) {
+        fidx = load32_any(h + 58) & 0xffffu;
+        len = a.len_nic[slot];
+      } else {
+        const uint32_t w = load32_any(h + 50);
+        fidx = w & 0xffffu;
+        want = w >> 16;
+        len = a.len_nic ? a.len_nic[slot] : load32_any(h + 54);
       }
-      if (cell != kRaNoCell) {
-        atomicAdd(&a.cnt[cell], 1u);
-        atomicAdd(&a.bytes[cell], (unsigned long long)len);
-        atomicMax(&a.last[cell], i);
-        if (!a.ref64) a.want[cell] = want;  // every fragment of a request says the same
+      const uint32_t hl = a.ref64 ? 64u : 58u;
+      if (len > a.slot_size - hl) {
+        atomicOr(a.status, kStBadLen);
+        len = 0;
+      } else {
+        pending = token != 0;  // token 0: dropped (src/transport/dpdk_transport_ng.h:231)
       }
     }
   }
-  a.arr_cell[i] = cell;
-  a.arr_len[i] = len;
-  a.arr_fidx[i] = fidx;
+  for (int round = 0; round < kRaRounds; round++) {
+    const unsigned long long waiting = __ballot(pending);
+    if (!waiting) break;
+    const int first = __ffsll((long long)waiting) - 1;
+    const unsigned long long t = ((unsigned long long)(uint32_t)__shfl((int)(token >> 32), first, kWave) << 32) |
+                                 (uint32_t)__shfl((int)(uint32_t)token, first, kWave);
+    const bool mine = pending && token == t;
+    const unsigned long long group = __ballot(mine);
+    const uint32_t g_bytes = wave_sum(mine ? len : 0u);
+    uint32_t c = kRaNoCell;
+    if ((int)lane == first) {
+      c = ra_find_cell(a, t);
+      if (c != kRaNoCell) {
+        atomicAdd(&a.cnt[c], (uint32_t)__popcll(group));
+        atomicAdd(&a.bytes[c], (unsigned long long)g_bytes);
+        atomicMax(&a.last[c], i - lane + (63u - (uint32_t)__clzll((long long)group)));
+        if (!a.ref64) a.want[c] = want;  // every fragment of a request says the same
+      }
+    }
+    c = (uint32_t)__shfl((int)c, first, kWave);
+    if (mine) {
+      cell = c;
+      pending = false;
+    }
+  }
+  if (pending) {
+    cell = ra_find_cell(a, token);
+    if (cell != kRaNoCell) {
+      atomicAdd(&a.cnt[cell], 1u);
+      atomicAdd(&a.bytes[cell], (unsigned long long)len);
+      atomicMax(&a.last[cell], i);
+      if (!a.ref64) a.want[cell] = want;
+    }
+  }
+  if (in_range) {
+    a.arr_cell[i] = cell;
+    a.arr_len[i] = len;
+    a.arr_fidx[i] = fidx;
+  }
 }
 
 __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell)
