@@ -25,13 +25,6 @@ constexpr uint32_t kStNotRule = 1u << 5;     // a fragment's length departs from
 constexpr uint32_t kInvalidReq = 0xffffffffu; // owner field of a descriptor the kernels must skip
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-struct __attribute__((packed, aligned(1))) u32x4_unaligned { u32x4 v; };
-
-__device__ __forceinline__ u32x4 load16_any(const uint8_t *p)
-{
-  return reinterpret_cast<const u32x4_unaligned *>(p)->v;
-}
-
 struct __attribute__((packed, aligned(1))) u32_unaligned { uint32_t v; };
 __device__ __forceinline__ uint32_t load32_any(const uint8_t *p)
 {

@@ -356,7 +356,6 @@ __device__ __forceinline__ uint32_t item_of_wave(bool remap)
 // r starts at cursor + r * size in the bump ring.
 struct RuleArgs {
   const uint32_t *item_slot;
-  const uint32_t *item_len;  // gather: optional explicit lengths to hold against the rule
   const uint32_t *first;     // CSR table to hold against the rule
   uint64_t size;
   uint32_t mtu;
@@ -843,10 +842,11 @@ __global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, 
 //                position with the request's fragment count; workgroup-local
 //                scan of the packed (requests, fragments) flags
 //   k_ra_scan    one workgroup scans the workgroup totals
-//   k_ra_assign  batch index = number of requests completed before (completion
-//                order, the order of the rx-ready ring); first fragment index
-//   k_ra_emit    every arrival of a complete request writes its table entry at
-//                first + seq_num, and wipes its hash cell for the next call
+//   k_ra_emit    batch index of a request = number of requests completed before
+//                it (completion order, the order of the rx-ready ring), read
+//                off the scan at its last arrival; every arrival of a complete
+//                request writes its table entry at first + seq_num
+//   k_ra_wipe    empties the cells this call used
 
 struct RaArgs {
   const uint8_t *ring;
@@ -858,7 +858,7 @@ struct RaArgs {
   uint32_t max_req;
   // hash table
   unsigned long long *keys;
-  uint32_t *cnt, *last, *want, *cell_first, *cell_rank;
+  uint32_t *cnt, *last, *want;
   unsigned long long *bytes;
   // per arrival
   uint32_t *arr_cell, *arr_len, *arr_fidx;
@@ -1017,53 +1017,51 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
     const uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
     a.counts[0] = n_req;
     a.counts[1] = n_frag;
+    a.counts[2] = 0;  // k_ra_emit counts the arrivals left out
     if (n_req <= a.max_req) a.req_first[n_req] = n_frag;
     else atomicOr(a.status, kStBadTable);
   }
 }
 
-__global__ __launch_bounds__(256) void k_ra_assign(RaArgs a)
-{
-  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= a.n) return;
-  const unsigned long long p = a.arr_pack[i];
-  if (!(p >> 63)) return;
-  const unsigned long long v = (p & ~(1ull << 63)) + a.blk[i / kRaBlock];
-  const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v;
-  if (r >= a.max_req) return;  // refused by k_ra_scan
-  const uint32_t cell = a.arr_cell[i];
-  a.cell_rank[cell] = r;
-  a.cell_first[cell] = first;
-  a.req_first[r] = first;
-  if (a.req_token) a.req_token[r] = a.keys[cell];
-}
-
+// Every arrival of a complete request writes its table entry.  The request's
+// rank and first fragment index hang on its LAST arrival (arr_pack there, plus
+// the scanned total of that arrival's workgroup); that arrival also writes the
+// request's row of req_first / req_token.
 __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
 {
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= a.n) return;
-  const uint32_t cell = a.arr_cell[i];
-  if (cell == kRaNoCell) {
-    atomicAdd(&a.counts[2], 1u);
-    return;
-  }
-  // completeness was decided on the counters; they are read here before any
-  // thread of this kernel wipes them only through the flag the assign pass left:
-  // a complete request's cell carries its rank in cell_rank, an incomplete one kRaNoCell
-  const uint32_t rank = a.cell_rank[cell];
-  if (rank != kRaNoCell && rank < a.max_req) {
-    const uint32_t first = a.cell_first[cell];
-    const uint32_t n = a.req_first[rank + 1] - first;
-    const uint32_t fidx = a.arr_fidx[i];
-    if (fidx < n) {
-      a.frag_slot[first + fidx] = a.arrivals[i];
-      a.frag_len[first + fidx] = a.arr_len[i];
-    } else {
-      atomicOr(a.status, kStBadTable);  // a sequence number beyond the request's fragments
+  bool left_out = false;
+  if (i < a.n) {
+    const uint32_t cell = a.arr_cell[i];
+    left_out = true;
+    if (cell != kRaNoCell) {
+      const uint32_t last = a.last[cell];
+      const unsigned long long p = a.arr_pack[last];
+      if (p >> 63) {  // the request completed among these arrivals
+        const unsigned long long v = (p & ~(1ull << 63)) + a.blk[last / kRaBlock];
+        const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v;
+        if (r < a.max_req) {  // else refused by k_ra_scan
+          left_out = false;
+          const uint32_t n = a.cnt[cell];
+          const uint32_t fidx = a.arr_fidx[i];
+          if (fidx < n) {
+            a.frag_slot[first + fidx] = a.arrivals[i];
+            a.frag_len[first + fidx] = a.arr_len[i];
+          } else {
+            atomicOr(a.status, kStBadTable);  // a sequence number beyond the request's fragments
+          }
+          if (i == last) {
+            a.req_first[r] = first;
+            if (a.req_token) a.req_token[r] = a.keys[cell];
+          }
+        }
+      }
     }
-  } else {
-    atomicAdd(&a.counts[2], 1u);  // its request did not complete among these arrivals
   }
+  // arrivals whose request did not complete: one add per wavefront
+  const unsigned long long m = __ballot(left_out);
+  if (m && (threadIdx.x & (kWave - 1)) == (uint32_t)(__ffsll((long long)m) - 1))
+    atomicAdd(&a.counts[2], (uint32_t)__popcll(m));
 }
 
 // Wipes the cells this call used, so that the table is empty for the next one.
@@ -1078,7 +1076,6 @@ __global__ __launch_bounds__(256) void k_ra_wipe(RaArgs a)
   a.bytes[cell] = 0;
   a.last[cell] = 0;
   a.want[cell] = 0;
-  a.cell_rank[cell] = kRaNoCell;
 }
 
 }  // namespace
@@ -1805,17 +1802,13 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_re
   if (!c->ra_mem) {
     uint32_t cells = 2;
     while (cells < 2 * n_max) cells <<= 1;
-    // keys u64, bytes u64, cnt/last/want/cell_first/cell_rank u32 per cell;
+    // keys u64, bytes u64, cnt/last/want u32 per cell;
     // arr_cell/arr_len/arr_fidx u32 + arr_pack u64 per arrival; blk u64 per workgroup
     const size_t n_blk = (n_max + kRaBlock - 1) / kRaBlock + 1;
-    const size_t bytes = (size_t)cells * (8 + 8 + 5 * 4) + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 64;
+    const size_t bytes = (size_t)cells * (8 + 8 + 3 * 4) + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 64;
     HIP_TRY(c, hipMalloc(&c->ra_mem, bytes));
     HIP_TRY(c, hipMemsetAsync(c->ra_mem, 0, bytes, c->stream));
     c->ra_cells = cells;
-    // cell_rank starts as "no request"
-    uint8_t *base = static_cast<uint8_t *>(c->ra_mem);
-    uint32_t *cell_rank = reinterpret_cast<uint32_t *>(base + (size_t)cells * (8 + 8 + 4 * 4));
-    HIP_TRY(c, hipMemsetAsync(cell_rank, 0xff, (size_t)cells * 4, c->stream));
     HIP_TRY(c, hipHostMalloc((void **)&c->h_counts, 4 * sizeof(uint32_t), hipHostMallocDefault));
   }
   RaArgs r;
@@ -1840,8 +1833,6 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_re
   r.cnt = reinterpret_cast<uint32_t *>(m); m += C * 4;
   r.last = reinterpret_cast<uint32_t *>(m); m += C * 4;
   r.want = reinterpret_cast<uint32_t *>(m); m += C * 4;
-  r.cell_first = reinterpret_cast<uint32_t *>(m); m += C * 4;
-  r.cell_rank = reinterpret_cast<uint32_t *>(m); m += C * 4;
   r.arr_pack = reinterpret_cast<unsigned long long *>(m); m += (size_t)n_max * 8;
   r.blk = reinterpret_cast<unsigned long long *>(m); m += ((n_max + kRaBlock - 1) / kRaBlock + 1) * 8;
   r.arr_cell = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
@@ -1858,11 +1849,9 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_re
   const uint32_t g256 = (a->n_arrivals + 255) / 256;
   rc = prof_begin(c, 5);
   if (rc != SG_OK) return rc;
-  HIP_TRY(c, hipMemsetAsync(r.counts, 0, 4 * sizeof(uint32_t), c->stream));
   k_ra_insert<<<g256, 256, 0, c->stream>>>(r);
   k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
   k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);
-  k_ra_assign<<<g256, 256, 0, c->stream>>>(r);
   k_ra_emit<<<g256, 256, 0, c->stream>>>(r);
   k_ra_wipe<<<g256, 256, 0, c->stream>>>(r);
   rc = prof_end(c);
