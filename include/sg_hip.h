@@ -276,8 +276,8 @@ int sg_hip_get_cursor(sg_hip_ctx *ctx, int which, uint64_t *value);
  * context's stream (the PROFILE_MODE GDelay/SDelay vectors of the reference,
  * src/p2p_rpc_sg_engine.h:83-92, at kernel granularity).  which: 0 descriptor
  * build, 1 gather copy, 2 scatter copy + header rewrite, 3 per-request run
- * copy, 4 header-only rewrite, 5 reassembly (its six small kernels together).  sg_hip_kernel_time synchronizes, returns the
- * accumulated milliseconds and launch count since profiling was switched on,
+ * copy, 4 header-only rewrite, 5 reassembly (all of its kernels together).
+ * sg_hip_kernel_time synchronizes, returns the accumulated milliseconds and launch count since profiling was switched on,
  * and leaves the accumulators running. */
 int sg_hip_set_profiling(sg_hip_ctx *ctx, int on);
 int sg_hip_kernel_time(sg_hip_ctx *ctx, int which, double *total_ms, uint64_t *launches);
