@@ -298,6 +298,41 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
   return done;
 }
 
+// Replays the worker's batching window over a slot ring.  ops[k] > 0: the
+// shunter publishes ops[k] more requests (get_next + RX_COMPLETE, a slot is
+// reused once the transmit side has set it FREE); ops[k] < 0: the worker
+// collects a window of at most -ops[k] slots, "runs" it and completes it, and
+// the transmit side frees those slots.  out gets (start, size) per collect.
+// Returns the number of windows, or negative on error.
+int64_t sgh_window_replay(int device_id, int pool_size, const int32_t *ops, uint32_t n_ops, int32_t *out)
+{
+  if (hipSetDevice(device_id) != hipSuccess) return -1;
+  P2pRpcAppRrPool pool(pool_size, device_id, 64, 64, false);
+  SgBatchWindow win;
+  int64_t n_win = 0;
+  for (uint32_t k = 0; k < n_ops; k++) {
+    if (ops[k] > 0) {
+      for (int i = 0; i < ops[k]; i++) {
+        P2pRpcAppRr *a = pool.get_next();
+        if (*a->h_state != FREE) return -2;  // the caller overran the ring
+        *a->h_state = RX_COMPLETE;
+      }
+    } else {
+      const int got = win.collect(&pool, -ops[k]);
+      out[2 * n_win] = win.start();
+      out[2 * n_win + 1] = got;
+      n_win++;
+      const int s0 = win.start();
+      win.complete(&pool);
+      for (int i = 0, s = s0; i < got; i++, s = (s + 1) % pool_size) {
+        if (*pool.get_app_rr(s)->h_state != WORK_COMPLETE) return -3;
+        *pool.get_app_rr(s)->h_state = FREE;
+      }
+    }
+  }
+  return n_win;
+}
+
 // A double-mapped arena for callers outside C++ (the tests): the request
 // range of a P2pRpcAppRrMemPool.  Returns a handle, or NULL.
 void *sgh_mempool_create(int device_id, int n, uint64_t req_size, uint64_t resp_size, int want_mirror)

@@ -247,3 +247,38 @@ class P2pRpcAppRrPool {
     return a;
   }
 };
+
+// The worker's view of the slot ring: the window logic of
+// dynamic_batching_sync_worker_loop and sync_worker_loop
+// (src/p2p_rpc_async_app_server.h:173-206, 220-263) as steps a loop calls.
+// collect() extends the window over consecutive RX_COMPLETE slots from the
+// consumer index, up to max_batch; the batch's requests are contiguous from
+// get_app_rr(start())->h_stub (the model reads curr_batch_size requests from
+// there, :213-218).  complete() publishes WORK_COMPLETE for the window and
+// moves on.
+struct SgBatchWindow {
+  int rr_si_idx = 0;  // first slot of the window
+  int rr_ci_idx = 0;  // next slot to look at
+  int rr_win_size = 0;
+
+  inline int collect(P2pRpcAppRrPool *pool, int max_batch)
+  {
+    const int n = pool->get_pool_size();
+    while (rr_win_size < max_batch && rr_win_size < n &&
+           *pool->get_app_rr(rr_ci_idx)->h_state == RX_COMPLETE) {
+      rr_win_size++;
+      rr_ci_idx = (rr_ci_idx + 1) % n;
+    }
+    return rr_win_size;
+  }
+  inline int start() const { return rr_si_idx; }
+  inline void complete(P2pRpcAppRrPool *pool)
+  {
+    const int n = pool->get_pool_size();
+    int i = rr_si_idx;
+    for (int k = 0; k < rr_win_size; k++, i = (i + 1) % n) *pool->get_app_rr(i)->h_state = WORK_COMPLETE;
+    rr_si_idx = rr_ci_idx;
+    rr_win_size = 0;
+  }
+};
+

@@ -24,6 +24,8 @@ def host():
                                 C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32, C.c_int, C.c_int,
                                 C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.POINTER(C.c_int)]
+    h.sgh_window_replay.restype = C.c_int64
+    h.sgh_window_replay.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_uint32, C.c_void_p]
     h.sgh_mempool_create.restype = C.c_void_p
     h.sgh_mempool_create.argtypes = [C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_int]
     h.sgh_mempool_destroy.argtypes = [C.c_void_p]
@@ -139,3 +141,38 @@ def test_batch_across_the_end_of_a_double_mapped_arena(host, ctx, mode):
         assert np.array_equal(got, tx), first_diff(got, tx)
     finally:
         host.sgh_mempool_destroy(pool)
+
+
+def test_batching_window_over_the_slot_ring(host):
+    """SgBatchWindow (the window of dynamic_batching_sync_worker_loop,
+    src/p2p_rpc_async_app_server.h:220-263) against a list simulation: windows
+    are runs of consecutive RX_COMPLETE slots from the consumer index, capped
+    at max_batch, wrapping around the ring."""
+    rng = np.random.default_rng(4)
+    pool_size = 11
+    ops, sim_state, pi, ci, want = [], [0] * pool_size, 0, 0, []
+    for _ in range(400):
+        free = sum(1 for x in sim_state if x == 0)
+        if rng.random() < 0.5 and free:
+            k = int(rng.integers(1, free + 1))
+            ops.append(k)
+            for _ in range(k):
+                assert sim_state[pi] == 0
+                sim_state[pi] = 1
+                pi = (pi + 1) % pool_size
+        else:
+            m = int(rng.integers(1, 9))
+            ops.append(-m)
+            start, n = ci, 0
+            while n < m and n < pool_size and sim_state[ci] == 1:
+                sim_state[ci] = 0
+                ci = (ci + 1) % pool_size
+                n += 1
+            want.append((start, n))
+    ops_a = np.array(ops, np.int32)
+    out = np.zeros(2 * len(ops), np.int32)
+    n = host.sgh_window_replay(0, pool_size, p(ops_a), len(ops_a), p(out))
+    assert n == len(want)
+    got = [(int(out[2 * i]), int(out[2 * i + 1])) for i in range(n)]
+    assert got == want
+    assert max(g[1] for g in got) > 1 and any(g[1] == 0 for g in got)
