@@ -109,7 +109,10 @@ typedef struct sg_ring_desc {
  * says the arena's pages are mapped twice back to back
  * (src/p2p_rpc_app_rr_mem_pool.h:302-306) so that [arena, arena + 2*cap) is
  * addressable and a request may run past the end; otherwise a run that
- * crosses the end is split.
+ * crosses the end is split.  The requests of one gather call must fit the
+ * arena together (the reference's slot states guarantee as much,
+ * src/p2p_rpc_app_rr.h:127-134): a larger batch would overwrite its own first
+ * requests and is refused.
  * n_tensors >= 1: tensor-major buffers in the sense of g_params_v2
  * (src/p2p_rpc_app_stub.h:11-20): a request's byte stream is tensor 0's
  * bytes, then tensor 1's, ...; tensor t of request r lives at

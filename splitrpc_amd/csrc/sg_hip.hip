@@ -275,20 +275,30 @@ __device__ __forceinline__ void scan_emit(const PrepArgs &a, uint32_t q0, const 
   }
 }
 
+// A gathered batch larger than its arena would lap itself: wavefronts of the
+// first and of the last requests would then write the same bytes in no
+// particular order.  Refused instead.
+__device__ __forceinline__ void scan_check_batch(const PrepArgs &a, uint64_t batch_bytes)
+{
+  if (a.mode == 0 && batch_bytes > a.cap) atomicOr(a.status, kStBadSize);
+}
+
 __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
-  uint64_t run = *a.cursor_in % a.cap;
+  uint64_t run = *a.cursor_in % a.cap, batch_bytes = 0;
   for (uint32_t base = 0; base < a.n_req; base += kScanTile) {
     const uint32_t q0 = base + threadIdx.x * kScanPerThread;
     uint64_t sz[kScanPerThread], tot;
     const uint64_t ex = scan_tile(a, q0, sz, wave_tot, &tot);
     scan_emit(a, q0, sz, (run + ex) % a.cap);
     run = (run + tot) % a.cap;
+    batch_bytes += tot;
   }
   if (threadIdx.x == 0) {
     *a.cursor_out = run;
     if (a.offsets_out) a.offsets_out[a.n_req] = run;
+    scan_check_batch(a, batch_bytes);
   }
 }
 
@@ -305,18 +315,20 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan_local(PrepArgs a, uint6
 __global__ __launch_bounds__(kScanBlock) void k_req_scan_tiles(PrepArgs a, uint64_t *tile_tot, uint32_t n_tiles)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
-  uint64_t run = *a.cursor_in % a.cap;
+  uint64_t run = *a.cursor_in % a.cap, batch_bytes = 0;
   for (uint32_t base = 0; base < n_tiles; base += kScanBlock) {
     const uint32_t t = base + threadIdx.x;
-    const uint64_t v = t < n_tiles ? tile_tot[t] % a.cap : 0;
+    const uint64_t v = t < n_tiles ? tile_tot[t] : 0;
     uint64_t tot;
     const uint64_t ex = block_exclusive_scan<kScanBlock>(v, wave_tot, &tot);
     if (t < n_tiles) tile_tot[t] = (run + ex % a.cap) % a.cap;
     run = (run + tot % a.cap) % a.cap;
+    batch_bytes += tot;
   }
   if (threadIdx.x == 0) {
     *a.cursor_out = run;
     if (a.offsets_out) a.offsets_out[a.n_req] = run;
+    scan_check_batch(a, batch_bytes);
   }
 }
 
@@ -565,7 +577,7 @@ struct GatherRuleArgs {
   uint32_t hl;
   uint32_t n_slots;
   uint32_t pieces;            // wavefronts per fragment
-  uint32_t opts;  // kOptRemap | kOptMirrored | kOptSingleWrap | kOptMultiTensor
+  uint32_t opts;  // kOptRemap | kOptMirrored | kOptMultiTensor | kOptHdrChunk
   // warm
   uint32_t n_req;
   const uint32_t *frag_len;
@@ -575,7 +587,10 @@ struct GatherRuleArgs {
   uint32_t *status;
   AppDev app;  // consulted for several tensor-major buffers only
 };
-constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptSingleWrap = 4u, kOptMultiTensor = 8u;
+constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
+// slots start at 16-byte aligned addresses: the header's length field can be read as part of
+// the aligned chunk at byte 48 (a ring only has to start at an even address)
+constexpr uint32_t kOptHdrChunk = 16u;
 
 template <bool LONG>
 __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
@@ -616,8 +631,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
     if (c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
     ro = c0 + (uint64_t)r * size;
-    if (opts & kOptSingleWrap) ro = ro >= cap ? ro - cap : ro;  // n_req * size <= capacity
-    else ro %= cap;
+    ro = ro >= cap ? ro - cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
     if (lane == 0 && piece == 0) {
       if (i == 0 && a.offsets_out) a.offsets_out[r] = ro;
       if (item == n_items - 1) {
@@ -640,18 +654,20 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   // with the payload, so that checking them does not lengthen the wavefront's
   // life by another memory round trip.
   const bool check_hdr = piece == 0 && a.frag_len == nullptr;
-  uint32_t w0 = 0, w1 = 0;
+  uint32_t hv = 0;
+  u32x4 hc = {0u, 0u, 0u, 0u};
   if (check_hdr) {
-    w0 = sload(reinterpret_cast<const uint32_t *>(pkt + 52));
-    w1 = sload(reinterpret_cast<const uint32_t *>(pkt + 56));
+    // every lane asks for the same bytes: one request, and on the cache line
+    // the payload's first chunk needs anyway
+    if (opts & kOptHdrChunk) hc = *reinterpret_cast<const u32x4 *>(pkt + 48);
+    else hv = load32_any(pkt + 54);
   }
   // copying the ruled length stays inside the slot whatever the header says
   RunState rs;
   uint32_t sub_off = 0, sub_len = len;
   if (LONG && plain) sub_run(to, len, piece, &sub_off, &sub_len);
   if (plain && sub_len) run_begin(rs, pkt + hl + sub_off, to + sub_off, sub_len, lane);
-  SG_PIN(w0);
-  SG_PIN(w1);
+  asm volatile("" ::"v"(hc), "v"(hv));  // consumed only after the payload loads are under way
   if (plain) {
     if (sub_len) run_end<false>(rs, lane);
   } else if (piece == 0) {
@@ -659,9 +675,9 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   }
   if (piece == 0) {
     uint32_t bad = 0;
-    // payload_len is the u32 at byte 54: the upper half of w0 and the lower half of w1
-    const bool as_ruled = check_hdr ? (((w0 >> 16) == (len & 0xffffu)) & ((w1 & 0xffffu) == (len >> 16)))
-                                    : sload(a.frag_len + item) == len;
+    // payload_len is the u32 at byte 54: bytes 6..9 of the chunk that starts at byte 48
+    const uint32_t hdr_len = (opts & kOptHdrChunk) ? ((hc[1] >> 16) | (hc[2] << 16)) : hv;
+    const bool as_ruled = (check_hdr ? hdr_len : sload(a.frag_len + item)) == len;
     if (!as_ruled) bad |= kStNotRule;
     if (i == 0 && sload(a.first + r) != item) bad |= kStBadTable;
     if (bad && lane == 0) atomicOr(a.status, bad);
@@ -1555,6 +1571,9 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     if (per * a->n_req != a->n_frags) return fail(c, SG_E_INVAL, "%u requests of %llu bytes at mtu %u are %llu fragments, not %u", a->n_req, (unsigned long long)a->fixed_req_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frags);
     if (a->fixed_req_size > 0xffffffffull || (app.n_tensors == 0 ? a->fixed_req_size > app.cap : a->fixed_req_size > max_req_bytes))
       return fail(c, SG_E_INVAL, "request size %llu does not fit its destination", (unsigned long long)a->fixed_req_size);
+    // a batch larger than the arena would lap itself and its wavefronts would race for the same bytes
+    if (app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_req_size > app.cap)
+      return fail(c, SG_E_INVAL, "%u requests of %llu bytes do not fit an arena of %llu bytes", a->n_req, (unsigned long long)a->fixed_req_size, (unsigned long long)app.cap);
     GatherRuleArgs ga;
     memset(&ga, 0, sizeof ga);
     ga.ring = static_cast<const uint8_t *>(a->ring.base);
@@ -1581,8 +1600,8 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     uint32_t grid, remap;
     geometry((uint64_t)a->n_frags * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
-              ((app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_req_size <= app.cap) ? kOptSingleWrap : 0u) |
-              (app.n_tensors > 1 ? kOptMultiTensor : 0u);
+              (app.n_tensors > 1 ? kOptMultiTensor : 0u) |
+              ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
     if (ga.pieces > 1) k_gather_rule<true><<<grid, kBlock, 0, c->stream>>>(ga);

@@ -244,9 +244,20 @@ class DeviceWorkload:
     """A synthetic workload staged in one GPU's memory: the landing-zone ring,
     the fragment tables and the application buffers."""
 
+    @staticmethod
+    def _shifted(t: torch.Tensor, shift: int) -> torch.Tensor:
+        if not shift:
+            return t
+        backing = torch.zeros(t.numel() + shift + 16, dtype=t.dtype, device=t.device)
+        view = backing[shift:shift + t.numel()]
+        view.copy_(t)
+        return view
+
     def __init__(self, w: Workload, device="cuda:0", arena_slack: int = 0, copies: int = 1,
-                 unique_tokens: bool = False):
-        """``copies`` > 1 lays that many copies of the ring (and of the tables,
+                 unique_tokens: bool = False, ring_shift: int = 0):
+        """``ring_shift`` moves both rings that many bytes off the allocator's
+        alignment (rings only have to start at an even address).
+        ``copies`` > 1 lays that many copies of the ring (and of the tables,
         slot indices shifted) side by side, so that one call moves ``copies``
         batches and the working set outgrows the caches."""
         self.w = w
@@ -267,6 +278,7 @@ class DeviceWorkload:
             used = torch.from_numpy(w.frag_slot.astype(np.int64)).to(dev)
             v[:, used, 47] = ((v[:, used, 47].to(torch.int32) + (c & 0xFF)) & 0xFF).to(torch.uint8)
             v[:, used, 48] = ((v[:, used, 48].to(torch.int32) + (c >> 8)) & 0xFF).to(torch.uint8)
+        self.ring = self._shifted(self.ring, ring_shift)
         self.rx = RingRef(self.ring, w.n_slots * k, w.slot_size, w.profile)
 
         def tile_slots(a: np.ndarray, n_slots: int) -> np.ndarray:
@@ -288,7 +300,7 @@ class DeviceWorkload:
             self.tx_ring = self.ring
         else:
             t1 = torch.from_numpy(w.tx_ring_init).to(dev)
-            self.tx_ring = t1.repeat(k) if k > 1 else t1
+            self.tx_ring = self._shifted(t1.repeat(k) if k > 1 else t1, ring_shift)
         self.tx = RingRef(self.tx_ring, w.tx_n_slots * k, w.slot_size, w.profile)
 
         # request side application buffers

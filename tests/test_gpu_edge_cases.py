@@ -250,13 +250,13 @@ def test_arena_wrap_and_cursor_persistence(ctx, mode):
     sizes = [4200] * 5 if rule else [3000, 5000, 700, 4100, 2222]
     w = synth.make_custom(sizes, [64] * 5, seed=10)
     total = int(sum(sizes))
-    cap = total - 1000  # the batch wraps
+    cap = total + 1234
     dw = DeviceWorkload(w)
     arena = torch.zeros(cap, dtype=torch.uint8, device=DEV)
     app = AppRef(arena=arena, cap=cap)
     offs = torch.zeros(w.n_req + 1, dtype=torch.int64, device=DEV)
-    ctx.set_cursor(0, 777)
-    cur = 777
+    cur = cap - 5000  # the second request of the first call crosses the end
+    ctx.set_cursor(0, cur)
     want = np.zeros(cap, np.uint8)
     for call in range(3):
         flags = capi.F_RULE_FRAGS if rule else 0
@@ -268,6 +268,72 @@ def test_arena_wrap_and_cursor_persistence(ctx, mode):
         assert np.array_equal(offs.cpu().numpy().view(np.uint64), eoffs)
         assert ctx.get_cursor(0) == ecur
         cur = ecur
+
+
+@pytest.mark.parametrize("shift", [2, 6, 14])
+@pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64])
+def test_rings_at_even_addresses_off_word_alignment(ctx, shift, profile):
+    """A ring only has to start at an even address: every header word then
+    sits at an address = 2 (mod 4).  All three gather modes, scatter and
+    reassembly must read the same bytes as on an aligned ring."""
+    w = synth.make_custom([4200] * 7, [3000] * 7, seed=60 + shift, profile=profile,
+                          flags=synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL)
+    print(f"case shifted ring shift={shift} profile={profile}", flush=True)
+    dw = DeviceWorkload(w, ring_shift=shift)
+    assert dw.ring.data_ptr() % 4 == 2
+    exp, offs, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    ref64 = profile == synth.HDR_REF64
+    for mode in ("scan", "fixed", "rule"):
+        ctx.set_cursor(0, 0)
+        dw.req_arena.zero_()
+        dw.gather(ctx, use_frag_len=ref64, fixed=mode != "scan", rule=mode == "rule")
+        got = dw.req_arena.cpu().numpy()
+        assert np.array_equal(got, exp), mode + ": " + first_diff(got, exp)
+    for fuse in (True, False):
+        ctx.set_cursor(1, 0)
+        dw.scatter(ctx, fuse=fuse)
+        exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
+        got = dw.tx_ring.cpu().numpy()
+        assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
+    # reassembly reads tokens and sequence numbers from the same headers
+    fs = torch.zeros(w.n_frags, dtype=torch.int32, device=DEV)
+    fl = torch.zeros(w.n_frags, dtype=torch.int32, device=DEV)
+    rf = torch.zeros(8193, dtype=torch.int32, device=DEV)
+    len_nic = None
+    if ref64:
+        ln = np.zeros(w.n_slots, np.uint32)
+        ln[w.frag_slot] = w.frag_len
+        len_nic = to_dev(ln, DEV)
+    n_req, n_frag, n_left = ctx.reassemble(dw.rx, dw.arrivals, int(dw.arrivals.numel()), fs, fl, rf,
+                                           len_nic=len_nic, req_size=4200 if ref64 else 0)
+    assert (n_req, n_frag, n_left) == (w.n_req, w.n_frags, 0)
+    assert np.array_equal(fs.cpu().numpy().view(np.uint32), w.frag_slot.astype(np.uint32))
+    assert np.array_equal(fl.cpu().numpy().view(np.uint32), w.frag_len.astype(np.uint32))
+
+
+@pytest.mark.parametrize("mode", ["scan", "rule"])
+def test_batch_larger_than_its_arena_is_refused(ctx, mode):
+    """Such a batch would lap itself: its first and last requests would share
+    bytes, written in no particular order.  Nothing is moved."""
+    rule = mode == "rule"
+    sizes = [4200] * 5 if rule else [3000, 5000, 700, 4100, 2222]
+    w = synth.make_custom(sizes, [64] * 5, seed=11)
+    cap = int(sum(sizes)) - 1
+    dw = DeviceWorkload(w)
+    arena = torch.full((cap,), 7, dtype=torch.uint8, device=DEV)
+    ctx.set_cursor(0, 0)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, AppRef(arena=arena, cap=cap),
+                         flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if rule else 0, mtu=w.mtu)
+    assert e.value.code == (capi.SG_E_INVAL if rule else capi.SG_E_DATA)
+    assert bool((arena == 7).all())
+    # one byte more and it fits
+    ctx.set_cursor(0, 0)
+    arena2 = torch.zeros(cap + 1, dtype=torch.uint8, device=DEV)
+    ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, AppRef(arena=arena2, cap=cap + 1),
+                     flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if rule else 0, mtu=w.mtu)
+    exp, _, _ = oracle.gather(w, arena_cap=cap + 1)
+    assert np.array_equal(arena2.cpu().numpy(), exp)
 
 
 def test_odd_arena_base_and_tensor_major_split(ctx):
