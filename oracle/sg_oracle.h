@@ -26,7 +26,15 @@
  *                         leaves this to NIC offload (dpdk_rx_tx.h:143)
  *   sgo_udp_full_csum     RFC 768 verify-to-ffff, scalar byte loop, 0->ffff
  *                         PARITY UNPINNED vs the reference (NIC offload)
- *   sgo_rr_* / sgo_pool_* arrival-order invariance, brute-force reassembly
+ *   sgo_gen_hdr_template  compiled reference eth_common.h templates (oracle/_ref)
+ *   sgo_set_conn_info     every byte range against its source, untouched
+ *                         bytes unchanged
+ *   sgo_template_resp_hdr identity: template path == swap path when the
+ *   sgo_rewrite_resp_hdr  template carries the identity the request was sent
+ *                         to (two independent routes to one header)
+ *   sgo_reassemble        arrival-order invariance, brute-force reassembly
+ *   sgo_gather_batch /    pure-Python brute force (byte-wise arena wrap,
+ *   sgo_scatter_batch     tensor-major split, big-endian header arithmetic)
  *   echo / vec_add bytes  lib_loadgen/echo_client.cc:11-32,
  *                         vec_add_client.cc:11-19 patterns
  */
