@@ -240,9 +240,9 @@ __global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
 // Scan of the request totals through the bump ring:
 //   ret = base + off; off = (off + size) % capacity   (src/p2p_rpc_tring.h:27-33)
 // Up to kScanTile requests: one workgroup does it all (k_req_scan).  Beyond:
-// one workgroup per tile scans locally (k_req_scan_local), one workgroup
-// scans the tile totals from the cursor (k_req_scan_tiles), and the tiles add
-// their base (k_req_scan_add).
+// one workgroup per tile totals its requests (k_req_scan_local), then every
+// tile takes the sum of the totals before it as its base and scans from there
+// (k_req_scan_add).
 constexpr int kScanBlock = 1024;
 constexpr int kScanPerThread = 4;
 constexpr uint32_t kScanTile = kScanBlock * kScanPerThread;
@@ -312,33 +312,35 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan_local(PrepArgs a, uint6
   if (threadIdx.x == 0) tile_tot[blockIdx.x] = tot;
 }
 
-__global__ __launch_bounds__(kScanBlock) void k_req_scan_tiles(PrepArgs a, uint64_t *tile_tot, uint32_t n_tiles)
+// Every tile sums the totals of the tiles before it (a few values) for its base
+// and scans again from there; the last tile also publishes the advanced cursor.
+__global__ __launch_bounds__(kScanBlock) void k_req_scan_add(PrepArgs a, const uint64_t *tile_tot, uint32_t n_tiles)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
-  uint64_t run = *a.cursor_in % a.cap, batch_bytes = 0;
-  for (uint32_t base = 0; base < n_tiles; base += kScanBlock) {
+  const bool is_last = blockIdx.x == n_tiles - 1;
+  const uint32_t upto = is_last ? n_tiles : blockIdx.x;  // the last tile needs the batch total too
+  uint64_t before = 0, batch_bytes = 0;
+  for (uint32_t base = 0; base < upto; base += kScanBlock) {
     const uint32_t t = base + threadIdx.x;
-    const uint64_t v = t < n_tiles ? tile_tot[t] : 0;
+    const uint64_t v = t < upto ? tile_tot[t] : 0;
     uint64_t tot;
     const uint64_t ex = block_exclusive_scan<kScanBlock>(v, wave_tot, &tot);
-    if (t < n_tiles) tile_tot[t] = (run + ex % a.cap) % a.cap;
-    run = (run + tot % a.cap) % a.cap;
+    (void)ex;
     batch_bytes += tot;
   }
-  if (threadIdx.x == 0) {
-    *a.cursor_out = run;
-    if (a.offsets_out) a.offsets_out[a.n_req] = run;
-    scan_check_batch(a, batch_bytes);
-  }
-}
-
-__global__ __launch_bounds__(kScanBlock) void k_req_scan_add(PrepArgs a, const uint64_t *tile_base)
-{
-  __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  before = is_last ? batch_bytes - tile_tot[blockIdx.x] : batch_bytes;
+  const uint64_t c0 = *a.cursor_in % a.cap;
+  const uint64_t tile_base = (c0 + before % a.cap) % a.cap;
   const uint32_t q0 = blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
   uint64_t sz[kScanPerThread], tot;
   const uint64_t ex = scan_tile(a, q0, sz, wave_tot, &tot);
-  scan_emit(a, q0, sz, (tile_base[blockIdx.x] + ex % a.cap) % a.cap);
+  scan_emit(a, q0, sz, (tile_base + ex % a.cap) % a.cap);
+  if (is_last && threadIdx.x == 0) {
+    const uint64_t end = (c0 + batch_bytes % a.cap) % a.cap;
+    *a.cursor_out = end;
+    if (a.offsets_out) a.offsets_out[a.n_req] = end;
+    scan_check_batch(a, batch_bytes);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1282,8 +1284,7 @@ int launch_prep(sg_hip_ctx *c, const PrepArgs &p)
       const uint32_t n_tiles = (p.n_req + kScanTile - 1) / kScanTile;
       uint64_t *tile_tot = c->tile_tot;
       k_req_scan_local<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot);
-      k_req_scan_tiles<<<1, kScanBlock, 0, c->stream>>>(p, tile_tot, n_tiles);
-      k_req_scan_add<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot);
+      k_req_scan_add<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot, n_tiles);
     }
   }
   return prof_end(c);
