@@ -165,6 +165,35 @@ def _cpu_run(w, seconds: float, threads: int):
     return passes, dt, n_copies
 
 
+def back_to_back(ctx, pool: Pool, which: str, launches: int) -> float:
+    """Seconds per launch of one kernel launched back to back: two HIP events on
+    the context's stream around the whole burst (no event between launches, so
+    the figure carries the gaps between kernels but not an event's own cost)."""
+    import torch
+    from splitrpc_amd import capi
+    stream = torch.cuda.ExternalStream(ctx.stream, device="cuda:0")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n_items = len(pool.items)
+
+    def launch(i):
+        dw = pool.items[i % n_items]
+        if which == "k_gather":
+            dw.gather(ctx, capi.F_ASYNC | pool.extra_flags, rule=pool.rule)
+        else:
+            dw.scatter(ctx, capi.F_ASYNC | pool.extra_flags, fuse=pool.rule)
+
+    for i in range(n_items):
+        launch(i)
+    ctx.sync()
+    e0.record(stream)
+    for i in range(launches):
+        launch(i)
+    e1.record(stream)
+    e1.synchronize()
+    ctx.sync()
+    return e0.elapsed_time(e1) * 1e-3 / launches
+
+
 def cpu_baseline(w, seconds: float):
     """The CPU oracle (a restatement of the reference's CPU scatter-gather
     path) timed on this host over rotated ring copies: on one thread -- the
@@ -227,6 +256,7 @@ def main() -> int:
     dom_bytes = pool.gather_bytes if dom == "k_gather" else pool.scatter_bytes
     dom_ms = kt[dom][0]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+    b2b = back_to_back(ctx, pool, dom, min(a.steps, 100))
 
     # request reassembly on the device for the same call's arrivals (synchronous: counts come back)
     dw0 = pool.items[0]
@@ -306,7 +336,11 @@ def main() -> int:
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": None if a.general else MEASURED_TRAFFIC.get((a.workload, bpl, dom)),
                      "traffic_unit": "HBM bytes per launch (rocprofv3 --pmc, see profiles/)",
-                     "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3)},
+                     "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3),
+                     # the same call launched back to back, two events around the burst (all of the
+                     # call's kernels and the gaps between launches, no per-launch event)
+                     "back_to_back_us_per_call": round(b2b * 1e6, 3),
+                     "back_to_back_GBps": round(dom_bytes / b2b / 1e9, 1)},
         "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in kt.items()},
         "single_batch_call": single,
         "device_reassembly": reassembly,
