@@ -194,6 +194,39 @@ def back_to_back(ctx, pool: Pool, which: str, launches: int) -> float:
     return e0.elapsed_time(e1) * 1e-3 / launches
 
 
+def per_request_calls(ctx, dw, calls: int = 300):
+    """The drop-in per-request path: one synchronous sg_hip_gather per request
+    from a host-built run table, as copy_engine->gather(rr, stub) issues them
+    (latency of table staging + launch + wait, one request at a time)."""
+    import ctypes as C
+    from splitrpc_amd import capi
+    w = dw.w
+    hl = 64 if w.profile == 1 else 58
+    skbs = []
+    for r in range(min(w.n_req, 8)):
+        f0, f1 = int(w.req_first[r]), int(w.req_first[r + 1])
+        skb = capi.SkBuf()
+        off = 0
+        for k, f in enumerate(range(f0, f1)):
+            skb.i_buf[k] = dw.ring.data_ptr() + int(w.frag_slot[f]) * w.slot_size + hl
+            skb.o_buf[k] = dw.req_arena.data_ptr() + r * int(w.req_sizes[r]) + off
+            skb.len[k] = int(w.frag_len[f])
+            off += int(w.frag_len[f])
+        skb.num_items = f1 - f0
+        skbs.append(skb)
+    fn = ctx.lib.sg_hip_gather
+    for i in range(20):
+        assert fn(ctx.h, C.byref(skbs[i % len(skbs)])) == 0
+    t0 = time.perf_counter()
+    for i in range(calls):
+        fn(ctx.h, C.byref(skbs[i % len(skbs)]))
+    dt = (time.perf_counter() - t0) / calls
+    size = int(w.req_sizes[0])
+    return {"us_per_gather_call": round(dt * 1e6, 2), "runs_per_request": int(skbs[0].num_items),
+            "request_bytes": size, "requests_per_sec": round(1.0 / dt, 1),
+            "GBps": round((2 * size + 16 * int(skbs[0].num_items)) / dt / 1e9, 2)}
+
+
 def cpu_baseline(w, seconds: float):
     """The CPU oracle (a restatement of the reference's CPU scatter-gather
     path) timed on this host over rotated ring copies: on one thread -- the
@@ -289,6 +322,7 @@ def main() -> int:
                   if k1["k_gather"][0] > 0 else None}
         del p1
 
+    per_req = per_request_calls(ctx, pool.items[0]) if not w.in_tensor_sizes else None
     rps = {WORKLOAD_NAMES[a.workload]: round(pool.n_req / sec, 1)}
     sweep = {}
     if not a.no_sweep:
@@ -343,6 +377,7 @@ def main() -> int:
                      "back_to_back_GBps": round(dom_bytes / b2b / 1e9, 1)},
         "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in kt.items()},
         "single_batch_call": single,
+        "per_request_call": per_req,
         "device_reassembly": reassembly,
         "other_workloads": sweep,
     }
