@@ -229,7 +229,7 @@ __device__ __forceinline__ uint32_t copy_run(const uint8_t *__restrict__ src,
 }
 
 // A LONG run (jumbo frames) is cut into sub-runs of kPieceChunks destination
-// chunks that different wavefronts (or one wavefront, two at a time) copy with
+// chunks that different wavefronts (or one wavefront, several at a time) copy with
 // the functions above: sub-run 0 is the head bytes plus the first
 // kPieceChunks aligned chunks, every later one starts on a 16-byte destination
 // boundary, the last one takes the tail bytes.  A sub-run's aligned source
@@ -257,23 +257,25 @@ __device__ __forceinline__ void sub_run(const uint8_t *dst, uint32_t len, uint32
   *n = start >= len ? 0 : (end < len ? end : len) - start;
 }
 
-// Copy a whole long run with one wavefront, two sub-runs in flight at a time.
-template <bool CSUM>
+// Copy a whole long run with one wavefront, DEPTH sub-runs in flight at a time.
+template <bool CSUM, int DEPTH>
 __device__ __forceinline__ uint32_t copy_long_run(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                                                   uint32_t len, uint32_t lane)
 {
   uint32_t acc = 0;
-  for (uint32_t piece = 0;; piece += 2) {
-    uint32_t o0, n0, o1, n1;
-    sub_run(dst, len, piece, &o0, &n0);
-    sub_run(dst, len, piece + 1, &o1, &n1);
-    if (n0 == 0) break;
-    RunState r0, r1;
-    run_begin(r0, src + o0, dst + o0, n0, lane);
-    if (n1) run_begin(r1, src + o1, dst + o1, n1, lane);
-    acc += run_end<CSUM>(r0, lane);
-    if (n1) acc += run_end<CSUM>(r1, lane);
-    else break;
+  for (uint32_t base = 0;; base += DEPTH) {
+    RunState r[DEPTH];
+    uint32_t n[DEPTH];
+#pragma unroll
+    for (int k = 0; k < DEPTH; k++) {
+      uint32_t o;
+      sub_run(dst, len, base + k, &o, &n[k]);
+      if (n[k]) run_begin(r[k], src + o, dst + o, n[k], lane);
+    }
+#pragma unroll
+    for (int k = 0; k < DEPTH; k++)
+      if (n[k]) acc += run_end<CSUM>(r[k], lane);
+    if (!n[DEPTH - 1]) break;
   }
   return acc;
 }

@@ -703,22 +703,28 @@ struct ScatterArgs {
   uint32_t flags;
   uint32_t n_items;
   uint32_t remap;
-  uint32_t pieces;  // wavefronts per frame (1 when the payload is summed: one wavefront owns the sum)
+  uint32_t pieces;  // wavefronts per frame
   uint32_t *status;
   RuleArgs rule;
   AppDev app;
 };
 
 // LONG: frames longer than kPieceChunks chunks are spread over a.pieces
-// wavefronts (never when the payload is summed: one wavefront owns the sum).
+// wavefronts; piece 0 also writes the header.  With the payload sum
+// (FULL_CSUM) a long frame stays with one wavefront, which walks its sub-runs
+// two at a time (more in flight cost registers, hence resident wavefronts, and
+// measured slower: 3 at a time +1 %, 5 at a time +8 %).  (Summing per piece and combining with one returning atomic
+// per wavefront was measured: the atomic's round trip at the end of every
+// wavefront's life cost more than the shorter tail gained.)
 template <bool FULL_CSUM, bool FUSED, bool LONG>
 __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
-  static_assert(!(FULL_CSUM && LONG), "a summed frame belongs to one wavefront");
+  constexpr bool SPLIT = LONG && !FULL_CSUM;  // several wavefronts per frame
+  constexpr bool WHOLE_LONG = LONG && FULL_CSUM;  // one wavefront walks all sub-runs of its frame
   const uint32_t w = item_of_wave(a.remap != 0);
-  const uint32_t pieces = LONG ? a.pieces : 1u;  // FULL_CSUM: a.pieces only says "long frames"
-  const uint32_t item = LONG ? w / pieces : w;
-  const uint32_t piece = LONG ? w - item * pieces : 0;
+  const uint32_t pieces = SPLIT ? a.pieces : 1u;
+  const uint32_t item = SPLIT ? w / pieces : w;
+  const uint32_t piece = SPLIT ? w - item * pieces : 0;
   if (item >= a.n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   u32x4 d;
@@ -745,16 +751,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     nf = a.rule.per_req;
   }
   uint8_t *slot = a.tx + (size_t)d[0] * a.tx_slot_size;
-  if (LONG && piece != 0) {
-    // a later piece of a long frame: payload only
-    uint8_t *from;
-    if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
-      uint32_t o, n;
-      sub_run(slot + a.hl, d[1], piece, &o, &n);
-      if (n) copy_run<false>(from + o, slot + a.hl + o, n, lane);
-    }
-    return;
-  }
+  // where the header comes from; a frame whose header source is out of range is left alone by
+  // all of its pieces
   const bool from_template = a.hdr_templates != nullptr;
   const uint8_t *hin;
   HdrFields hf{a.hl, a.ref64, a.flags, item - f0, nf, d[1], 0, 0, 0};
@@ -768,13 +766,24 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   } else {
     const uint32_t hs = a.hdr_src_slot[item];
     if (hs >= a.rx_n_slots) {
-      if (lane == 0) atomicOr(a.status, kStBadSlot);
+      if (lane == 0 && piece == 0) atomicOr(a.status, kStBadSlot);
       return;
     }
-    // read the request header before anything of this slot is overwritten
-    // (the TX slot may be the very slot the header comes from)
     hin = a.rx + (size_t)hs * a.rx_slot_size;
   }
+
+  if (SPLIT && piece != 0) {
+    // a later piece of a long frame: payload only
+    uint8_t *from;
+    if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
+      uint32_t o, n;
+      sub_run(slot + a.hl, d[1], piece, &o, &n);
+      if (n) copy_run<false>(from + o, slot + a.hl + o, n, lane);
+    }
+    return;
+  }
+  // read the request header before anything of this slot is overwritten
+  // (the TX slot may be the very slot the header comes from);
   // header bytes and payload chunks are fetched together; the header arithmetic
   // then runs while the payload is still on its way
   const uint32_t raw = hdr_fetch(hin, lane, a.hl, !from_template);
@@ -782,18 +791,15 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   uint8_t *from = nullptr;
   const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
   RunState rs;
-  // a summed frame stays with one wavefront; a long one is then walked two
-  // sub-runs at a time
-  const bool whole_long = FULL_CSUM && a.pieces > 1;
   uint32_t first_len = d[1];
-  if (LONG && plain) {
+  if (SPLIT && plain) {
     uint32_t o;
     sub_run(slot + a.hl, d[1], 0, &o, &first_len);
   }
-  if (plain && !whole_long) run_begin(rs, from, slot + a.hl, first_len, lane);
+  if (plain && !WHOLE_LONG) run_begin(rs, from, slot + a.hl, first_len, lane);
   if (!FULL_CSUM) hb = hdr_finish(raw, lane, hf, 0);
   if (plain) {
-    if (whole_long) acc = copy_long_run<FULL_CSUM>(from, slot + a.hl, d[1], lane);
+    if (WHOLE_LONG) acc = copy_long_run<FULL_CSUM, 2>(from, slot + a.hl, d[1], lane);
     else acc = run_end<FULL_CSUM>(rs, lane);
   } else if (d[1]) {
     acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
@@ -1303,6 +1309,16 @@ int finish(sg_hip_ctx *c, uint32_t flags)
 
 }  // namespace
 
+template <bool FUSED>
+static void launch_scatter(sg_hip_ctx *c, const ScatterArgs &sa, uint32_t grid, bool full_csum)
+{
+  const bool lng = sa.pieces > 1;
+  if (full_csum && lng) k_scatter<true, FUSED, true><<<grid, kBlock, 0, c->stream>>>(sa);
+  else if (full_csum) k_scatter<true, FUSED, false><<<grid, kBlock, 0, c->stream>>>(sa);
+  else if (lng) k_scatter<false, FUSED, true><<<grid, kBlock, 0, c->stream>>>(sa);
+  else k_scatter<false, FUSED, false><<<grid, kBlock, 0, c->stream>>>(sa);
+}
+
 extern "C" {
 
 int sg_hip_abi_version(void) { return SG_HIP_ABI_VERSION; }
@@ -1724,14 +1740,12 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     if (app.n_tensors == 0) c->parity[1] ^= 1u;
     sa.rule.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
     sa.pieces = pieces_for(a->mtu);
-    const uint32_t waves_per_frame = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces;
     uint32_t grid;
-    geometry((uint64_t)a->n_frames * waves_per_frame, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry((uint64_t)a->n_frames * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
+             !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, true, false><<<grid, kBlock, 0, c->stream>>>(sa);
-    else if (sa.pieces > 1) k_scatter<false, true, true><<<grid, kBlock, 0, c->stream>>>(sa);
-    else k_scatter<false, true, false><<<grid, kBlock, 0, c->stream>>>(sa);
+    launch_scatter<true>(c, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
     return finish(c, a->flags);
@@ -1786,14 +1800,12 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.status = c->status;
     sa.app = app;
     sa.pieces = pieces_for(a->mtu);
-    const uint32_t waves_per_frame = (a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces;
     uint32_t grid;
-    geometry((uint64_t)a->n_frames * waves_per_frame, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    geometry((uint64_t)a->n_frames * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
+             !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    if (a->flags & SG_F_UDP_CSUM_FULL) k_scatter<true, false, false><<<grid, kBlock, 0, c->stream>>>(sa);
-    else if (sa.pieces > 1) k_scatter<false, false, true><<<grid, kBlock, 0, c->stream>>>(sa);
-    else k_scatter<false, false, false><<<grid, kBlock, 0, c->stream>>>(sa);
+    launch_scatter<false>(c, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }

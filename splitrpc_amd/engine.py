@@ -98,6 +98,13 @@ class SgContext:
         except Exception:
             pass
 
+    @staticmethod
+    def _after_torch() -> None:
+        """The context launches on its own non-blocking stream: what torch has
+        queued on its stream (fills, uploads, copies of test data) must be done
+        before a kernel of this library reads or overwrites the same memory."""
+        torch.cuda.current_stream().synchronize()
+
     def _check(self, rc: int) -> None:
         if rc != capi.SG_OK:
             raise SgError(rc, self.lib.sg_hip_last_error(self.h).decode())
@@ -149,6 +156,8 @@ class SgContext:
         self.gather_batch_raw(self.gather_args(*args, **kw))
 
     def gather_batch_raw(self, a: capi.GatherArgs) -> None:
+        if not (a.flags & capi.F_ASYNC):
+            self._after_torch()
         rc = self.lib.sg_hip_gather_batch(self.h, C.byref(a))
         if rc != capi.SG_OK:
             self._check(rc)
@@ -183,6 +192,8 @@ class SgContext:
         self.scatter_batch_raw(self.scatter_args(*args, **kw))
 
     def scatter_batch_raw(self, a: capi.ScatterArgs) -> None:
+        if not (a.flags & capi.F_ASYNC):
+            self._after_torch()
         rc = self.lib.sg_hip_scatter_batch(self.h, C.byref(a))
         if rc != capi.SG_OK:
             self._check(rc)
@@ -203,6 +214,7 @@ class SgContext:
         a.req_first = req_first.data_ptr()
         a.req_token = req_token.data_ptr() if req_token is not None else None
         n_req, n_frag, n_left = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+        self._after_torch()
         self._check(self.lib.sg_hip_reassemble(self.h, C.byref(a), C.byref(n_req), C.byref(n_frag),
                                                C.byref(n_left)))
         return int(n_req.value), int(n_frag.value), int(n_left.value)
@@ -219,6 +231,7 @@ class SgContext:
             skb.len[i] = lens[i]
         skb.num_items = n
         fn = self.lib.sg_hip_scatter if scatter else self.lib.sg_hip_gather
+        self._after_torch()
         self._check(fn(self.h, C.byref(skb)))
 
     def swap_hdrs(self, hdr_ptrs: Sequence[int], profile: int, payload_size: int, mtu: int,
@@ -227,6 +240,7 @@ class SgContext:
         for i, p in enumerate(hdr_ptrs):
             hb.burst_items[i] = p
         hb.num_items = len(hdr_ptrs)
+        self._after_torch()
         self._check(self.lib.sg_hip_swap_hdrs(self.h, C.byref(hb), profile, payload_size, mtu, flags))
 
     def set_hdrs(self, hdr_ptrs: Sequence[int], template: bytes, token: int, profile: int,
@@ -237,6 +251,7 @@ class SgContext:
         hb.num_items = len(hdr_ptrs)
         assert len(template) >= 64
         t = (C.c_uint8 * 64).from_buffer_copy(bytes(template[:64]))
+        self._after_torch()
         self._check(self.lib.sg_hip_set_hdrs(self.h, C.byref(hb), t, token, profile, payload_size, mtu, flags))
 
 

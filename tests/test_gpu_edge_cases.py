@@ -420,6 +420,48 @@ def be_sum_rows(rows: np.ndarray) -> np.ndarray:
     return s
 
 
+@pytest.mark.parametrize("layout", ["arena", "arena-wrap", "tensor"])
+@pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64])
+def test_long_frames_summed_by_several_wavefronts(ctx, layout, profile):
+    """Jumbo response frames with the full UDP checksum: the payload sum of a
+    frame is put together from the partial sums of the wavefronts that copy its
+    sub-runs.  Both scatter kernels (rule declared / descriptor path), twice in
+    a row (the accumulators must be back at zero), with a response that crosses
+    the end of an arena mapped once, and with tensor-major outputs."""
+    flags = synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL
+    if layout == "tensor":
+        resp = [26400] * 5
+        w = synth.make_custom([100] * 5, resp, mtu=8800, slot_size=9216, seed=91, profile=profile, flags=flags,
+                              out_tensor_sizes=[10000, 16400])
+    else:
+        resp = [26401] * 5
+        w = synth.make_custom([100] * 5, resp, mtu=8800, slot_size=9216, seed=92, profile=profile, flags=flags)
+    print(f"case long summed frames layout={layout} profile={profile}", flush=True)
+    dw = DeviceWorkload(w)
+    ctx.set_cursor(0, 0)
+    dw.gather(ctx, use_frag_len=profile == synth.HDR_REF64)
+    exp, _, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    start = 0
+    if layout == "arena-wrap":
+        # rotate the response arena so that the batch starts 30000 bytes before its end
+        cap = dw.resp_app.cap
+        start = cap - 30000
+        dw.resp_arena.copy_(torch.roll(dw.resp_arena.clone(), start))
+    for fuse in (True, False, True):
+        ctx.set_cursor(1, start)
+        dw.tx_ring.copy_(to_dev(w.tx_ring_init, DEV))
+        dw.scatter(ctx, fuse=fuse)
+        if layout == "arena-wrap":
+            tx = w.tx_ring_init.copy()
+            src = np.roll(w.resp_payload, start)
+            oracle.scatter(w, w.ring, tx, src, arena_cap=cap, cursor=start)
+            exp_tx = tx
+        else:
+            exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
+        got = dw.tx_ring.cpu().numpy()
+        assert np.array_equal(got, exp_tx), f"fuse={fuse}: " + first_diff(got, exp_tx)
+
+
 def test_full_size_jumbo_checksums_verify(ctx):
     """Workload 5 at full size: every response frame's IPv4 and UDP checksum
     verifies to 0xffff the way a receiver would check it (RFC 1071 / 768), and
