@@ -47,6 +47,16 @@ __device__ __forceinline__ T sload(const T *p)
   return *(cptr)(uintptr_t)p;
 }
 
+// The same, issued where it stands: the optimizer may not sink it below a
+// branch into the block that uses the value, so independent table reads placed
+// side by side travel together instead of one round trip after the other.
+template <class T>
+__device__ __forceinline__ T sload_here(const T *p)
+{
+  typedef const volatile __attribute__((address_space(4))) T *cptr;
+  return *(cptr)(uintptr_t)p;
+}
+
 // Sum of the eight 16-bit little-endian words of a 16-byte chunk.
 __device__ __forceinline__ uint32_t words_sum(u32x4 v)
 {

@@ -539,8 +539,8 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   const uint32_t piece = LONG ? w - item * pieces : 0;
   if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  if (sload(status)) return;  // the descriptor pass refused the batch: move nothing
-  const u32x4 d = sload(desc + item);
+  const u32x4 d = sload_here(desc + item);  // asked for together with the status word
+  if (sload_here(status)) return;           // the descriptor pass refused the batch: move nothing
   if (d[1] == 0 || d[3] == kInvalidReq) return;
   const uint64_t ro = a.app.n_tensors == 0 ? sload(req_off + d[3]) : 0;
   uint8_t *pkt = const_cast<uint8_t *>(ring) + (size_t)d[0] * slot_size + hl;
@@ -721,23 +721,43 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
   constexpr bool SPLIT = LONG && !FULL_CSUM;  // several wavefronts per frame
   constexpr bool WHOLE_LONG = LONG && FULL_CSUM;  // one wavefront walks all sub-runs of its frame
-  const uint32_t w = item_of_wave(a.remap != 0);
-  const uint32_t pieces = SPLIT ? a.pieces : 1u;
+  // every argument of the common path in one burst of scalar loads
+  const u32x4 *desc = a.desc;
+  const uint64_t *req_off = a.req_off;
+  const uint32_t *first = a.first, *hdr_src_slot = a.hdr_src_slot;
+  const uint8_t *hdr_templates = a.hdr_templates, *rx = a.rx;
+  uint8_t *tx = a.tx;
+  const uint32_t rx_slot_size = a.rx_slot_size, rx_n_slots = a.rx_n_slots, tx_slot_size = a.tx_slot_size;
+  const uint32_t hl = a.hl, n_items = a.n_items, remap = a.remap, n_pieces = a.pieces;
+  const uint32_t *status = a.status;
+  SG_PIN(desc); SG_PIN(req_off); SG_PIN(first); SG_PIN(hdr_src_slot); SG_PIN(hdr_templates); SG_PIN(rx);
+  SG_PIN(tx); SG_PIN(rx_slot_size); SG_PIN(rx_n_slots); SG_PIN(tx_slot_size); SG_PIN(hl); SG_PIN(n_items);
+  SG_PIN(remap); SG_PIN(n_pieces); SG_PIN(status);
+  SG_PIN(a.app.n_tensors); SG_PIN(a.app.arena); SG_PIN(a.app.cap); SG_PIN(a.app.mirrored);
+  if (FUSED) {
+    SG_PIN(a.rule.item_slot); SG_PIN(a.rule.first); SG_PIN(a.rule.size); SG_PIN(a.rule.mtu);
+    SG_PIN(a.rule.per_req); SG_PIN(a.rule.n_slots); SG_PIN(a.rule.single_wrap); SG_PIN(a.rule.cursor_in);
+  }
+  const uint32_t w = item_of_wave(remap != 0);
+  const uint32_t pieces = SPLIT ? n_pieces : 1u;
   const uint32_t item = SPLIT ? w / pieces : w;
   const uint32_t piece = SPLIT ? w - item * pieces : 0;
-  if (item >= a.n_items) return;
+  if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
+  const bool from_template = hdr_templates != nullptr;
+  // independent table reads, asked for together
+  const uint32_t hs = from_template ? 0u : sload_here(hdr_src_slot + item);
   u32x4 d;
   uint32_t r, f0, nf;
   uint64_t ro;
   if (!FUSED) {
-    if (*a.status) return;  // the descriptor pass refused the batch: move nothing
-    d = a.desc[item];
+    d = sload_here(desc + item);
+    if (sload_here(status)) return;  // the descriptor pass refused the batch: move nothing
     r = d[3];
     if (r == kInvalidReq) return;
-    f0 = a.first[r];
-    nf = a.first[r + 1] - f0;
-    ro = a.app.n_tensors == 0 ? a.req_off[r] : 0;
+    f0 = sload(first + r);
+    nf = sload(first + r + 1) - f0;
+    ro = a.app.n_tensors == 0 ? sload(req_off + r) : 0;
   } else {
     uint32_t slot_i, len, off, i;
     const uint32_t bad = rule_desc(a.rule, a.app, item, a.n_items, piece == 0 ? lane : 1u, &slot_i, &len,
@@ -750,26 +770,24 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     f0 = item - i;
     nf = a.rule.per_req;
   }
-  uint8_t *slot = a.tx + (size_t)d[0] * a.tx_slot_size;
+  uint8_t *slot = tx + (size_t)d[0] * tx_slot_size;
   // where the header comes from; a frame whose header source is out of range is left alone by
   // all of its pieces
-  const bool from_template = a.hdr_templates != nullptr;
   const uint8_t *hin;
-  HdrFields hf{a.hl, a.ref64, a.flags, item - f0, nf, d[1], 0, 0, 0};
+  HdrFields hf{hl, a.ref64, a.flags, item - f0, nf, d[1], 0, 0, 0};
   if (from_template) {
-    hin = a.hdr_templates + (size_t)r * 64;
+    hin = hdr_templates + (size_t)r * 64;
     hf.from_template = 1;
     if (a.req_token) {
       hf.set_token = 1;
       hf.token = a.req_token[r];
     }
   } else {
-    const uint32_t hs = a.hdr_src_slot[item];
-    if (hs >= a.rx_n_slots) {
+    if (hs >= rx_n_slots) {
       if (lane == 0 && piece == 0) atomicOr(a.status, kStBadSlot);
       return;
     }
-    hin = a.rx + (size_t)hs * a.rx_slot_size;
+    hin = rx + (size_t)hs * rx_slot_size;
   }
 
   if (SPLIT && piece != 0) {
@@ -777,8 +795,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     uint8_t *from;
     if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
       uint32_t o, n;
-      sub_run(slot + a.hl, d[1], piece, &o, &n);
-      if (n) copy_run<false>(from + o, slot + a.hl + o, n, lane);
+      sub_run(slot + hl, d[1], piece, &o, &n);
+      if (n) copy_run<false>(from + o, slot + hl + o, n, lane);
     }
     return;
   }
@@ -786,7 +804,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   // (the TX slot may be the very slot the header comes from);
   // header bytes and payload chunks are fetched together; the header arithmetic
   // then runs while the payload is still on its way
-  const uint32_t raw = hdr_fetch(hin, lane, a.hl, !from_template);
+  const uint32_t raw = hdr_fetch(hin, lane, hl, !from_template);
   uint32_t hb = 0, acc = 0;
   uint8_t *from = nullptr;
   const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
@@ -794,20 +812,20 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   uint32_t first_len = d[1];
   if (SPLIT && plain) {
     uint32_t o;
-    sub_run(slot + a.hl, d[1], 0, &o, &first_len);
+    sub_run(slot + hl, d[1], 0, &o, &first_len);
   }
-  if (plain && !WHOLE_LONG) run_begin(rs, from, slot + a.hl, first_len, lane);
+  if (plain && !WHOLE_LONG) run_begin(rs, from, slot + hl, first_len, lane);
   if (!FULL_CSUM) hb = hdr_finish(raw, lane, hf, 0);
   if (plain) {
-    if (WHOLE_LONG) acc = copy_long_run<FULL_CSUM, 2>(from, slot + a.hl, d[1], lane);
+    if (WHOLE_LONG) acc = copy_long_run<FULL_CSUM, 2>(from, slot + hl, d[1], lane);
     else acc = run_end<FULL_CSUM>(rs, lane);
   } else if (d[1]) {
-    acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + a.hl, d[1], lane);
+    acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + hl, d[1], lane);
   }
   if (FULL_CSUM) hb = hdr_finish(raw, lane, hf, wave_sum(acc));
   // the payload went past the header only, so a TX slot that is the header's own
   // source still held the request header when it was fetched above
-  if (lane < a.hl) slot[lane] = (uint8_t)hb;
+  if (lane < hl) slot[lane] = (uint8_t)hb;
 }
 
 // ---------------------------------------------------------------------------
