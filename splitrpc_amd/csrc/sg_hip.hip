@@ -405,15 +405,17 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
   uint32_t bad = 0;
   *r = item / g.per_req;
   *i = item - *r * g.per_req;
+  // the three table reads are independent: asked for together
+  *slot = sload_here(g.item_slot + item);
+  const uint32_t first_r = sload_here(g.first + *r);
+  uint64_t c0 = app.n_tensors == 0 ? sload_here(g.cursor_in) : 0;
   *off = *i * g.mtu;
   const uint64_t rem = g.size - *off;
   *len = (uint32_t)(rem <= g.mtu ? rem : g.mtu);
-  *slot = g.item_slot[item];
   if (*slot >= g.n_slots) bad |= kStBadSlot;
-  if (*i == 0 && g.first[*r] != item) bad |= kStBadTable;
+  if (*i == 0 && first_r != item) bad |= kStBadTable;
   *req_off = 0;
   if (app.n_tensors == 0) {
-    uint64_t c0 = *g.cursor_in;
     if (c0 >= app.cap) c0 %= app.cap;  // only after a set_cursor beyond the capacity
     uint64_t o = c0 + (uint64_t)*r * g.size;
     if (g.single_wrap) o = o >= app.cap ? o - app.cap : o;  // n_req * size <= capacity
