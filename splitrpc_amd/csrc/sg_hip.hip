@@ -12,7 +12,11 @@
 //   k_gather   one wavefront per fragment run: ring slot payload -> tensor.
 //   k_scatter  one wavefront per response frame: tensor -> TX slot payload,
 //              header rewrite, checksums.
-// plus k_copy_runs / k_swap_hdrs for the per-request entry points.
+// When the caller declares one request size and the fragmenting rule, the
+// descriptor pass is skipped: k_gather_rule and the FUSED form of k_scatter
+// derive every offset themselves and hold the tables against the rule.
+// Plus k_copy_runs / k_swap_hdrs for the per-request entry points and k_ra_*
+// for sorting a burst of arrivals into requests (sg_hip_reassemble).
 #include <hip/hip_runtime.h>
 
 #include <errno.h>
