@@ -655,6 +655,9 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
       else if (o + len > cap) plain = false;  // crosses the end of an arena mapped once
     }
     to = dst + o;
+  } else if (opts & kOptMultiTensor) {
+    // tensor-major buffers: a fragment inside one tensor still takes the fast path
+    plain = plain_target(a.app, 0, r, off, len, &to);
   } else {
     to = dst + (uint64_t)r * size + off;
   }
