@@ -100,3 +100,41 @@ def test_bad_arrival_is_refused(ctx):
     assert e.value.code == capi.SG_E_DATA
     got = device_reassemble(ctx, w, w.arrivals)  # and the context recovers
     assert np.array_equal(got[0], w.frag_slot)
+
+
+@pytest.mark.parametrize("kind", ["echo", "vec_add"])
+def test_client_requests_served_on_the_device_end_to_end(ctx, kind):
+    """A burst of the reference clients' requests (REF64 headers) goes through
+    reassembly, gather, the "model" and scatter on the device, and the
+    clients' own checks (lib_loadgen/*_client.cc) accept every response."""
+    import torch
+    from splitrpc_amd import capi, loadgen
+    from splitrpc_amd.engine import AppRef, DeviceWorkload, to_dev
+    size, rsize = (30000, 30000) if kind == "echo" else (9000, 5000)
+    w = loadgen.client_workload(kind, 37, size, resp_size=rsize, flags=synth.F_UDP_CSUM_PSEUDO | synth.F_REF_QUIRKS)
+    print(f"case client {kind} n_req={w.n_req} frags={w.n_frags}", flush=True)
+    dw = DeviceWorkload(w)
+    dev = "cuda"
+    ln = np.zeros(w.n_slots, np.uint32)
+    ln[w.frag_slot] = w.frag_len
+    fs = torch.zeros(w.n_frags, dtype=torch.int32, device=dev)
+    fl = torch.zeros(w.n_frags, dtype=torch.int32, device=dev)
+    rf = torch.zeros(8193, dtype=torch.int32, device=dev)
+    n_req, n_frag, n_left = ctx.reassemble(dw.rx, dw.arrivals, w.n_frags, fs, fl, rf, len_nic=to_dev(ln, dev),
+                                           req_size=size)
+    assert (n_req, n_frag, n_left) == (w.n_req, w.n_frags, 0)
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    ctx.gather_batch(dw.rx, fs, fl, rf, n_req, n_frag, dw.req_app, dw.req_offsets,
+                     flags=capi.F_RULE_FRAGS, fixed_req_size=size, mtu=w.mtu)
+    if kind == "echo":
+        resp_app = dw.req_app
+        tx, tx_slot, hsrc, first = dw.rx, fs, fs, rf          # answered in place, frame for frame
+        n_frames = n_frag
+    else:
+        served = (dw.req_arena.view(w.n_req, size)[:, :rsize] + 1).contiguous().view(-1)   # the model
+        resp_app = AppRef(arena=served, cap=int(served.numel()))
+        tx, tx_slot, hsrc, first, n_frames = dw.tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first, dw.n_frames
+    ctx.scatter_batch(dw.rx, tx, tx_slot, hsrc, first, None, rsize, n_req, n_frames, w.mtu, resp_app, None, w.flags)
+    out = (dw.ring if kind == "echo" else dw.tx_ring).cpu().numpy()
+    assert loadgen.verify_responses(w, out, kind) == 0

@@ -148,3 +148,36 @@ def test_pool_grows_when_exhausted(host):
 def test_pointer_ring_multi_producer_multi_consumer(host):
     assert host.sgh_ring_stress(4, 20000, 64) == 1
     assert host.sgh_ring_stress(2, 1000, 2) == 1
+
+
+# ---------------------------------------------------------------- client patterns (load generator)
+
+def test_client_patterns_and_checks_through_the_cpu_path():
+    """The reference clients' request patterns and reply checks
+    (lib_loadgen/echo_client.cc, vec_add_client.cc) around the oracle's gather
+    and scatter: what the echo client gets back passes its own check, a
+    flipped byte does not."""
+    import oracle
+    from splitrpc_amd import loadgen, synth
+    assert bytes(loadgen.create_echo_request(8193)[[0, 1, 8191, 8192]]) == bytes([0xDE, 2, 2, 0xAD])
+    assert bytes(loadgen.create_vec_add_request(6)) == bytes([0xDE, 0xAD, 0xBE, 0xEF, 0xDE, 0xAD])
+    assert loadgen.complete_echo_reply(loadgen.create_echo_request(20000), 20000) == 0
+    assert loadgen.complete_echo_reply(loadgen.create_echo_request(20000), 20001) == 1
+    assert loadgen.complete_vec_add_reply(loadgen.create_vec_add_request(64) + 1, 64) == 0
+    assert loadgen.complete_vec_add_reply(loadgen.create_vec_add_request(64), 64) == 1
+
+    w = loadgen.client_workload("echo", 5, 20000)
+    assert w.profile == synth.HDR_REF64 and w.tx_in_place
+    arena, _, _ = oracle.gather(w, use_frag_len=True)
+    ring = w.ring.copy()
+    oracle.scatter(w, ring, ring, arena)
+    assert loadgen.verify_responses(w, ring, "echo") == 0
+    ring[int(w.tx_slot[3]) * w.slot_size + 64 + 7] ^= 1
+    assert loadgen.verify_responses(w, ring, "echo") == 1
+
+    w = loadgen.client_workload("vec_add", 4, 5000, resp_size=3000)
+    arena, _, _ = oracle.gather(w, use_frag_len=True)
+    served = (arena.reshape(4, 5000)[:, :3000].astype(np.uint16) + 1).astype(np.uint8).reshape(-1)  # the model
+    tx = w.tx_ring_init.copy()
+    oracle.scatter(w, w.ring, tx, served)
+    assert loadgen.verify_responses(w, tx, "vec_add") == 0
