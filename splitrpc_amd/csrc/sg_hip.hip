@@ -1597,8 +1597,8 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   if (a->n_req == 0) return SG_OK;
   if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
   if (a->n_frags > c->max_frames) return fail(c, SG_E_INVAL, "n_frags %u > max_frames %u of this context", a->n_frags, c->max_frames);
-  if (!a->frag_slot || !a->req_first) return fail(c, SG_E_INVAL, "null fragment tables");
-  if (!a->frag_len && a->ring.hdr_profile != SG_HDR_BL58)
+  if ((!a->frag_slot && a->n_frags) || !a->req_first) return fail(c, SG_E_INVAL, "null fragment tables");
+  if (!a->frag_len && a->n_frags && a->ring.hdr_profile != SG_HDR_BL58)
     return fail(c, SG_E_INVAL, "REF64 headers carry no payload length: frag_len is required");
   AppDev app;
   uint64_t max_req_bytes;
@@ -1718,7 +1718,7 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   if (a->n_req == 0) return SG_OK;
   if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
   if (a->n_frames > c->max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u of this context", a->n_frames, c->max_frames);
-  if (!a->tx_slot || !a->resp_first || (!a->hdr_src_slot && !a->hdr_templates))
+  if (!a->resp_first || (a->n_frames && (!a->tx_slot || (!a->hdr_src_slot && !a->hdr_templates))))
     return fail(c, SG_E_INVAL, "null frame tables");
   const uint32_t hl = hdr_len_of(a->tx.hdr_profile);
   if (a->mtu == 0 || (uint64_t)a->mtu + hl > a->tx.slot_size)
