@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the dominant kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of this file scaled by a plain 512 MiB copy in the same runs (FETCH_SIZE x 2.000,
 # WRITE_SIZE x 1.000): 340.2 MB read + 308.3 MB written.  Known for the default call only.
-MEASURED_TRAFFIC = {(2, 32, "k_gather"): 648.5e6}
+MEASURED_TRAFFIC = {(2, 32, "k_gather"): 652.2e6}
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 

@@ -31,9 +31,19 @@ __device__ __forceinline__ uint32_t load32_any(const uint8_t *p)
   return reinterpret_cast<const u32_unaligned *>(p)->v;
 }
 
+// Payload chunks are touched once: read from a ring slot, written to a tensor
+// (or the other way round) and not looked at again by this library.  The
+// nontemporal hint on both sides keeps them from displacing each other in the
+// caches; measured on the 32-batch gather it is worth 8 % (stores alone 5 %,
+// loads alone -5 %), and a plain 16-byte-per-lane copy kernel gains the same.
 __device__ __forceinline__ void store16_aligned(uint8_t *p, u32x4 v)
 {
-  *reinterpret_cast<u32x4 *>(p) = v;
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+}
+
+__device__ __forceinline__ u32x4 load16_aligned(const uint8_t *p)
+{
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
 }
 
 // Load through the scalar data cache: for wave-uniform addresses of data that
@@ -182,8 +192,8 @@ __device__ __forceinline__ void run_begin(RunState &r, const uint8_t *__restrict
   r.v0 = (u32x4){0, 0, 0, 0};
   r.v1 = (u32x4){0, 0, 0, 0};
   if (body) {
-    if (lane <= r.lim) r.v0 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)lane << 4));
-    if (63u + lane <= r.lim) r.v1 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)(63u + lane) << 4));
+    if (lane <= r.lim) r.v0 = load16_aligned(r.sa + ((size_t)lane << 4));
+    if (63u + lane <= r.lim) r.v1 = load16_aligned(r.sa + ((size_t)(63u + lane) << 4));
   }
 }
 
@@ -208,8 +218,8 @@ __device__ __forceinline__ uint32_t run_end(RunState &r, uint32_t lane)
   for (uint32_t base = 126; base < r.body; base += 126) {
     const uint32_t c0 = base + lane, c1 = base + 63u + lane;
     u32x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-    if (c0 <= r.lim) v0 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c0 << 4));
-    if (c1 <= r.lim) v1 = *reinterpret_cast<const u32x4 *>(r.sa + ((size_t)c1 << 4));
+    if (c0 <= r.lim) v0 = load16_aligned(r.sa + ((size_t)c0 << 4));
+    if (c1 <= r.lim) v1 = load16_aligned(r.sa + ((size_t)c1 << 4));
     const u32x4 q0 = realign(v0, r.p);
     const u32x4 q1 = realign(v1, r.p);
     if (lane < 63 && c0 < r.body) {
