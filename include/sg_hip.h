@@ -257,7 +257,13 @@ int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_te
  * semantics are those of P2pRpcSgCpuEngine::gather / scatter
  * (src/p2p_rpc_sg_engine.h:150-164) applied to every request of the batch,
  * with request offsets taken from the bump ring.  Synchronous unless
- * SG_F_ASYNC is set. */
+ * SG_F_ASYNC is set; an SG_F_ASYNC call does nothing on the stream but launch
+ * kernels (no allocation, no copy, no memset).  The bump-ring cursor of an
+ * arena lives in two device words, each call reading the one the previous
+ * call wrote; which is which is fixed when the call is issued, so a caller
+ * that records calls into a HIP graph records an even number of calls per
+ * arena (or uses an arena of exactly one batch, where the cursor always
+ * returns to the same place) for replays to continue the ring. */
 int sg_hip_gather_batch(sg_hip_ctx *ctx, const sg_gather_args *args);
 int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
 
