@@ -227,6 +227,39 @@ def per_request_calls(ctx, dw, calls: int = 300):
             "GBps": round((2 * size + 16 * int(skbs[0].num_items)) / dt / 1e9, 2)}
 
 
+def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, replays: int = 50) -> float:
+    """Seconds per step of the single-batch call when `steps` steps (an even
+    number of calls per arena) are recorded into one HIP graph on the context's
+    stream and the graph is replayed: the launch-bound loop without the
+    per-launch host cost."""
+    import torch
+    from splitrpc_amd import capi
+    from splitrpc_amd.engine import SgContext
+    stream = torch.cuda.Stream()
+    ctx = SgContext(0, max_reqs=max(4096, w.n_req), max_frames=max(65536, w.n_frags, w.n_resp_frames),
+                    stream=stream.cuda_stream)
+    pool = Pool(w, 1, rotate_mb, extra, rule=rule)
+    for i in range(len(pool.items)):
+        pool.step(ctx, i, capi.F_ASYNC)
+    ctx.sync()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        for i in range(steps):
+            pool.step(ctx, i, capi.F_ASYNC)
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        g.replay()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / (replays * steps)
+    ctx.sync()
+    ctx.close()
+    return dt
+
+
 def cpu_baseline(w, seconds: float):
     """The CPU oracle (a restatement of the reference's CPU scatter-gather
     path) timed on this host over rotated ring copies: on one thread -- the
@@ -321,6 +354,9 @@ def main() -> int:
                   "k_gather_GBps": round(p1.gather_bytes / (k1["k_gather"][0] * 1e-3) / 1e9, 1)
                   if k1["k_gather"][0] > 0 else None}
         del p1
+        sg = graph_step_time(w, extra, not a.general, a.rotate_mb)
+        single["hip_graph_ms_per_step"] = round(sg * 1e3, 5)
+        single["hip_graph_requests_per_sec"] = round(w.n_req / sg, 1)
 
     per_req = per_request_calls(ctx, pool.items[0]) if not w.in_tensor_sizes else None
     rps = {WORKLOAD_NAMES[a.workload]: round(pool.n_req / sec, 1)}
