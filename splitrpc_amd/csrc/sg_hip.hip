@@ -33,6 +33,19 @@
 using namespace sg;
 
 namespace {
+// A kernel refuses part of its input: the bits go into the device status word
+// (later kernels of the call look at it and then move nothing) and a flag goes
+// up in pinned host memory, where the host finds it after synchronizing
+// without having to copy anything back.  The flag is a plain store of a
+// constant: whoever writes, the value is the same.
+__device__ __forceinline__ void refuse(uint32_t *status, volatile uint32_t *flag, uint32_t bits)
+{
+  atomicOr(status, bits);
+  *flag = 1u;
+}
+}  // namespace
+
+namespace {
 
 // ---------------------------------------------------------------------------
 // device-side argument blocks
@@ -75,6 +88,7 @@ struct PrepArgs {
   uint64_t *cursor_out;
   uint64_t *offsets_out;
   uint32_t *status;
+  volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
 
 // Exclusive scan over the threads of a workgroup of BLOCK threads, built from
@@ -170,7 +184,7 @@ __device__ __forceinline__ void prep_finish(const PrepArgs &a, uint32_t r, uint6
   if (!a.packed && total > a.max_req_bytes) bad |= kStBadSize;
   if (a.packed && total > a.cap) bad |= kStBadSize;
   if (a.mode == 0 && a.fixed_size && total != a.fixed_size) bad |= kStBadSize;
-  if (bad) atomicOr(a.status, bad);
+  if (bad) refuse(a.status, a.status_flag, bad);
   a.req_size[r] = total;
   if (a.packed && a.fixed_offsets) {
     // bump ring with equal sizes: ret = base + off; off = (off + size) % capacity
@@ -211,7 +225,7 @@ __global__ __launch_bounds__(BLOCK) void k_prep_block(PrepArgs a)
   }
   // fold the status bits of all threads into thread 0
   bad = wave_or(bad);
-  if ((threadIdx.x & (kWave - 1)) == 0 && bad) atomicOr(a.status, bad);
+  if ((threadIdx.x & (kWave - 1)) == 0 && bad) refuse(a.status, a.status_flag, bad);
   if (threadIdx.x == 0) prep_finish(a, r, carry, 0);
 }
 
@@ -284,7 +298,7 @@ __device__ __forceinline__ void scan_emit(const PrepArgs &a, uint32_t q0, const 
 // particular order.  Refused instead.
 __device__ __forceinline__ void scan_check_batch(const PrepArgs &a, uint64_t batch_bytes)
 {
-  if (a.mode == 0 && batch_bytes > a.cap) atomicOr(a.status, kStBadSize);
+  if (a.mode == 0 && batch_bytes > a.cap) refuse(a.status, a.status_flag, kStBadSize);
 }
 
 __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
@@ -396,6 +410,7 @@ struct GatherArgs {
   uint32_t remap;
   uint32_t pieces;  // wavefronts per fragment
   uint32_t *status;
+  volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   AppDev app;
 };
 
@@ -593,6 +608,7 @@ struct GatherRuleArgs {
   uint64_t *offsets_out;
   uint64_t *cursor_out;
   uint32_t *status;
+  volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   AppDev app;  // consulted for several tensor-major buffers only
 };
 constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
@@ -627,7 +643,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint64_t rem = size - off;
   const uint32_t len = (uint32_t)(rem <= mtu ? rem : mtu);
   if (slot >= n_slots) {
-    if (lane == 0 && piece == 0) atomicOr(a.status, kStBadSlot);
+    if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
     return;
   }
   uint8_t *pkt = const_cast<uint8_t *>(ring) + (size_t)slot * slot_size;
@@ -691,7 +707,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     const bool as_ruled = (check_hdr ? hdr_len : sload(a.frag_len + item)) == len;
     if (!as_ruled) bad |= kStNotRule;
     if (i == 0 && sload(a.first + r) != item) bad |= kStBadTable;
-    if (bad && lane == 0) atomicOr(a.status, bad);
+    if (bad && lane == 0) refuse(a.status, a.status_flag, bad);
   }
 }
 
@@ -714,6 +730,7 @@ struct ScatterArgs {
   uint32_t remap;
   uint32_t pieces;  // wavefronts per frame
   uint32_t *status;
+  volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   RuleArgs rule;
   AppDev app;
 };
@@ -772,7 +789,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     const uint32_t bad = rule_desc(a.rule, a.app, item, a.n_items, piece == 0 ? lane : 1u, &slot_i, &len,
                                    &off, &r, &i, &ro);
     if (bad) {
-      if (lane == 0 && piece == 0) atomicOr(a.status, bad);
+      if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, bad);
       return;
     }
     d = (u32x4){slot_i, len, off, r};
@@ -793,7 +810,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     }
   } else {
     if (hs >= rx_n_slots) {
-      if (lane == 0 && piece == 0) atomicOr(a.status, kStBadSlot);
+      if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
       return;
     }
     hin = rx + (size_t)hs * rx_slot_size;
@@ -919,8 +936,9 @@ struct RaArgs {
   // outputs
   uint32_t *frag_slot, *frag_len, *req_first;
   uint64_t *req_token;
-  uint32_t *counts;  // [0] requests, [1] fragments, [2] arrivals left out
+  volatile uint32_t *counts;  // pinned host memory: [0] requests, [1] fragments
   uint32_t *status;
+  volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
 
 constexpr uint32_t kRaNoCell = 0xffffffffu;
@@ -966,7 +984,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
   if (in_range) {
     const uint32_t slot = a.arrivals[i];
     if (slot >= a.n_slots) {
-      atomicOr(a.status, kStBadSlot);
+      refuse(a.status, a.status_flag, kStBadSlot);
     } else {
       const uint8_t *h = a.ring + (size_t)slot * a.slot_size;
       const uint32_t t0 = load32_any(h + 42), t1 = load32_any(h + 46);
@@ -982,7 +1000,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
       }
       const uint32_t hl = a.ref64 ? 64u : 58u;
       if (len > a.slot_size - hl) {
-        atomicOr(a.status, kStBadLen);
+        refuse(a.status, a.status_flag, kStBadLen);
         len = 0;
       } else {
         pending = token != 0;  // token 0: dropped (src/transport/dpdk_transport_ng.h:231)
@@ -1066,11 +1084,10 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
   if (threadIdx.x == 0) {
     a.blk[a.n_blocks] = run;
     const uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
-    a.counts[0] = n_req;
+    a.counts[0] = n_req;  // straight into pinned host memory: nothing to copy back
     a.counts[1] = n_frag;
-    a.counts[2] = 0;  // k_ra_emit counts the arrivals left out
     if (n_req <= a.max_req) a.req_first[n_req] = n_frag;
-    else atomicOr(a.status, kStBadTable);
+    else refuse(a.status, a.status_flag, kStBadTable);
   }
 }
 
@@ -1081,10 +1098,8 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
 __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
 {
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  bool left_out = false;
   if (i < a.n) {
     const uint32_t cell = a.arr_cell[i];
-    left_out = true;
     if (cell != kRaNoCell) {
       const uint32_t last = a.last[cell];
       const unsigned long long p = a.arr_pack[last];
@@ -1092,14 +1107,13 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
         const unsigned long long v = (p & ~(1ull << 63)) + a.blk[last / kRaBlock];
         const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v;
         if (r < a.max_req) {  // else refused by k_ra_scan
-          left_out = false;
           const uint32_t n = a.cnt[cell];
           const uint32_t fidx = a.arr_fidx[i];
           if (fidx < n) {
             a.frag_slot[first + fidx] = a.arrivals[i];
             a.frag_len[first + fidx] = a.arr_len[i];
           } else {
-            atomicOr(a.status, kStBadTable);  // a sequence number beyond the request's fragments
+            refuse(a.status, a.status_flag, kStBadTable);  // a sequence number beyond the request's fragments
           }
           if (i == last) {
             a.req_first[r] = first;
@@ -1109,10 +1123,6 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
       }
     }
   }
-  // arrivals whose request did not complete: one add per wavefront
-  const unsigned long long m = __ballot(left_out);
-  if (m && (threadIdx.x & (kWave - 1)) == (uint32_t)(__ffsll((long long)m) - 1))
-    atomicAdd(&a.counts[2], (uint32_t)__popcll(m));
 }
 
 // Wipes the cells this call used, so that the table is empty for the next one.
@@ -1159,7 +1169,8 @@ struct sg_hip_ctx {
   Run *h_runs = nullptr;
   uint32_t h_runs_cap = 0;
   uint64_t *h_ptrs = nullptr;
-  uint32_t *h_status = nullptr;  // pinned mirror of status
+  uint32_t *h_status = nullptr;  // pinned: [0] copy of status (read back only after a refusal), [1] the refusal flag
+  volatile uint32_t *h_flag = nullptr;
   // profiling
   bool profiling = false;
   std::vector<EvPair> ev_used, ev_free;
@@ -1168,7 +1179,7 @@ struct sg_hip_ctx {
   // reassembly scratch, allocated by the first sg_hip_reassemble call
   void *ra_mem = nullptr;
   uint32_t ra_cells = 0;  // hash table size (power of two >= 2 * max_frames)
-  uint32_t *h_counts = nullptr;  // pinned: requests, fragments, arrivals left out
+  uint32_t *h_counts = nullptr;  // pinned: requests, fragments (written by k_ra_scan itself)
   char err[512] = {0};
 };
 
@@ -1386,7 +1397,9 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   c->h_runs_cap = 8192;
   HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
   HIP_TRY(nullptr, hipHostMalloc(&c->h_ptrs, sizeof(uint64_t) * (SG_MAX_BI_SIZE + 8), hipHostMallocDefault));
-  HIP_TRY(nullptr, hipHostMalloc(&c->h_status, sizeof(uint32_t), hipHostMallocDefault));
+  HIP_TRY(nullptr, hipHostMalloc(&c->h_status, 2 * sizeof(uint32_t), hipHostMallocDefault));
+  c->h_status[0] = c->h_status[1] = 0;
+  c->h_flag = c->h_status + 1;
   HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
   return SG_OK;
 }
@@ -1436,14 +1449,16 @@ int sg_hip_sync(sg_hip_ctx *c)
 {
   if (!c) return SG_E_INVAL;
   DeviceGuard g(c->device);
-  HIP_TRY(c, hipMemcpyAsync(c->h_status, c->status, sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
   HIP_TRY(c, hipStreamSynchronize(c->stream));
   int rc = prof_drain(c);
   if (rc != SG_OK) return rc;
-  const uint32_t st = *c->h_status;
-  if (st) {
+  if (*c->h_flag) {
+    // the rare path: fetch the bits, then clear both words
+    HIP_TRY(c, hipMemcpyAsync(c->h_status, c->status, sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(c, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
     HIP_TRY(c, hipStreamSynchronize(c->stream));
+    *c->h_flag = 0;
+    const uint32_t st = c->h_status[0];
     return fail(c, SG_E_DATA, "kernel refused input:%s%s%s%s%s%s",
                 (st & kStBadSlot) ? " slot index beyond ring;" : "",
                 (st & kStBadLen) ? " fragment longer than a slot holds;" : "",
@@ -1639,6 +1654,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.first = a->req_first;
     ga.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
     ga.status = c->status;
+    ga.status_flag = c->h_flag;
     ga.app = app;
     ga.pieces = pieces_for(a->mtu);
     uint32_t grid, remap;
@@ -1680,6 +1696,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   if (p.packed) c->parity[0] ^= 1u;
   p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
   p.status = c->status;
+  p.status_flag = c->h_flag;
   rc = launch_prep(c, p);
   if (rc != SG_OK) return rc;
 
@@ -1693,6 +1710,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.hl = p.hl;
     ga.n_items = a->n_frags;
     ga.status = c->status;
+    ga.status_flag = c->h_flag;
     ga.app = app;
     ga.pieces = pieces_for(p.slot_size - p.hl);
     uint32_t grid;
@@ -1753,6 +1771,7 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.flags = a->flags & 0xfu;
     sa.n_items = a->n_frames;
     sa.status = c->status;
+    sa.status_flag = c->h_flag;
     sa.app = app;
     sa.rule.item_slot = a->tx_slot;
     sa.rule.first = a->resp_first;
@@ -1803,6 +1822,7 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   if (p.packed) c->parity[1] ^= 1u;
   p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
   p.status = c->status;
+  p.status_flag = c->h_flag;
   rc = launch_prep(c, p);
   if (rc != SG_OK) return rc;
 
@@ -1825,6 +1845,7 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.flags = a->flags & 0xfu;
     sa.n_items = a->n_frames;
     sa.status = c->status;
+    sa.status_flag = c->h_flag;
     sa.app = app;
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
@@ -1902,8 +1923,9 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_re
   r.frag_len = a->frag_len;
   r.req_first = a->req_first;
   r.req_token = a->req_token;
-  r.counts = reinterpret_cast<uint32_t *>(c->req_size);  // the descriptor pass's scratch is idle here
+  r.counts = c->h_counts;
   r.status = c->status;
+  r.status_flag = c->h_flag;
 
   const uint32_t g256 = (a->n_arrivals + 255) / 256;
   rc = prof_begin(c, 5);
@@ -1915,12 +1937,12 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_re
   k_ra_wipe<<<g256, 256, 0, c->stream>>>(r);
   rc = prof_end(c);
   if (rc != SG_OK) return rc;
-  HIP_TRY(c, hipMemcpyAsync(c->h_counts, r.counts, 3 * sizeof(uint32_t), hipMemcpyDeviceToHost, c->stream));
   rc = finish(c, 0);
   if (rc != SG_OK) return rc;
   if (n_req_out) *n_req_out = c->h_counts[0];
   if (n_frags_out) *n_frags_out = c->h_counts[1];
-  if (n_left_out) *n_left_out = c->h_counts[2];
+  // every arrival either belongs to a request that completed or is left out
+  if (n_left_out) *n_left_out = a->n_arrivals - c->h_counts[1];
   return SG_OK;
 }
 
