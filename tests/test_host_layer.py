@@ -181,3 +181,29 @@ def test_client_patterns_and_checks_through_the_cpu_path():
     tx = w.tx_ring_init.copy()
     oracle.scatter(w, w.ring, tx, served)
     assert loadgen.verify_responses(w, tx, "vec_add") == 0
+
+
+# ---------------------------------------------------------------- sanitizers on the host layer
+
+@pytest.mark.parametrize("san", ["thread", "address,undefined"])
+def test_rings_and_pool_under_sanitizers(san, tmp_path):
+    """The request pool and its rings between a receive and a shunter thread,
+    built with the thread sanitizer and with the address + undefined-behaviour
+    sanitizers (host code only: tests/host_sanitize.cpp)."""
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no g++")
+    exe = str(tmp_path / "host_sanitize")
+    cmd = [gxx, "-std=c++17", "-O1", "-g", f"-fsanitize={san}", "-fno-sanitize-recover=all",
+           "-I", os.path.join(root, "splitrpc_amd", "host"), "-I", os.path.join(root, "include"),
+           os.path.join(root, "tests", "host_sanitize.cpp"), "-o", exe, "-lpthread"]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    if built.returncode != 0 and "sanitize" in built.stderr and "cannot find" in built.stderr:
+        pytest.skip("sanitizer runtime not installed")
+    assert built.returncode == 0, built.stderr[-2000:]
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-3000:]
+    assert "host sanitize: ok" in run.stdout
