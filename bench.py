@@ -58,7 +58,7 @@ def parse():
     return ap.parse_args()
 
 
-DEFAULT_BPL = {1: 256, 2: 32, 3: 64, 4: 8, 5: 4}
+DEFAULT_BPL = {1: 2048, 2: 32, 3: 512, 4: 8, 5: 4}
 
 
 class Pool:
