@@ -612,37 +612,13 @@ struct GatherRuleArgs {
   AppDev app;  // consulted for several tensor-major buffers only
 };
 constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
-// average fragment size below which a wavefront takes two fragments
-constexpr uint64_t kPairBelow = 1200;
 // slots start at 16-byte aligned addresses: the header's length field can be read as part of
 // the aligned chunk at byte 48 (a ring only has to start at an even address)
 constexpr uint32_t kOptHdrChunk = 16u;
 
-// One fragment of a rule-declared batch as its wavefront sees it.
-struct RuleItem {
-  uint32_t item, r, i, off, len;
-  uint8_t *pkt;
-  uint8_t *to;
-  uint64_t ro;
-  bool live;       // the wavefront has this item and its slot index is in range
-  bool plain;      // one contiguous destination
-  bool check_hdr;  // the real length comes from the slot's header
-  u32x4 hc;
-  uint32_t hv;
-  uint32_t sub_off, sub_len;
-  RunState rs;
-};
-
-// K fragments per wavefront (LONG: one sub-run of one fragment).  Short
-// fragments leave a wavefront's life -- a few memory round trips, whatever the
-// size -- as the limit: with K = 2 the loads of both fragments share those
-// round trips.  The host picks K = 2 below an average fragment size of
-// kPairBelow bytes (measured: 6 % on 1400/648-byte and 1400/1400/336-byte
-// requests, nothing either way on 1400-byte fragments).
-template <bool LONG, int K>
+template <bool LONG>
 __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
 {
-  static_assert(!LONG || K == 1, "sub-runs of long fragments go one per wavefront");
   const uint8_t *ring = a.ring;
   const uint32_t *frag_slot = a.frag_slot;
   uint8_t *dst = a.dst;
@@ -655,102 +631,83 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   SG_PIN(pieces); SG_PIN(opts);
 
   const uint32_t w = item_of_wave((opts & kOptRemap) != 0);
-  const uint32_t item0 = LONG ? w / pieces : w * K;
-  const uint32_t piece = LONG ? w - item0 * pieces : 0;
-  if (item0 >= n_items) return;
+  const uint32_t item = LONG ? w / pieces : w;
+  const uint32_t piece = LONG ? w - item * pieces : 0;
+  if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t slot = sload(frag_slot + item);
   uint64_t c0 = cap ? sload(cursor_in) : 0;
-  if (cap && c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
+  const uint32_t r = item / per_req;
+  const uint32_t i = item - r * per_req;
+  const uint32_t off = i * mtu;
+  const uint64_t rem = size - off;
+  const uint32_t len = (uint32_t)(rem <= mtu ? rem : mtu);
+  if (slot >= n_slots) {
+    if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
+    return;
+  }
+  uint8_t *pkt = const_cast<uint8_t *>(ring) + (size_t)slot * slot_size;
 
-  RuleItem it[K];
-  uint32_t slots[K];
-#pragma unroll
-  for (int k = 0; k < K; k++) {
-    it[k].item = item0 + k;
-    it[k].live = it[k].item < n_items;
-    slots[k] = it[k].live ? sload(frag_slot + it[k].item) : 0u;
-  }
-#pragma unroll
-  for (int k = 0; k < K; k++) {
-    RuleItem &t = it[k];
-    t.r = t.item / per_req;
-    t.i = t.item - t.r * per_req;
-    t.off = t.i * mtu;
-    const uint64_t rem = size - t.off;
-    t.len = (uint32_t)(rem <= mtu ? rem : mtu);
-    t.plain = true;
-    t.to = nullptr;
-    t.ro = 0;
-    t.check_hdr = false;
-    t.hv = 0;
-    t.hc = (u32x4){0u, 0u, 0u, 0u};
-    t.sub_off = 0;
-    t.sub_len = 0;
-    if (t.live && slots[k] >= n_slots) {
-      if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
-      t.live = false;
-    }
-    if (!t.live) continue;
-    t.pkt = const_cast<uint8_t *>(ring) + (size_t)slots[k] * slot_size;
-    if (cap) {
-      // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
-      t.ro = c0 + (uint64_t)t.r * size;
-      t.ro = t.ro >= cap ? t.ro - cap : t.ro;  // the batch fits the arena (checked by the host): one wrap at most
-      if (lane == 0 && piece == 0) {
-        if (t.i == 0 && a.offsets_out) a.offsets_out[t.r] = t.ro;
-        if (t.item == n_items - 1) {
-          uint64_t end = t.ro + size;  // size <= capacity
-          end = end >= cap ? end - cap : end;
-          *a.cursor_out = end;
-          if (a.offsets_out) a.offsets_out[a.n_req] = end;
-        }
+  uint64_t ro = 0;
+  bool plain = !(opts & kOptMultiTensor);
+  uint8_t *to = nullptr;
+  if (cap) {
+    // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
+    if (c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
+    ro = c0 + (uint64_t)r * size;
+    ro = ro >= cap ? ro - cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
+    if (lane == 0 && piece == 0) {
+      if (i == 0 && a.offsets_out) a.offsets_out[r] = ro;
+      if (item == n_items - 1) {
+        uint64_t end = ro + size;  // size <= capacity
+        end = end >= cap ? end - cap : end;
+        *a.cursor_out = end;
+        if (a.offsets_out) a.offsets_out[a.n_req] = end;
       }
-      uint64_t o = t.ro + t.off;  // < 2 * capacity
-      if (!(opts & kOptMirrored)) {
-        if (o >= cap) o -= cap;
-        else if (o + t.len > cap) t.plain = false;  // crosses the end of an arena mapped once
-      }
-      t.to = dst + o;
-    } else if (opts & kOptMultiTensor) {
-      // tensor-major buffers: a fragment inside one tensor still takes the fast path
-      t.plain = plain_target(a.app, 0, t.r, t.off, t.len, &t.to);
-    } else {
-      t.to = dst + (uint64_t)t.r * size + t.off;
     }
-    // The header words that hold the fragment's real length are fetched together
-    // with the payload, so that checking them does not lengthen the wavefront's
-    // life by another memory round trip.
-    t.check_hdr = piece == 0 && a.frag_len == nullptr;
-    if (t.check_hdr) {
-      // every lane asks for the same bytes: one request, and on the cache line
-      // the payload's first chunk needs anyway
-      if (opts & kOptHdrChunk) t.hc = *reinterpret_cast<const u32x4 *>(t.pkt + 48);
-      else t.hv = load32_any(t.pkt + 54);
+    uint64_t o = ro + off;  // < 2 * capacity
+    if (!(opts & kOptMirrored)) {
+      if (o >= cap) o -= cap;
+      else if (o + len > cap) plain = false;  // crosses the end of an arena mapped once
     }
-    // copying the ruled length stays inside the slot whatever the header says
-    t.sub_len = t.len;
-    if (LONG && t.plain) sub_run(t.to, t.len, piece, &t.sub_off, &t.sub_len);
-    if (t.plain && t.sub_len) run_begin(t.rs, t.pkt + hl + t.sub_off, t.to + t.sub_off, t.sub_len, lane);
+    to = dst + o;
+  } else if (opts & kOptMultiTensor) {
+    // tensor-major buffers: a fragment inside one tensor still takes the fast path
+    plain = plain_target(a.app, 0, r, off, len, &to);
+  } else {
+    to = dst + (uint64_t)r * size + off;
   }
-#pragma unroll
-  for (int k = 0; k < K; k++) {
-    RuleItem &t = it[k];
-    asm volatile("" ::"v"(t.hc), "v"(t.hv));  // consumed only after the payload loads are under way
-    if (!t.live) continue;
-    if (t.plain) {
-      if (t.sub_len) run_end<false>(t.rs, lane);
-    } else if (piece == 0) {
-      move_run<true, false>(a.app, t.ro, t.r, t.off, t.pkt + hl, t.len, lane);
-    }
-    if (piece == 0) {
-      uint32_t bad = 0;
-      // payload_len is the u32 at byte 54: bytes 6..9 of the chunk that starts at byte 48
-      const uint32_t hdr_len = (opts & kOptHdrChunk) ? ((t.hc[1] >> 16) | (t.hc[2] << 16)) : t.hv;
-      const bool as_ruled = (t.check_hdr ? hdr_len : sload(a.frag_len + t.item)) == t.len;
-      if (!as_ruled) bad |= kStNotRule;
-      if (t.i == 0 && sload(a.first + t.r) != t.item) bad |= kStBadTable;
-      if (bad && lane == 0) refuse(a.status, a.status_flag, bad);
-    }
+  // The header words that hold the fragment's real length are fetched together
+  // with the payload, so that checking them does not lengthen the wavefront's
+  // life by another memory round trip.
+  const bool check_hdr = piece == 0 && a.frag_len == nullptr;
+  uint32_t hv = 0;
+  u32x4 hc = {0u, 0u, 0u, 0u};
+  if (check_hdr) {
+    // every lane asks for the same bytes: one request, and on the cache line
+    // the payload's first chunk needs anyway
+    if (opts & kOptHdrChunk) hc = *reinterpret_cast<const u32x4 *>(pkt + 48);
+    else hv = load32_any(pkt + 54);
+  }
+  // copying the ruled length stays inside the slot whatever the header says
+  RunState rs;
+  uint32_t sub_off = 0, sub_len = len;
+  if (LONG && plain) sub_run(to, len, piece, &sub_off, &sub_len);
+  if (plain && sub_len) run_begin(rs, pkt + hl + sub_off, to + sub_off, sub_len, lane);
+  asm volatile("" ::"v"(hc), "v"(hv));  // consumed only after the payload loads are under way
+  if (plain) {
+    if (sub_len) run_end<false>(rs, lane);
+  } else if (piece == 0) {
+    move_run<true, false>(a.app, ro, r, off, pkt + hl, len, lane);
+  }
+  if (piece == 0) {
+    uint32_t bad = 0;
+    // payload_len is the u32 at byte 54: bytes 6..9 of the chunk that starts at byte 48
+    const uint32_t hdr_len = (opts & kOptHdrChunk) ? ((hc[1] >> 16) | (hc[2] << 16)) : hv;
+    const bool as_ruled = (check_hdr ? hdr_len : sload(a.frag_len + item)) == len;
+    if (!as_ruled) bad |= kStNotRule;
+    if (i == 0 && sload(a.first + r) != item) bad |= kStBadTable;
+    if (bad && lane == 0) refuse(a.status, a.status_flag, bad);
   }
 }
 
@@ -1700,20 +1657,15 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.status_flag = c->h_flag;
     ga.app = app;
     ga.pieces = pieces_for(a->mtu);
-    uint32_t per_wave = 1;
-    if (ga.pieces == 1) {
-      per_wave = a->fixed_req_size / per < kPairBelow ? 2u : 1u;
-    }
     uint32_t grid, remap;
-    geometry(((uint64_t)a->n_frags * ga.pieces + per_wave - 1) / per_wave, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
+    geometry((uint64_t)a->n_frags * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
               (app.n_tensors > 1 ? kOptMultiTensor : 0u) |
               ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    if (ga.pieces > 1) k_gather_rule<true, 1><<<grid, kBlock, 0, c->stream>>>(ga);
-    else if (per_wave == 2) k_gather_rule<false, 2><<<grid, kBlock, 0, c->stream>>>(ga);
-    else k_gather_rule<false, 1><<<grid, kBlock, 0, c->stream>>>(ga);
+    if (ga.pieces > 1) k_gather_rule<true><<<grid, kBlock, 0, c->stream>>>(ga);
+    else k_gather_rule<false><<<grid, kBlock, 0, c->stream>>>(ga);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
     return finish(c, a->flags);
