@@ -48,6 +48,9 @@ def parse():
                     help="rotate over ring copies until the working set exceeds this many MB")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip requests/s of the other workloads")
+    ap.add_argument("--ref64", action="store_true",
+                    help="the reference's own 64-byte p2p_rpc_hdr (payload lengths from a table) instead of "
+                         "the 58-byte benchmark header")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-remap", action="store_true", help="disable the XCD-aware launch order")
     ap.add_argument("--calib-copy", action="store_true",
@@ -302,7 +305,8 @@ def main() -> int:
     torch.cuda.set_device(0)
     extra = capi.F_NO_XCD_REMAP if a.no_remap else 0
     bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
-    w = synth.make_workload(a.workload)
+    prof = synth.HDR_REF64 if a.ref64 else synth.HDR_BL58
+    w = synth.make_workload(a.workload, profile=prof)
     ctx = SgContext(0, max_reqs=max(4096, w.n_req * bpl), max_frames=max(65536, max(w.n_frags, w.n_resp_frames) * bpl))
     pool = Pool(w, bpl, a.rotate_mb, extra, rule=not a.general)
 
@@ -330,11 +334,18 @@ def main() -> int:
     ra_fs = torch.zeros(n_arr, dtype=torch.int32, device="cuda:0")
     ra_fl = torch.zeros(n_arr, dtype=torch.int32, device="cuda:0")
     ra_rf = torch.zeros(pool.n_req + 1, dtype=torch.int32, device="cuda:0")
+    ra_kw = {}
+    if a.ref64:
+        # the reference's header carries no lengths: they come per slot, as from the NIC, and a
+        # request is complete when its bytes add up to the server-wide request size
+        ln = torch.zeros(int(dw0.rx.n_slots), dtype=torch.int32, device="cuda:0")
+        ln[dw0.frag_slot.long()] = dw0.frag_len
+        ra_kw = {"len_nic": ln, "req_size": int(w.req_sizes[0])}
     for _ in range(3):
-        got = ctx.reassemble(dw0.rx, dw0.arrivals, n_arr, ra_fs, ra_fl, ra_rf)
+        got = ctx.reassemble(dw0.rx, dw0.arrivals, n_arr, ra_fs, ra_fl, ra_rf, **ra_kw)
     t0 = time.perf_counter()
     for _ in range(20):
-        got = ctx.reassemble(dw0.rx, dw0.arrivals, n_arr, ra_fs, ra_fl, ra_rf)
+        got = ctx.reassemble(dw0.rx, dw0.arrivals, n_arr, ra_fs, ra_fl, ra_rf, **ra_kw)
     ra_sec = (time.perf_counter() - t0) / 20
     reassembly = {"arrivals": n_arr, "requests": got[0], "ms_per_call": round(ra_sec * 1e3, 4),
                   "arrivals_per_sec": round(n_arr / ra_sec, 1),
@@ -378,6 +389,15 @@ def main() -> int:
             c2.close()
             torch.cuda.empty_cache()
 
+    if not a.no_sweep and not a.ref64:
+        # the headline workload again with the reference's own 64-byte header
+        wr = synth.make_workload(a.workload, profile=synth.HDR_REF64)
+        pr = Pool(wr, bpl, a.rotate_mb, extra, rule=not a.general)
+        sr = timed(ctx, pr, max(20, a.steps // 4), max(5, a.warmup // 4))
+        sweep[wr.name + "_ref64_headers"] = {"batches_per_launch": bpl, "ms_per_step": round(sr * 1e3, 5),
+                                             "GBps": round((pr.gather_bytes + pr.scatter_bytes) / sr / 1e9, 2)}
+        del pr
+
     out = {
         "metric": "gather+scatter GB/s (algorithmic bytes) on 1 MI355X",
         "value": round(value, 2),
@@ -395,7 +415,7 @@ def main() -> int:
                                f"{w.n_frags // w.n_req} frames of <= {w.mtu} B, {w.slot_size}-B slots, "
                                f"{w.n_resp_frames // w.n_req} response frames per request",
                    "batches_per_launch": bpl, "rotated_ring_copies": len(pool.items),
-                   "requests_per_step": pool.n_req, "header_profile": "BL58",
+                   "requests_per_step": pool.n_req, "header_profile": "REF64" if a.ref64 else "BL58",
                    "descriptor_pass": "general (prefix scan)" if a.general else
                    "fused where the workload has one size (fragmenting rule declared and checked)",
                    "flags": w.flags},
@@ -404,7 +424,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None if a.general else MEASURED_TRAFFIC.get((a.workload, bpl, dom)),
+                     "traffic": None if (a.general or a.ref64) else MEASURED_TRAFFIC.get((a.workload, bpl, dom)),
                      "traffic_unit": "HBM bytes per launch (rocprofv3 --pmc, see profiles/)",
                      "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3),
                      # the same call launched back to back, two events around the burst (all of the
