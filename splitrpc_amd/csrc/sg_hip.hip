@@ -595,6 +595,7 @@ struct GatherRuleArgs {
   uint64_t cap;               // packed: arena capacity; 0: tensor-major
   uint32_t n_items;
   uint32_t per_req;
+  uint32_t div_mul, div_shift;  // item / per_req == (item * div_mul) >> div_shift for item < 2^27
   uint32_t mtu;
   uint32_t slot_size;
   uint32_t hl;
@@ -626,9 +627,10 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint64_t size = a.size, cap = a.cap;
   const uint32_t n_items = a.n_items, per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
   const uint32_t hl = a.hl, n_slots = a.n_slots, pieces = a.pieces, opts = a.opts;
+  const uint32_t div_mul = a.div_mul, div_shift = a.div_shift;
   SG_PIN(ring); SG_PIN(frag_slot); SG_PIN(dst); SG_PIN(cursor_in); SG_PIN(size); SG_PIN(cap);
   SG_PIN(n_items); SG_PIN(per_req); SG_PIN(mtu); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_slots);
-  SG_PIN(pieces); SG_PIN(opts);
+  SG_PIN(pieces); SG_PIN(opts); SG_PIN(div_mul); SG_PIN(div_shift);
 
   const uint32_t w = item_of_wave((opts & kOptRemap) != 0);
   const uint32_t item = LONG ? w / pieces : w;
@@ -637,11 +639,13 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t slot = sload(frag_slot + item);
   uint64_t c0 = cap ? sload(cursor_in) : 0;
-  const uint32_t r = item / per_req;
+  // division by the fragments per request as a multiplication the host prepared (a division of
+  // two scalars is some twenty scalar instructions, and the scalar unit is the busiest here)
+  const uint32_t r = (uint32_t)(((uint64_t)item * div_mul) >> div_shift);
   const uint32_t i = item - r * per_req;
   const uint32_t off = i * mtu;
-  const uint64_t rem = size - off;
-  const uint32_t len = (uint32_t)(rem <= mtu ? rem : mtu);
+  const uint32_t rem = (uint32_t)size - off;  // sizes are below 4 GiB (checked by the host)
+  const uint32_t len = rem <= mtu ? rem : mtu;
   if (slot >= n_slots) {
     if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
     return;
@@ -1347,6 +1351,15 @@ int finish(sg_hip_ctx *c, uint32_t flags)
 
 }  // namespace
 
+// floor(n / d) == (n * M) >> (27 + l) for every n < 2^27, with l = ceil(log2 d), M = ceil(2^(27 + l) / d)
+static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
+{
+  uint32_t l = 0;
+  while ((1ull << l) < d) l++;
+  *shift = 27 + l;
+  *mul = (uint32_t)(((1ull << *shift) + d - 1) / d);
+}
+
 template <bool FUSED>
 static void launch_scatter(sg_hip_ctx *c, const ScatterArgs &sa, uint32_t grid, bool full_csum)
 {
@@ -1628,6 +1641,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     if ((uint64_t)a->mtu + hl0 > a->ring.slot_size) return fail(c, SG_E_INVAL, "mtu %u + %u header bytes does not fit a %u-byte slot", a->mtu, hl0, a->ring.slot_size);
     const uint64_t per = (a->fixed_req_size + a->mtu - 1) / a->mtu;
     if (per * a->n_req != a->n_frags) return fail(c, SG_E_INVAL, "%u requests of %llu bytes at mtu %u are %llu fragments, not %u", a->n_req, (unsigned long long)a->fixed_req_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frags);
+    if (a->n_frags >= (1u << 27)) return fail(c, SG_E_INVAL, "%u fragments in one call: the limit is 2^27 - 1", a->n_frags);
     if (a->fixed_req_size > 0xffffffffull || (app.n_tensors == 0 ? a->fixed_req_size > app.cap : a->fixed_req_size > max_req_bytes))
       return fail(c, SG_E_INVAL, "request size %llu does not fit its destination", (unsigned long long)a->fixed_req_size);
     // a batch larger than the arena would lap itself and its wavefronts would race for the same bytes
@@ -1645,6 +1659,7 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.cap = app.n_tensors == 0 ? app.cap : 0;
     ga.n_items = a->n_frags;
     ga.per_req = (uint32_t)per;
+    magic_div(per, &ga.div_mul, &ga.div_shift);
     ga.mtu = a->mtu;
     ga.slot_size = a->ring.slot_size;
     ga.hl = hl0;
