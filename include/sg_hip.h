@@ -259,11 +259,20 @@ int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_te
  * with request offsets taken from the bump ring.  Synchronous unless
  * SG_F_ASYNC is set; an SG_F_ASYNC call does nothing on the stream but launch
  * kernels (no allocation, no copy, no memset).  The bump-ring cursor of an
- * arena lives in two device words, each call reading the one the previous
- * call wrote; which is which is fixed when the call is issued, so a caller
- * that records calls into a HIP graph records an even number of calls per
- * arena (or uses an arena of exactly one batch, where the cursor always
- * returns to the same place) for replays to continue the ring. */
+ * arena is one device word that only kernels advance (a one-workgroup kernel
+ * behind the copy kernel, or the copy kernel itself where a descriptor pass has
+ * read the cursor before it), so calls recorded into a HIP graph -- any number
+ * of them -- continue the ring on every replay.
+ *
+ * The cursor after a refusal.  A call the host refuses (SG_E_INVAL) launches
+ * nothing and leaves the cursor alone.  With a descriptor pass (no
+ * SG_F_RULE_FRAGS; scatter with resp_size or SG_F_NO_FUSE) a batch the device
+ * refuses (SG_E_DATA) moves nothing and does not advance the cursor.  Without
+ * one (SG_F_RULE_FRAGS; scatter of one response size) the advance depends on
+ * n_req and the size alone: the cursor moves by the whole batch, and
+ * offsets_out is complete, even if a fragment was dropped for a bad slot index.
+ * The refusal bits stay up until the next sg_hip_sync(): asynchronous
+ * descriptor-pass calls queued behind a refused one move nothing either. */
 int sg_hip_gather_batch(sg_hip_ctx *ctx, const sg_gather_args *args);
 int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
 

@@ -84,9 +84,16 @@ struct PrepArgs {
   u32x4 *desc;             // {slot, len, offset in request, request}
   uint64_t *req_size;
   uint64_t *req_off;
-  const uint64_t *cursor_in;
-  uint64_t *cursor_out;
+  // The bump-ring cursor is one device word.  The descriptor pass only reads
+  // it and leaves the advanced value in *next_cursor; the copy kernel of the
+  // same call, which does not read the cursor, commits it.
+  const uint64_t *cursor;
+  uint64_t *next_cursor;
   uint64_t *offsets_out;
+  // mode 1: where each frame's header comes from, held against the RX ring here
+  // so that a bad index refuses the batch before anything is written
+  const uint32_t *hdr_src_slot;
+  uint32_t rx_n_slots;
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
@@ -144,6 +151,7 @@ __device__ __forceinline__ void prep_item(const PrepArgs &a, uint32_t f, uint32_
     const uint64_t taken = (uint64_t)i * a.mtu;
     const uint64_t rem = taken < size ? size - taken : 0;
     l = (uint32_t)(rem <= a.mtu ? rem : a.mtu);
+    if (a.hdr_src_slot && a.hdr_src_slot[f] >= a.rx_n_slots) *bad |= kStBadSlot;
   }
   *slot = s;
   *len = l;
@@ -188,13 +196,13 @@ __device__ __forceinline__ void prep_finish(const PrepArgs &a, uint32_t r, uint6
   a.req_size[r] = total;
   if (a.packed && a.fixed_offsets) {
     // bump ring with equal sizes: ret = base + off; off = (off + size) % capacity
-    const uint64_t c0 = *a.cursor_in % a.cap;
+    const uint64_t c0 = *a.cursor % a.cap;
     const uint64_t off = (c0 + (uint64_t)r * (a.fixed_size % a.cap)) % a.cap;
     a.req_off[r] = off;
     if (a.offsets_out) a.offsets_out[r] = off;
     if (r == a.n_req - 1) {
       const uint64_t end = (off + a.fixed_size) % a.cap;
-      *a.cursor_out = end;
+      *a.next_cursor = end;
       if (a.offsets_out) a.offsets_out[a.n_req] = end;
     }
   }
@@ -304,7 +312,7 @@ __device__ __forceinline__ void scan_check_batch(const PrepArgs &a, uint64_t bat
 __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
-  uint64_t run = *a.cursor_in % a.cap, batch_bytes = 0;
+  uint64_t run = *a.cursor % a.cap, batch_bytes = 0;
   for (uint32_t base = 0; base < a.n_req; base += kScanTile) {
     const uint32_t q0 = base + threadIdx.x * kScanPerThread;
     uint64_t sz[kScanPerThread], tot;
@@ -314,7 +322,7 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
     batch_bytes += tot;
   }
   if (threadIdx.x == 0) {
-    *a.cursor_out = run;
+    *a.next_cursor = run;
     if (a.offsets_out) a.offsets_out[a.n_req] = run;
     scan_check_batch(a, batch_bytes);
   }
@@ -347,7 +355,7 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan_add(PrepArgs a, const u
     batch_bytes += tot;
   }
   before = is_last ? batch_bytes - tile_tot[blockIdx.x] : batch_bytes;
-  const uint64_t c0 = *a.cursor_in % a.cap;
+  const uint64_t c0 = *a.cursor % a.cap;
   const uint64_t tile_base = (c0 + before % a.cap) % a.cap;
   const uint32_t q0 = blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
   uint64_t sz[kScanPerThread], tot;
@@ -355,7 +363,7 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan_add(PrepArgs a, const u
   scan_emit(a, q0, sz, (tile_base + ex % a.cap) % a.cap);
   if (is_last && threadIdx.x == 0) {
     const uint64_t end = (c0 + batch_bytes % a.cap) % a.cap;
-    *a.cursor_out = end;
+    *a.next_cursor = end;
     if (a.offsets_out) a.offsets_out[a.n_req] = end;
     scan_check_batch(a, batch_bytes);
   }
@@ -381,6 +389,33 @@ __device__ __forceinline__ uint32_t item_of_wave(bool remap)
   return __builtin_amdgcn_readfirstlane(g * kWavesPerBlock + threadIdx.x / kWave);
 }
 
+// Advancing the cursor.  A copy kernel that derives its offsets from the
+// bump-ring cursor cannot advance that cursor itself: its own wavefronts may
+// still read it, and a second word to write into would need a device word
+// saying which of the two is live -- with the same problem.  (Letting the
+// wavefronts count themselves in or out with atomics so that the last one may
+// write was built and measured: one returning atomic per workgroup costs the
+// 32-batch gather 4 to 11 % -- the wavefront that waits for its ticket holds its
+// registers that much longer.)  So the advance is the business of a one-workgroup
+// kernel launched right behind the copy kernel, which also publishes slot
+// states where the caller keeps them.  A recorded graph may therefore hold any
+// number of calls.
+struct FinishArgs {
+  uint64_t *cursor;      // advanced by n_req * size modulo cap; nullptr: nothing to advance
+  uint64_t size;
+  uint64_t cap;
+  uint32_t n_req;
+};
+
+__global__ __launch_bounds__(kBlock) void k_finish(FinishArgs a)
+{
+  if (a.cursor && threadIdx.x == 0) {
+    // bump ring with equal sizes: off = (off + size) % capacity, n_req times
+    const uint64_t c = *a.cursor;
+    *a.cursor = (c % a.cap + ((uint64_t)a.n_req * a.size) % a.cap) % a.cap;
+  }
+}
+
 // What the fused kernels need to derive a descriptor themselves when all
 // requests (responses) have one size and are cut by the fragmenting rule:
 // item f belongs to request f / per_req, is its fragment f % per_req, carries
@@ -395,8 +430,7 @@ struct RuleArgs {
   uint32_t n_req;
   uint32_t n_slots;
   uint32_t single_wrap;  // n_req * size <= capacity: a request offset wraps at most once
-  const uint64_t *cursor_in;
-  uint64_t *cursor_out;
+  const uint64_t *cursor;  // read only here; k_finish advances it behind this kernel
   uint64_t *offsets_out;
 };
 
@@ -411,6 +445,8 @@ struct GatherArgs {
   uint32_t pieces;  // wavefronts per fragment
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
+  uint64_t *cursor;             // packed: wavefront 0 commits *next_cursor unless the batch was refused
+  const uint64_t *next_cursor;
   AppDev app;
 };
 
@@ -427,7 +463,7 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
   // the three table reads are independent: asked for together
   *slot = sload_here(g.item_slot + item);
   const uint32_t first_r = sload_here(g.first + *r);
-  uint64_t c0 = app.n_tensors == 0 ? sload_here(g.cursor_in) : 0;
+  uint64_t c0 = app.n_tensors == 0 ? sload_here(g.cursor) : 0;
   *off = *i * g.mtu;
   const uint64_t rem = g.size - *off;
   *len = (uint32_t)(rem <= g.mtu ? rem : g.mtu);
@@ -442,11 +478,10 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
     *req_off = o;
     if (lane == 0) {
       if (*i == 0 && g.offsets_out) g.offsets_out[*r] = *req_off;
-      if (item == n_items - 1) {
+      if (item == n_items - 1 && g.offsets_out) {
         uint64_t end = *req_off + g.size;  // size <= capacity
         end = end >= app.cap ? end - app.cap : end;
-        *g.cursor_out = end;
-        if (g.offsets_out) g.offsets_out[g.n_req] = end;
+        g.offsets_out[g.n_req] = end;
       }
     }
   }
@@ -558,8 +593,10 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   const uint32_t w = item_of_wave(remap != 0);
   const uint32_t item = LONG ? w / pieces : w;
   const uint32_t piece = LONG ? w - item * pieces : 0;
-  if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
+  // this kernel does not read the cursor: the value the descriptor pass left is committed here
+  if (w == 0 && lane == 0 && a.cursor && !sload(status)) *a.cursor = sload(a.next_cursor);
+  if (item >= n_items) return;
   const u32x4 d = sload_here(desc + item);  // asked for together with the status word
   if (sload_here(status)) return;           // the descriptor pass refused the batch: move nothing
   if (d[1] == 0 || d[3] == kInvalidReq) return;
@@ -590,7 +627,7 @@ struct GatherRuleArgs {
   const uint8_t *ring;
   const uint32_t *frag_slot;
   uint8_t *dst;               // arena (packed) or the tensor (one tensor-major buffer)
-  const uint64_t *cursor_in;  // packed only
+  const uint64_t *cursor;     // packed only; read only here, k_finish advances it behind this kernel
   uint64_t size;
   uint64_t cap;               // packed: arena capacity; 0: tensor-major
   uint32_t n_items;
@@ -607,7 +644,6 @@ struct GatherRuleArgs {
   const uint32_t *frag_len;
   const uint32_t *first;
   uint64_t *offsets_out;
-  uint64_t *cursor_out;
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   AppDev app;  // consulted for several tensor-major buffers only
@@ -623,7 +659,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint8_t *ring = a.ring;
   const uint32_t *frag_slot = a.frag_slot;
   uint8_t *dst = a.dst;
-  const uint64_t *cursor_in = a.cursor_in;
+  const uint64_t *cursor_in = a.cursor;
   const uint64_t size = a.size, cap = a.cap;
   const uint32_t n_items = a.n_items, per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
   const uint32_t hl = a.hl, n_slots = a.n_slots, pieces = a.pieces, opts = a.opts;
@@ -646,10 +682,6 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint32_t off = i * mtu;
   const uint32_t rem = (uint32_t)size - off;  // sizes are below 4 GiB (checked by the host)
   const uint32_t len = rem <= mtu ? rem : mtu;
-  if (slot >= n_slots) {
-    if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
-    return;
-  }
   uint8_t *pkt = const_cast<uint8_t *>(ring) + (size_t)slot * slot_size;
 
   uint64_t ro = 0;
@@ -660,13 +692,11 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     if (c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
     ro = c0 + (uint64_t)r * size;
     ro = ro >= cap ? ro - cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
-    if (lane == 0 && piece == 0) {
-      if (i == 0 && a.offsets_out) a.offsets_out[r] = ro;
+    if (lane == 0 && piece == 0 && a.offsets_out) {
+      if (i == 0) a.offsets_out[r] = ro;
       if (item == n_items - 1) {
         uint64_t end = ro + size;  // size <= capacity
-        end = end >= cap ? end - cap : end;
-        *a.cursor_out = end;
-        if (a.offsets_out) a.offsets_out[a.n_req] = end;
+        a.offsets_out[a.n_req] = end >= cap ? end - cap : end;
       }
     }
     uint64_t o = ro + off;  // < 2 * capacity
@@ -680,6 +710,12 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     plain = plain_target(a.app, 0, r, off, len, &to);
   } else {
     to = dst + (uint64_t)r * size + off;
+  }
+  // offsets depend on the item, the size and the cursor only: they are out before a
+  // fragment with a bad slot index is dropped
+  if (slot >= n_slots) {
+    if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
+    return;
   }
   // The header words that hold the fragment's real length are fetched together
   // with the payload, so that checking them does not lengthen the wavefront's
@@ -735,6 +771,8 @@ struct ScatterArgs {
   uint32_t pieces;  // wavefronts per frame
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
+  uint64_t *cursor;             // descriptor path, packed: wavefront 0 commits *next_cursor
+  const uint64_t *next_cursor;
   RuleArgs rule;
   AppDev app;
 };
@@ -766,14 +804,16 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   SG_PIN(a.app.n_tensors); SG_PIN(a.app.arena); SG_PIN(a.app.cap); SG_PIN(a.app.mirrored);
   if (FUSED) {
     SG_PIN(a.rule.item_slot); SG_PIN(a.rule.first); SG_PIN(a.rule.size); SG_PIN(a.rule.mtu);
-    SG_PIN(a.rule.per_req); SG_PIN(a.rule.n_slots); SG_PIN(a.rule.single_wrap); SG_PIN(a.rule.cursor_in);
+    SG_PIN(a.rule.per_req); SG_PIN(a.rule.n_slots); SG_PIN(a.rule.single_wrap); SG_PIN(a.rule.cursor);
   }
   const uint32_t w = item_of_wave(remap != 0);
   const uint32_t pieces = SPLIT ? n_pieces : 1u;
   const uint32_t item = SPLIT ? w / pieces : w;
   const uint32_t piece = SPLIT ? w - item * pieces : 0;
-  if (item >= n_items) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
+  // descriptor path: this kernel does not read the cursor and commits what the descriptor pass left
+  if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status)) *a.cursor = sload(a.next_cursor);
+  if (item >= n_items) return;
   const bool from_template = hdr_templates != nullptr;
   // independent table reads, asked for together
   const uint32_t hs = from_template ? 0u : sload_here(hdr_src_slot + item);
@@ -814,7 +854,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     }
   } else {
     if (hs >= rx_n_slots) {
-      if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
+      // descriptor path: the descriptor pass has refused the batch already and nothing gets here
+      if (FUSED && lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
       return;
     }
     hin = rx + (size_t)hs * rx_slot_size;
@@ -1154,6 +1195,23 @@ struct EvPair {
   int which;
 };
 
+// Device memory a batched call works in, beyond its inputs and outputs.  A
+// context owns one set (allocated at creation); the allocation-free entry
+// point uses a set carved out of a static device array.
+struct Scratch {
+  uint32_t max_reqs = 0, max_frames = 0;
+  u32x4 *desc = nullptr;         // run descriptors, max_frames
+  uint64_t *req_size = nullptr;  // max_reqs
+  uint64_t *req_off = nullptr;   // max_reqs
+  uint64_t *tile_tot = nullptr;  // one total per kScanTile requests, for the tiled request scan
+  // bump-ring cursors (request arena, response arena) and the values a
+  // descriptor pass stages for the copy kernel to commit
+  uint64_t *cursor[2] = {nullptr, nullptr};
+  uint64_t *next_cursor[2] = {nullptr, nullptr};
+  uint32_t *status = nullptr;
+  volatile uint32_t *flag = nullptr;  // raised with every refusal (pinned host memory in a context)
+};
+
 struct sg_hip_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
@@ -1164,11 +1222,10 @@ struct sg_hip_ctx {
   uint64_t *req_size = nullptr;
   uint64_t *req_off = nullptr;
   uint64_t *tile_tot = nullptr;  // one total per 4096 requests, for the tiled request scan
-  // bump-ring cursors: request arena at [0 + parity], response arena at
-  // [2 + parity]; a launch reads one parity and writes the other
+  // [0] request-arena cursor, [1] response-arena cursor, [2], [3] their staged successors
   uint64_t *cursors = nullptr;
-  uint32_t parity[2] = {0, 0};
   uint32_t *status = nullptr;
+  Scratch sc;
   // pinned staging for the per-request entry points (device reads it in place)
   Run *h_runs = nullptr;
   uint32_t h_runs_cap = 0;
@@ -1276,7 +1333,7 @@ void geometry(uint64_t n_waves, bool want_remap, uint32_t *grid, uint32_t *remap
 
 int prof_begin(sg_hip_ctx *c, int which)
 {
-  if (!c->profiling) return SG_OK;
+  if (!c || !c->profiling) return SG_OK;
   EvPair p;
   if (!c->ev_free.empty()) {
     p = c->ev_free.back();
@@ -1293,7 +1350,7 @@ int prof_begin(sg_hip_ctx *c, int which)
 
 int prof_end(sg_hip_ctx *c)
 {
-  if (!c->profiling) return SG_OK;
+  if (!c || !c->profiling) return SG_OK;
   HIP_TRY(c, hipEventRecord(c->ev_used.back().b, c->stream));
   return SG_OK;
 }
@@ -1313,34 +1370,46 @@ int prof_drain(sg_hip_ctx *c)
 
 // Descriptor build: kernel shape by the average request, then the bump-ring
 // scan of the request totals where offsets are not plain multiples.
-int launch_prep(sg_hip_ctx *c, const PrepArgs &p)
+int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs &p)
 {
   int rc = prof_begin(c, 0);
   if (rc != SG_OK) return rc;
   const uint32_t avg = p.n_items / p.n_req;
   if (avg <= 32) {
-    k_prep_wave<<<(p.n_req + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(p);
+    k_prep_wave<<<(p.n_req + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, st>>>(p);
   } else if (avg <= 256) {
-    k_prep_block<256><<<p.n_req, 256, 0, c->stream>>>(p);
+    k_prep_block<256><<<p.n_req, 256, 0, st>>>(p);
   } else {
-    k_prep_block<1024><<<p.n_req, 1024, 0, c->stream>>>(p);
+    k_prep_block<1024><<<p.n_req, 1024, 0, st>>>(p);
   }
   if (p.packed && !p.fixed_offsets) {
     if (p.n_req <= 2 * kScanTile) {
-      k_req_scan<<<1, kScanBlock, 0, c->stream>>>(p);
+      k_req_scan<<<1, kScanBlock, 0, st>>>(p);
     } else {
       const uint32_t n_tiles = (p.n_req + kScanTile - 1) / kScanTile;
-      uint64_t *tile_tot = c->tile_tot;
-      k_req_scan_local<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot);
-      k_req_scan_add<<<n_tiles, kScanBlock, 0, c->stream>>>(p, tile_tot, n_tiles);
+      k_req_scan_local<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot);
+      k_req_scan_add<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot, n_tiles);
     }
   }
   return prof_end(c);
 }
 
+// Behind the copy kernel of a single-kernel call on a packed arena.
+void launch_finish(hipStream_t st, uint64_t *cursor, uint64_t size, uint64_t cap, uint32_t n_req)
+{
+  FinishArgs f;
+  memset(&f, 0, sizeof f);
+  f.cursor = cursor;
+  f.size = size;
+  f.cap = cap;
+  f.n_req = n_req;
+  k_finish<<<1, kBlock, 0, st>>>(f);
+}
+
 int finish(sg_hip_ctx *c, uint32_t flags)
 {
   HIP_TRY(c, hipGetLastError());
+  if (!c) return SG_OK;  // allocation-free entry point: launches only
   if (flags & SG_F_ASYNC) {
     // keep the event list bounded on long asynchronous runs
     if (c->profiling && c->ev_used.size() > 4096) return sg_hip_sync(c);
@@ -1361,13 +1430,13 @@ static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
 }
 
 template <bool FUSED>
-static void launch_scatter(sg_hip_ctx *c, const ScatterArgs &sa, uint32_t grid, bool full_csum)
+static void launch_scatter(hipStream_t st, const ScatterArgs &sa, uint32_t grid, bool full_csum)
 {
   const bool lng = sa.pieces > 1;
-  if (full_csum && lng) k_scatter<true, FUSED, true><<<grid, kBlock, 0, c->stream>>>(sa);
-  else if (full_csum) k_scatter<true, FUSED, false><<<grid, kBlock, 0, c->stream>>>(sa);
-  else if (lng) k_scatter<false, FUSED, true><<<grid, kBlock, 0, c->stream>>>(sa);
-  else k_scatter<false, FUSED, false><<<grid, kBlock, 0, c->stream>>>(sa);
+  if (full_csum && lng) k_scatter<true, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
+  else if (full_csum) k_scatter<true, FUSED, false><<<grid, kBlock, 0, st>>>(sa);
+  else if (lng) k_scatter<false, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
+  else k_scatter<false, FUSED, false><<<grid, kBlock, 0, st>>>(sa);
 }
 
 extern "C" {
@@ -1414,6 +1483,19 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   c->h_status[0] = c->h_status[1] = 0;
   c->h_flag = c->h_status + 1;
   HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
+  Scratch &sc = c->sc;
+  sc.max_reqs = c->max_reqs;
+  sc.max_frames = c->max_frames;
+  sc.desc = c->desc;
+  sc.req_size = c->req_size;
+  sc.req_off = c->req_off;
+  sc.tile_tot = c->tile_tot;
+  sc.cursor[0] = c->cursors + 0;
+  sc.cursor[1] = c->cursors + 1;
+  sc.next_cursor[0] = c->cursors + 2;
+  sc.next_cursor[1] = c->cursors + 3;
+  sc.status = c->status;
+  sc.flag = c->h_flag;
   return SG_OK;
 }
 
@@ -1488,7 +1570,7 @@ int sg_hip_set_cursor(sg_hip_ctx *c, int which, uint64_t value)
   if (!c || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
-  HIP_TRY(c, hipMemcpy(c->cursors + 2 * which + c->parity[which], &value, sizeof value, hipMemcpyHostToDevice));
+  HIP_TRY(c, hipMemcpy(c->cursors + which, &value, sizeof value, hipMemcpyHostToDevice));
   return SG_OK;
 }
 
@@ -1497,7 +1579,7 @@ int sg_hip_get_cursor(sg_hip_ctx *c, int which, uint64_t *value)
   if (!c || !value || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
-  HIP_TRY(c, hipMemcpy(value, c->cursors + 2 * which + c->parity[which], sizeof *value, hipMemcpyDeviceToHost));
+  HIP_TRY(c, hipMemcpy(value, c->cursors + which, sizeof *value, hipMemcpyDeviceToHost));
   return SG_OK;
 }
 
@@ -1617,14 +1699,15 @@ int sg_hip_set_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, const uint8_t *hdr_temp
 
 // ---- batched ------------------------------------------------------------------
 
-int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
+// The gather call proper.  `c` may be null (allocation-free entry point): then
+// errors go to the creation-error text, nothing is profiled and nothing waits.
+static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const sg_gather_args *a)
 {
-  if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
   int rc = check_ring(c, a->ring, "rx");
   if (rc != SG_OK) return rc;
   if (a->n_req == 0) return SG_OK;
-  if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
-  if (a->n_frags > c->max_frames) return fail(c, SG_E_INVAL, "n_frags %u > max_frames %u of this context", a->n_frags, c->max_frames);
+  if (a->n_req > sc.max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u", a->n_req, sc.max_reqs);
+  if (a->n_frags > sc.max_frames) return fail(c, SG_E_INVAL, "n_frags %u > max_frames %u", a->n_frags, sc.max_frames);
   if ((!a->frag_slot && a->n_frags) || !a->req_first) return fail(c, SG_E_INVAL, "null fragment tables");
   if (!a->frag_len && a->n_frags && a->ring.hdr_profile != SG_HDR_BL58)
     return fail(c, SG_E_INVAL, "REF64 headers carry no payload length: frag_len is required");
@@ -1632,7 +1715,11 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   uint64_t max_req_bytes;
   rc = check_app(c, a->app, &app, &max_req_bytes);
   if (rc != SG_OK) return rc;
-  DeviceGuard g(c->device);
+  const bool packed = app.n_tensors == 0;
+  // a batch larger than the arena would lap itself and its wavefronts would race for the same bytes
+  if (packed && a->fixed_req_size && (uint64_t)a->n_req * a->fixed_req_size > app.cap)
+    return fail(c, SG_E_INVAL, "%u requests of %llu bytes do not fit an arena of %llu bytes", a->n_req,
+                (unsigned long long)a->fixed_req_size, (unsigned long long)app.cap);
 
   const uint32_t hl0 = hdr_len_of(a->ring.hdr_profile);
   if (a->flags & SG_F_RULE_FRAGS) {
@@ -1642,21 +1729,16 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     const uint64_t per = (a->fixed_req_size + a->mtu - 1) / a->mtu;
     if (per * a->n_req != a->n_frags) return fail(c, SG_E_INVAL, "%u requests of %llu bytes at mtu %u are %llu fragments, not %u", a->n_req, (unsigned long long)a->fixed_req_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frags);
     if (a->n_frags >= (1u << 27)) return fail(c, SG_E_INVAL, "%u fragments in one call: the limit is 2^27 - 1", a->n_frags);
-    if (a->fixed_req_size > 0xffffffffull || (app.n_tensors == 0 ? a->fixed_req_size > app.cap : a->fixed_req_size > max_req_bytes))
+    if (a->fixed_req_size > 0xffffffffull || (packed ? a->fixed_req_size > app.cap : a->fixed_req_size > max_req_bytes))
       return fail(c, SG_E_INVAL, "request size %llu does not fit its destination", (unsigned long long)a->fixed_req_size);
-    // a batch larger than the arena would lap itself and its wavefronts would race for the same bytes
-    if (app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_req_size > app.cap)
-      return fail(c, SG_E_INVAL, "%u requests of %llu bytes do not fit an arena of %llu bytes", a->n_req, (unsigned long long)a->fixed_req_size, (unsigned long long)app.cap);
     GatherRuleArgs ga;
     memset(&ga, 0, sizeof ga);
     ga.ring = static_cast<const uint8_t *>(a->ring.base);
     ga.frag_slot = a->frag_slot;
-    ga.dst = app.n_tensors == 0 ? app.arena : app.tensor_base[0];
-    ga.cursor_in = c->cursors + 0 + c->parity[0];
-    ga.cursor_out = c->cursors + 0 + (c->parity[0] ^ 1u);
-    if (app.n_tensors == 0) c->parity[0] ^= 1u;
+    ga.dst = packed ? app.arena : app.tensor_base[0];
+    ga.cursor = sc.cursor[0];
     ga.size = a->fixed_req_size;
-    ga.cap = app.n_tensors == 0 ? app.cap : 0;
+    ga.cap = packed ? app.cap : 0;
     ga.n_items = a->n_frags;
     ga.per_req = (uint32_t)per;
     magic_div(per, &ga.div_mul, &ga.div_shift);
@@ -1667,9 +1749,9 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
     ga.n_req = a->n_req;
     ga.frag_len = a->frag_len;
     ga.first = a->req_first;
-    ga.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
-    ga.status = c->status;
-    ga.status_flag = c->h_flag;
+    ga.offsets_out = packed ? a->offsets_out : nullptr;
+    ga.status = sc.status;
+    ga.status_flag = sc.flag;
     ga.app = app;
     ga.pieces = pieces_for(a->mtu);
     uint32_t grid, remap;
@@ -1679,10 +1761,11 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
               ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    if (ga.pieces > 1) k_gather_rule<true><<<grid, kBlock, 0, c->stream>>>(ga);
-    else k_gather_rule<false><<<grid, kBlock, 0, c->stream>>>(ga);
+    if (ga.pieces > 1) k_gather_rule<true><<<grid, kBlock, 0, st>>>(ga);
+    else k_gather_rule<false><<<grid, kBlock, 0, st>>>(ga);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
+    if (packed) launch_finish(st, sc.cursor[0], a->fixed_req_size, app.cap, a->n_req);
     return finish(c, a->flags);
   }
 
@@ -1698,59 +1781,69 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   p.item_len = a->frag_len;
   p.first = a->req_first;
   p.n_items = a->n_frags;
-  p.packed = app.n_tensors == 0;
+  p.packed = packed;
   p.cap = app.cap;
   p.max_req_bytes = max_req_bytes;
-  p.desc = c->desc;
-  p.req_size = c->req_size;
-  p.req_off = c->req_off;
+  p.desc = sc.desc;
+  p.req_size = sc.req_size;
+  p.req_off = sc.req_off;
   p.fixed_size = a->fixed_req_size;
   p.fixed_offsets = p.packed && a->fixed_req_size != 0;
-  p.cursor_in = c->cursors + 0 + c->parity[0];
-  p.cursor_out = c->cursors + 0 + (c->parity[0] ^ 1u);
-  if (p.packed) c->parity[0] ^= 1u;
-  p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
-  p.status = c->status;
-  p.status_flag = c->h_flag;
-  rc = launch_prep(c, p);
+  p.cursor = sc.cursor[0];
+  p.next_cursor = sc.next_cursor[0];
+  p.offsets_out = packed ? a->offsets_out : nullptr;
+  p.status = sc.status;
+  p.status_flag = sc.flag;
+  rc = launch_prep(c, sc, st, p);
   if (rc != SG_OK) return rc;
 
-  if (a->n_frags) {
+  // the copy kernel also commits the advanced cursor, so a batch of empty requests still launches it
+  if (a->n_frags || packed) {
     GatherArgs ga;
     memset(&ga, 0, sizeof ga);
-    ga.desc = c->desc;
-    ga.req_off = c->req_off;
+    ga.desc = sc.desc;
+    ga.req_off = sc.req_off;
     ga.ring = p.ring;
     ga.slot_size = p.slot_size;
     ga.hl = p.hl;
     ga.n_items = a->n_frags;
-    ga.status = c->status;
-    ga.status_flag = c->h_flag;
+    ga.status = sc.status;
+    ga.status_flag = sc.flag;
+    if (packed) {
+      ga.cursor = sc.cursor[0];
+      ga.next_cursor = sc.next_cursor[0];
+    }
     ga.app = app;
     ga.pieces = pieces_for(p.slot_size - p.hl);
     uint32_t grid;
-    geometry((uint64_t)a->n_frags * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
+    geometry((uint64_t)(a->n_frags ? a->n_frags : 1u) * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &ga.remap);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    if (ga.pieces > 1) k_gather<true><<<grid, kBlock, 0, c->stream>>>(ga);
-    else k_gather<false><<<grid, kBlock, 0, c->stream>>>(ga);
+    if (ga.pieces > 1) k_gather<true><<<grid, kBlock, 0, st>>>(ga);
+    else k_gather<false><<<grid, kBlock, 0, st>>>(ga);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }
   return finish(c, a->flags);
 }
 
-int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
+int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
 {
   if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
+  DeviceGuard g(c->device);
+  return gather_impl(c, c->sc, c->stream, a);
+}
+
+static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const sg_scatter_args *a)
+{
   int rc = check_ring(c, a->rx, "rx");
   if (rc != SG_OK) return rc;
   rc = check_ring(c, a->tx, "tx");
   if (rc != SG_OK) return rc;
   if (a->rx.hdr_profile != a->tx.hdr_profile) return fail(c, SG_E_INVAL, "rx and tx rings differ in header profile");
   if (a->n_req == 0) return SG_OK;
-  if (a->n_req > c->max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u of this context", a->n_req, c->max_reqs);
-  if (a->n_frames > c->max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u of this context", a->n_frames, c->max_frames);
+  if (a->n_req > sc.max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u", a->n_req, sc.max_reqs);
+  if (a->n_frames > sc.max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u", a->n_frames, sc.max_frames);
   if (!a->resp_first || (a->n_frames && (!a->tx_slot || (!a->hdr_src_slot && !a->hdr_templates))))
     return fail(c, SG_E_INVAL, "null frame tables");
   const uint32_t hl = hdr_len_of(a->tx.hdr_profile);
@@ -1761,7 +1854,7 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   uint64_t max_req_bytes;
   rc = check_app(c, a->app, &app, &max_req_bytes);
   if (rc != SG_OK) return rc;
-  DeviceGuard g(c->device);
+  const bool packed = app.n_tensors == 0;
 
   const bool fused = a->resp_size == nullptr && !(a->flags & SG_F_NO_FUSE);
   if (fused) {
@@ -1785,8 +1878,8 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.ref64 = a->tx.hdr_profile == SG_HDR_REF64;
     sa.flags = a->flags & 0xfu;
     sa.n_items = a->n_frames;
-    sa.status = c->status;
-    sa.status_flag = c->h_flag;
+    sa.status = sc.status;
+    sa.status_flag = sc.flag;
     sa.app = app;
     sa.rule.item_slot = a->tx_slot;
     sa.rule.first = a->resp_first;
@@ -1796,19 +1889,18 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.rule.n_req = a->n_req;
     sa.rule.n_slots = a->tx.n_slots;
     sa.rule.single_wrap = app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_resp_size <= app.cap;
-    sa.rule.cursor_in = c->cursors + 2 + c->parity[1];
-    sa.rule.cursor_out = c->cursors + 2 + (c->parity[1] ^ 1u);
-    if (app.n_tensors == 0) c->parity[1] ^= 1u;
-    sa.rule.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
+    sa.rule.cursor = sc.cursor[1];
+    sa.rule.offsets_out = packed ? a->offsets_out : nullptr;
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
     geometry((uint64_t)a->n_frames * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
              !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    launch_scatter<true>(c, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
+    launch_scatter<true>(st, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
+    if (packed) launch_finish(st, sc.cursor[1], a->fixed_resp_size, app.cap, a->n_req);
     return finish(c, a->flags);
   }
 
@@ -1828,24 +1920,27 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   p.packed = app.n_tensors == 0;
   p.cap = app.cap;
   p.max_req_bytes = max_req_bytes;
-  p.desc = c->desc;
-  p.req_size = c->req_size;
-  p.req_off = c->req_off;
+  p.desc = sc.desc;
+  p.req_size = sc.req_size;
+  p.req_off = sc.req_off;
   p.fixed_offsets = p.packed && a->resp_size == nullptr;
-  p.cursor_in = c->cursors + 2 + c->parity[1];
-  p.cursor_out = c->cursors + 2 + (c->parity[1] ^ 1u);
-  if (p.packed) c->parity[1] ^= 1u;
-  p.offsets_out = app.n_tensors == 0 ? a->offsets_out : nullptr;
-  p.status = c->status;
-  p.status_flag = c->h_flag;
-  rc = launch_prep(c, p);
+  p.cursor = sc.cursor[1];
+  p.next_cursor = sc.next_cursor[1];
+  p.offsets_out = packed ? a->offsets_out : nullptr;
+  if (!a->hdr_templates) {
+    p.hdr_src_slot = a->hdr_src_slot;
+    p.rx_n_slots = a->rx.n_slots;
+  }
+  p.status = sc.status;
+  p.status_flag = sc.flag;
+  rc = launch_prep(c, sc, st, p);
   if (rc != SG_OK) return rc;
 
-  if (a->n_frames) {
+  if (a->n_frames || packed) {
     ScatterArgs sa;
     memset(&sa, 0, sizeof sa);
-    sa.desc = c->desc;
-    sa.req_off = c->req_off;
+    sa.desc = sc.desc;
+    sa.req_off = sc.req_off;
     sa.first = a->resp_first;
     sa.hdr_src_slot = a->hdr_src_slot;
     sa.hdr_templates = a->hdr_templates;
@@ -1859,20 +1954,31 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
     sa.ref64 = a->tx.hdr_profile == SG_HDR_REF64;
     sa.flags = a->flags & 0xfu;
     sa.n_items = a->n_frames;
-    sa.status = c->status;
-    sa.status_flag = c->h_flag;
+    sa.status = sc.status;
+    sa.status_flag = sc.flag;
+    if (packed) {
+      sa.cursor = sc.cursor[1];
+      sa.next_cursor = sc.next_cursor[1];
+    }
     sa.app = app;
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
-    geometry((uint64_t)a->n_frames * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
+    geometry((uint64_t)(a->n_frames ? a->n_frames : 1u) * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
              !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    launch_scatter<false>(c, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
+    launch_scatter<false>(st, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }
   return finish(c, a->flags);
+}
+
+int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
+{
+  if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
+  DeviceGuard g(c->device);
+  return scatter_impl(c, c->sc, c->stream, a);
 }
 
 // ---- reassembly ----------------------------------------------------------------

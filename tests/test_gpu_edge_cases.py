@@ -311,12 +311,14 @@ def test_rings_at_even_addresses_off_word_alignment(ctx, shift, profile):
     assert np.array_equal(fl.cpu().numpy().view(np.uint32), w.frag_len.astype(np.uint32))
 
 
-@pytest.mark.parametrize("mode", ["scan", "rule"])
+@pytest.mark.parametrize("mode", ["scan", "fixed", "rule"])
 def test_batch_larger_than_its_arena_is_refused(ctx, mode):
     """Such a batch would lap itself: its first and last requests would share
-    bytes, written in no particular order.  Nothing is moved."""
+    bytes, written in no particular order.  Nothing is moved.  With a declared
+    request size the host refuses the call; with scanned sizes the device does."""
     rule = mode == "rule"
-    sizes = [4200] * 5 if rule else [3000, 5000, 700, 4100, 2222]
+    declared = mode != "scan"
+    sizes = [4200] * 5 if declared else [3000, 5000, 700, 4100, 2222]
     w = synth.make_custom(sizes, [64] * 5, seed=11)
     cap = int(sum(sizes)) - 1
     dw = DeviceWorkload(w)
@@ -324,16 +326,58 @@ def test_batch_larger_than_its_arena_is_refused(ctx, mode):
     ctx.set_cursor(0, 0)
     with pytest.raises(SgError) as e:
         ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, AppRef(arena=arena, cap=cap),
-                         flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if rule else 0, mtu=w.mtu)
-    assert e.value.code == (capi.SG_E_INVAL if rule else capi.SG_E_DATA)
+                         flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if declared else 0, mtu=w.mtu)
+    assert e.value.code == (capi.SG_E_INVAL if declared else capi.SG_E_DATA)
     assert bool((arena == 7).all())
+    assert ctx.get_cursor(0) == 0, "a refused batch does not advance the bump ring"
     # one byte more and it fits
     ctx.set_cursor(0, 0)
     arena2 = torch.zeros(cap + 1, dtype=torch.uint8, device=DEV)
     ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, AppRef(arena=arena2, cap=cap + 1),
-                     flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if rule else 0, mtu=w.mtu)
+                     flags=capi.F_RULE_FRAGS if rule else 0, fixed_req_size=sizes[0] if declared else 0, mtu=w.mtu)
     exp, _, _ = oracle.gather(w, arena_cap=cap + 1)
     assert np.array_equal(arena2.cpu().numpy(), exp)
+
+
+def test_cursor_after_a_rule_batch_with_a_bad_last_slot(ctx):
+    """A rule batch whose LAST fragment names a slot beyond the ring: that
+    fragment is dropped and the call reports SG_E_DATA, but the bump ring still
+    advances by the whole batch (the advance does not depend on the tables), so
+    the next batch lands where the host-side ring says it does."""
+    sizes = [4200] * 6
+    w = synth.make_custom(sizes, [64] * 6, seed=77)
+    dw = DeviceWorkload(w)
+    cap = 3 * int(sum(sizes)) + 100
+    arena = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+    app = AppRef(arena=arena, cap=cap)
+    offs = torch.zeros(w.n_req + 1, dtype=torch.int64, device=DEV)
+    bad = w.frag_slot.copy()
+    bad[-1] = w.n_slots + 1
+    start = cap - 9000
+    ctx.set_cursor(0, start)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch(dw.rx, to_dev(bad, DEV), None, dw.req_first, dw.n_req, dw.n_frags, app, offs,
+                         flags=capi.F_RULE_FRAGS, fixed_req_size=sizes[0], mtu=w.mtu)
+    assert e.value.code == capi.SG_E_DATA
+    want = np.zeros(cap, np.uint8)
+    _, eoffs, cur = oracle.gather(w, arena_cap=cap, cursor=start, out=want)
+    assert ctx.get_cursor(0) == cur
+    assert np.array_equal(offs.cpu().numpy().view(np.uint64), eoffs)
+    # every fragment but the dropped one is in place
+    got = arena.cpu().numpy()
+    last_len = int(w.frag_len[-1])
+    hole = (int(eoffs[-2]) + sizes[0] - last_len + np.arange(last_len)) % cap
+    keep = np.ones(cap, bool)
+    keep[hole] = False
+    assert np.array_equal(got[keep], want[keep])
+    # and the next batch continues from there
+    ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, app, offs,
+                     flags=capi.F_RULE_FRAGS, fixed_req_size=sizes[0], mtu=w.mtu)
+    want, eoffs, cur2 = oracle.gather(w, arena_cap=cap, cursor=cur, out=want)
+    assert ctx.get_cursor(0) == cur2
+    assert np.array_equal(offs.cpu().numpy().view(np.uint64), eoffs)
+    got = arena.cpu().numpy()
+    assert np.array_equal(got[keep], want[keep])
 
 
 def test_odd_arena_base_and_tensor_major_split(ctx):

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_gather_scatter_recorded_into_a_graph_and_replayed():
-    """Two steps (an even number of calls per arena, see sg_hip.h) of the
+    """Two steps of the
     single-batch gather + scatter are recorded on the context's stream and
     replayed; every replay is held against the oracle, with eager work and
     synchronisation between the replays."""
@@ -54,14 +54,18 @@ def test_gather_scatter_recorded_into_a_graph_and_replayed():
     ctx.close()
 
 
-def test_replays_continue_the_bump_ring():
-    """An arena of three batches and a graph of two gather calls: every replay
-    takes up the cursor where the previous one left it."""
+@pytest.mark.parametrize("mode", ["rule", "fixed", "scan"])
+@pytest.mark.parametrize("calls", [1, 2, 3])
+def test_replays_continue_the_bump_ring(mode, calls):
+    """An arena that no whole number of batches fills and a graph of one, two
+    or three gather calls: every replay takes up the cursor where the previous
+    one left it, whatever the number of calls recorded (the cursor is one
+    device word that only the device advances)."""
     import oracle
     from splitrpc_amd.engine import AppRef
     w = synth.make_workload(1, 8)
     batch = int(w.req_sizes.sum())
-    cap = 3 * batch
+    cap = 3 * batch + 1000
     s = torch.cuda.Stream()
     ctx = SgContext(0, max_reqs=64, max_frames=8192, stream=s.cuda_stream)
     dw = DeviceWorkload(w)
@@ -69,19 +73,20 @@ def test_replays_continue_the_bump_ring():
     app = AppRef(arena=arena, cap=cap)
     offs = torch.zeros(w.n_req + 1, dtype=torch.int64, device="cuda")
     a = ctx.gather_args(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, app, offs,
-                        flags=capi.F_ASYNC | capi.F_RULE_FRAGS, fixed_req_size=int(w.req_sizes[0]), mtu=w.mtu)
+                        flags=capi.F_ASYNC | (capi.F_RULE_FRAGS if mode == "rule" else 0),
+                        fixed_req_size=int(w.req_sizes[0]) if mode != "scan" else 0, mtu=w.mtu)
     ctx.set_cursor(0, 0)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g, stream=s):
-        ctx.gather_batch_raw(a)
-        ctx.gather_batch_raw(a)
+        for _ in range(calls):
+            ctx.gather_batch_raw(a)
     want = np.zeros(cap, np.uint8)
     cur = 0
     for rep in range(5):
         g.replay()
         torch.cuda.synchronize()
-        for _ in range(2):
+        for _ in range(calls):
             want, eoffs, cur = oracle.gather(w, arena_cap=cap, cursor=cur, out=want)
         got = arena.cpu().numpy()
         assert np.array_equal(got, want), f"replay {rep}: " + first_diff(got, want)
