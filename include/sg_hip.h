@@ -276,6 +276,33 @@ int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_te
 int sg_hip_gather_batch(sg_hip_ctx *ctx, const sg_gather_args *args);
 int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
 
+/* The gather call for callers that cannot allocate.  No counterpart in the
+ * reference: it is for code running under HIP graph capture, tight serving
+ * loops and harnesses that forbid hipMalloc.  Same semantics and same kernels
+ * as sg_hip_gather_batch, but without a context: the descriptor scratch lives
+ * in a static device array of about 1.1 MiB that each GPU the library runs on
+ * holds until the process ends, which is why one call takes at most
+ * SG_STATIC_MAX_REQS requests in SG_STATIC_MAX_FRAMES fragments (a larger batch
+ * is refused with SG_E_INVAL; split it or use a context).  The call launches
+ * kernels on `stream` (NULL: the default stream) and returns; it allocates and
+ * frees nothing, copies nothing, and never waits.  The first call on a device
+ * looks up that device's copy of the array.
+ *   cursor  device word holding the bump-ring position of the arena, read and
+ *           advanced by the call; NULL: a word inside the array, which starts
+ *           at zero and carries over from call to call
+ *   status  device word that receives refusal bits (non-zero after the stream
+ *           has drained: something was refused, as SG_E_DATA from
+ *           sg_hip_sync).  The caller zeroes it: with a descriptor pass a
+ *           non-zero status on entry means "refused" and nothing moves.  NULL:
+ *           a word inside the array, cleared by each call, that nobody reads.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (two streams, two threads) race and must not be made.
+ * sg_hip_last_error(NULL) gives the text of a refusal by the host. */
+#define SG_STATIC_MAX_REQS 4096u
+#define SG_STATIC_MAX_FRAMES 65536u
+int sg_hip_gather_batch_static(int device_id, void *stream, const sg_gather_args *args, uint64_t *cursor,
+                               uint32_t *status);
+
 /* Sorts a burst of arrivals into requests (see sg_reassemble_args).
  * Synchronous: the counts come back to the host because the caller sizes the
  * gather call with them.  n_left: arrivals that belong to no completed

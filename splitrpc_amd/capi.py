@@ -38,8 +38,11 @@ SYMBOLS = [
     "sg_hip_create", "sg_hip_destroy", "sg_hip_last_error", "sg_hip_abi_version", "sg_hip_stream",
     "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_set_hdrs", "sg_hip_gather_batch",
     "sg_hip_scatter_batch", "sg_hip_reassemble", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
-    "sg_hip_kernel_time",
+    "sg_hip_kernel_time", "sg_hip_gather_batch_static",
 ]
+
+STATIC_MAX_REQS = 4096
+STATIC_MAX_FRAMES = 65536
 
 
 class HBufs(C.Structure):
@@ -125,6 +128,7 @@ def load() -> C.CDLL:
                                     C.c_uint32, C.c_uint32]
     lib.sg_hip_gather_batch.argtypes = [P, C.POINTER(GatherArgs)]
     lib.sg_hip_scatter_batch.argtypes = [P, C.POINTER(ScatterArgs)]
+    lib.sg_hip_gather_batch_static.argtypes = [C.c_int, P, C.POINTER(GatherArgs), P, P]
     lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32),
                                       C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
     lib.sg_hip_set_cursor.argtypes = [P, C.c_int, C.c_uint64]

@@ -24,6 +24,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -1184,7 +1185,30 @@ __global__ __launch_bounds__(256) void k_ra_wipe(RaArgs a)
   a.want[cell] = 0;
 }
 
+// Sets `n` 32-bit words to zero (a fill kernel rather than a memset node, so
+// that callers may record the launch into a graph).
+__global__ __launch_bounds__(kBlock) void k_zero_words(uint32_t *p, uint32_t n)
+{
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
 }  // namespace
+
+// ---------------------------------------------------------------------------
+// scratch of the allocation-free entry point
+// ---------------------------------------------------------------------------
+// One array per GPU the library runs on, held until the process ends.  Host
+// code never uses the array's name as an address: the address on each device
+// comes from hipGetSymbolAddress (static_scratch_of below).
+namespace {
+constexpr size_t kStaticDesc = sizeof(u32x4) * (size_t)SG_STATIC_MAX_FRAMES;
+constexpr size_t kStaticReq = sizeof(uint64_t) * (size_t)SG_STATIC_MAX_REQS;
+constexpr size_t kStaticTile = sizeof(uint64_t) * (SG_STATIC_MAX_REQS / kScanTile + 2);
+constexpr size_t kStaticWords = 256;  // cursors, staged cursors, status, refusal flag
+constexpr size_t kStaticBytes = kStaticDesc + 2 * kStaticReq + kStaticTile + kStaticWords;
+}  // namespace
+static __device__ __align__(256) uint8_t scratch[kStaticBytes];
 
 // ---------------------------------------------------------------------------
 // host side
@@ -1979,6 +2003,66 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
   DeviceGuard g(c->device);
   return scatter_impl(c, c->sc, c->stream, a);
+}
+
+// ---- allocation-free gather ---------------------------------------------------
+
+namespace {
+constexpr int kStaticMaxDevices = 64;
+std::mutex g_static_mu;
+uint8_t *g_static_ptr[kStaticMaxDevices];  // device address of `scratch` on each GPU, once asked for
+
+// The device address of this GPU's copy of the static array (every GPU holds
+// its own copy at its own address).  The device must be current.
+int static_scratch_of(int device, uint8_t **out)
+{
+  if (device < 0 || device >= kStaticMaxDevices) return fail(nullptr, SG_E_INVAL, "device %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[device]) {
+    uint8_t *p = nullptr;
+    HIP_TRY(nullptr, hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(nullptr, SG_E_HIP, "hipGetSymbolAddress returned a null address on device %d", device);
+    g_static_ptr[device] = p;
+  }
+  *out = g_static_ptr[device];
+  return SG_OK;
+}
+}  // namespace
+
+int sg_hip_gather_batch_static(int device_id, void *stream, const sg_gather_args *a, uint64_t *cursor,
+                               uint32_t *status)
+{
+  if (!a) return fail(nullptr, SG_E_INVAL, "null argument");
+  DeviceGuard g(device_id);
+  if (!g.ok) return fail(nullptr, SG_E_HIP, "cannot select device %d", device_id);
+  uint8_t *base = nullptr;
+  int rc = static_scratch_of(device_id, &base);
+  if (rc != SG_OK) return rc;
+  if (a->n_req > SG_STATIC_MAX_REQS || a->n_frags > SG_STATIC_MAX_FRAMES)
+    return fail(nullptr, SG_E_INVAL,
+                "%u requests in %u fragments: the allocation-free gather takes at most %u requests in %u fragments",
+                a->n_req, a->n_frags, (unsigned)SG_STATIC_MAX_REQS, (unsigned)SG_STATIC_MAX_FRAMES);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Scratch sc;
+  sc.max_reqs = SG_STATIC_MAX_REQS;
+  sc.max_frames = SG_STATIC_MAX_FRAMES;
+  uint8_t *m = base;
+  sc.desc = reinterpret_cast<u32x4 *>(m); m += kStaticDesc;
+  sc.req_size = reinterpret_cast<uint64_t *>(m); m += kStaticReq;
+  sc.req_off = reinterpret_cast<uint64_t *>(m); m += kStaticReq;
+  sc.tile_tot = reinterpret_cast<uint64_t *>(m); m += kStaticTile;
+  uint64_t *w64 = reinterpret_cast<uint64_t *>(m);      // [0] the array's own cursor, [1] unused, [2] staged cursor
+  uint32_t *w32 = reinterpret_cast<uint32_t *>(m + 64);  // [0] the array's own status word, [1] refusal flag
+  sc.cursor[0] = cursor ? cursor : w64;
+  sc.cursor[1] = nullptr;
+  sc.next_cursor[0] = w64 + 2;
+  sc.next_cursor[1] = nullptr;
+  sc.status = status ? status : w32;
+  sc.flag = w32 + 1;
+  // descriptors, request totals, offsets and the staged cursor are written by this call's own
+  // kernels before they are read; the array's own status word would carry the last call's refusals
+  if (!status) k_zero_words<<<1, kBlock, 0, st>>>(w32, 2);
+  return gather_impl(nullptr, sc, st, a);
 }
 
 // ---- reassembly ----------------------------------------------------------------
