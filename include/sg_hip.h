@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define SG_HIP_ABI_VERSION 1
+#define SG_HIP_ABI_VERSION 2
 
 /* Error codes. */
 #define SG_OK 0
@@ -63,6 +63,12 @@ extern "C" {
                                           kernel could derive the descriptors (for experiments) */
 #define SG_F_ASYNC (1u << 16)          /* enqueue only; completion through sg_hip_sync() */
 #define SG_F_NO_XCD_REMAP (1u << 17)   /* launch-order = item order (for experiments) */
+
+/* States of an application slot (APP_RR_STATUS, src/p2p_rpc_app_ctx.h:22). */
+#define SG_SLOT_FREE 0u
+#define SG_SLOT_RX_COMPLETE 1u
+#define SG_SLOT_WORK_COMPLETE 2u
+#define SG_SLOT_TX_COMPLETE 3u
 
 #define SG_MAX_BI_SIZE 1024 /* src/p2p_bufs.h:10 */
 #define SG_MAX_TENSORS 4    /* src/p2p_rpc_app_stub.h:10 */
@@ -147,6 +153,26 @@ typedef struct sg_gather_args {
                               src/p2p_rpc_rr_ng.h:107-110); a batch holding another size is
                               refused with SG_E_DATA.  0: sizes are whatever the fragments add
                               up to and offsets come from a prefix scan */
+  /* Counts that stay on the device: [0] requests, [1] fragments, as
+   * sg_hip_reassemble leaves them in sg_reassemble_args.counts_out.  n_req and
+   * n_frags above are then upper bounds that size the launches (a count beyond
+   * its bound is refused with SG_E_DATA); no host synchronization sits between
+   * the reassembly and this call.  NULL: n_req and n_frags are the counts. */
+  const uint32_t *counts; /* device, or NULL */
+  /* Application slot ring (the h_state words of P2pRpcAppRrPool,
+   * src/p2p_rpc_app_rr.h:15-46,127-134): request k of the batch fills slot
+   * (producer index + k) mod n_slot_states; once the batch is in place a kernel
+   * behind the copy kernel sets those words from SG_SLOT_FREE to
+   * SG_SLOT_RX_COMPLETE (what the shunter does at
+   * src/splitrpc_server/p2p_rpc_dpdk_server.cc:130) and advances the producer
+   * index, which lives on the device (sg_hip_set_slot_index).  A slot found in
+   * another state is still overwritten and the call reports SG_E_DATA: the
+   * caller keeps at most n_slot_states requests between gather and scatter, as
+   * the reference's flow control does (:117).  The words may live in device
+   * memory or in pinned host memory the worker's loop polls.  NULL: no ring. */
+  uint32_t *slot_state; /* device-addressable, n_slot_states words, or NULL */
+  uint32_t n_slot_states;
+  uint32_t reserved2;
 } sg_gather_args;
 
 /* One scatter batch.  Response r has resp_size[r] bytes (fixed_resp_size when
@@ -182,31 +208,59 @@ typedef struct sg_scatter_args {
    * lengths and sums.  Nothing is swapped and hdr_src_slot is not read. */
   const uint8_t *hdr_templates; /* device, n_req * 64 bytes, or NULL: swap request headers */
   const uint64_t *req_token;    /* device, n_req, or NULL */
+  /* One header source per request instead of one per frame: every frame of
+   * response r answers the header in RX slot hdr_src_req[r] (what
+   * sg_hip_reassemble leaves in req_hdr_slot).  Used when hdr_src_slot is NULL. */
+  const uint32_t *hdr_src_req; /* device, n_req, or NULL */
+  /* Device-resident request count, as in sg_gather_args: counts[0] responses
+   * are served, n_req and n_frames are upper bounds (frame tables must be
+   * valid up to the bounds). */
+  const uint32_t *counts;      /* device, or NULL */
+  /* Application slot ring: the n_req slots from the consumer index on
+   * (sg_hip_set_slot_index, which = 1) are expected in SG_SLOT_WORK_COMPLETE;
+   * behind the copy kernel they are set to SG_SLOT_FREE
+   * (src/splitrpc_server/p2p_rpc_dpdk_server.cc:158-175) and the index advances. */
+  uint32_t *slot_state;        /* device-addressable, n_slot_states words, or NULL */
+  uint32_t n_slot_states;
+  uint32_t reserved2;
 } sg_scatter_args;
 
 /* One burst of arrivals to sort into requests on the device.  Replaces the
  * per-packet work of the receive thread: get_rr / rr_emplace_mbuf /
  * is_rr_ready / mark_rx_ready_rr (src/p2p_rpc_rr_pool_ng.h:97-119,149-155;
- * src/transport/dpdk_transport_ng.h:221-252).  A request is complete when
- * num_frags fragments are in (BL58) or when its payload bytes reach req_size
- * (REF64, src/p2p_rpc_rr_ng.h:107-110).  Completed requests come out in
- * completion order -- the order in which their last fragment arrived, which
- * is the order of the reference's rx-ready ring -- as the CSR tables
- * sg_hip_gather_batch takes.  Packets with token 0 are dropped (:231);
- * arrivals of requests that do not complete within this burst are left out
- * and counted.  As in the reference, duplicate fragments are not detected. */
+ * src/transport/dpdk_transport_ng.h:176-252, one NIC burst per call).  A
+ * request is complete when num_frags fragments are in (BL58) or when its
+ * payload bytes reach req_size (REF64, src/p2p_rpc_rr_ng.h:107-110).  Requests
+ * that are still incomplete stay on the device, as rr_cache keeps them
+ * (src/p2p_rpc_rr_pool_ng.h:97-119), and complete in whichever later call
+ * brings their last fragment; up to max_reqs of the context may be in flight.
+ * The requests completed by a call come out in completion order -- the order
+ * in which their last fragment arrived, which is the order of the reference's
+ * rx-ready ring -- as the CSR tables sg_hip_gather_batch takes, fragments of
+ * earlier calls included, so the output tables need room for max_frames
+ * fragments and max_reqs requests of the context.  Packets with token 0 are
+ * dropped (:231).  As in the reference, duplicate fragments are not detected,
+ * and a request holds at most SG_MAX_BI_SIZE fragments.  A token that comes
+ * back within the burst that completes it is taken for the same request. */
 typedef struct sg_reassemble_args {
   sg_ring_desc ring;
   const uint32_t *arrivals; /* device, n_arrivals: ring slots in arrival order */
   const uint32_t *len_nic;  /* device, n_slots: payload bytes of each slot as the NIC reports
                                them (required for REF64; NULL for BL58: read from the header) */
-  uint32_t n_arrivals;
-  uint32_t reserved;
+  uint32_t n_arrivals;      /* arrivals of this call; their upper bound with n_arrivals_dev */
+  uint32_t flags;           /* SG_F_ASYNC: launch only, counts stay on the device */
   uint64_t req_size;        /* REF64: the server-wide request size */
-  uint32_t *frag_slot;      /* device out, n_arrivals */
-  uint32_t *frag_len;       /* device out, n_arrivals */
+  uint32_t *frag_slot;      /* device out, max_frames of the context */
+  uint32_t *frag_len;       /* device out, max_frames of the context */
   uint32_t *req_first;      /* device out, max_reqs + 1 of the context */
   uint64_t *req_token;      /* device out, max_reqs, or NULL */
+  uint32_t *req_hdr_slot;   /* device out, max_reqs, or NULL: the slot of each request's fragment 0,
+                               whose header the responses answer (sg_scatter_args.hdr_src_req) */
+  uint32_t *counts_out;     /* device out, 4 words, or NULL: requests completed, their fragments,
+                               arrivals dropped, requests still in flight -- what
+                               sg_gather_args.counts / sg_scatter_args.counts take */
+  const uint32_t *n_arrivals_dev; /* device, or NULL: the arrival count when it is only known on
+                                     the device (a burst whose length changes between graph replays) */
 } sg_reassemble_args;
 
 /* ---- lifetime -------------------------------------------------------------
@@ -304,17 +358,35 @@ int sg_hip_gather_batch_static(int device_id, void *stream, const sg_gather_args
                                uint32_t *status);
 
 /* Sorts a burst of arrivals into requests (see sg_reassemble_args).
- * Synchronous: the counts come back to the host because the caller sizes the
- * gather call with them.  n_left: arrivals that belong to no completed
- * request. */
-int sg_hip_reassemble(sg_hip_ctx *ctx, const sg_reassemble_args *args, uint32_t *n_req_out,
-                      uint32_t *n_frags_out, uint32_t *n_left_out);
+ * Synchronous unless SG_F_ASYNC is set; then counts_host_out is not written and
+ * the counts are where counts_out says.  counts_host_out (4 words, or NULL):
+ * requests completed, their fragments, arrivals dropped, requests still in
+ * flight.  The first call on a context allocates the request table and the
+ * record pool (8 KiB per request of max_reqs): make it, or
+ * sg_hip_reassemble_reset, before recording calls into a graph. */
+int sg_hip_reassemble(sg_hip_ctx *ctx, const sg_reassemble_args *args, uint32_t *counts_host_out);
+
+/* Drops every request in flight (and allocates the state on first use). */
+int sg_hip_reassemble_reset(sg_hip_ctx *ctx);
+
+/* Drops the requests that no fragment has come in for during the last
+ * max_age_calls calls of sg_hip_reassemble: a request that lost a fragment is
+ * parked for good in the reference (src/p2p_rpc_rr_pool_ng.h:57-64 lists such
+ * leftovers at shutdown); here the caller can clear them out.  Synchronous. */
+int sg_hip_reassemble_evict(sg_hip_ctx *ctx, uint32_t max_age_calls, uint32_t *n_evicted_out);
 
 /* Device-resident bump-ring cursors (P2pRpcTring::prev_offset,
  * src/p2p_rpc_tring.h:14-16), one for the request arena (which = 0) and one
  * for the response arena (which = 1).  Both calls synchronize. */
 int sg_hip_set_cursor(sg_hip_ctx *ctx, int which, uint64_t value);
 int sg_hip_get_cursor(sg_hip_ctx *ctx, int which, uint64_t *value);
+
+/* Device-resident indices into the application slot ring, the shunter's
+ * rr_pi_idx and rr_ci_idx (src/splitrpc_server/p2p_rpc_dpdk_server.cc:98,141,183):
+ * which = 0 the next slot a gather fills, which = 1 the next slot a scatter
+ * serves.  Both calls synchronize. */
+int sg_hip_set_slot_index(sg_hip_ctx *ctx, int which, uint32_t value);
+int sg_hip_get_slot_index(sg_hip_ctx *ctx, int which, uint32_t *value);
 
 /* ---- measurement -------------------------------------------------------------
  * With profiling on, every kernel launch is bracketed by HIP events on the

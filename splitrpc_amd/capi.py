@@ -38,8 +38,11 @@ SYMBOLS = [
     "sg_hip_create", "sg_hip_destroy", "sg_hip_last_error", "sg_hip_abi_version", "sg_hip_stream",
     "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_set_hdrs", "sg_hip_gather_batch",
     "sg_hip_scatter_batch", "sg_hip_reassemble", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
-    "sg_hip_kernel_time", "sg_hip_gather_batch_static",
+    "sg_hip_kernel_time", "sg_hip_gather_batch_static", "sg_hip_reassemble_reset", "sg_hip_reassemble_evict",
+    "sg_hip_set_slot_index", "sg_hip_get_slot_index",
 ]
+
+SLOT_FREE, SLOT_RX_COMPLETE, SLOT_WORK_COMPLETE, SLOT_TX_COMPLETE = 0, 1, 2, 3
 
 STATIC_MAX_REQS = 4096
 STATIC_MAX_FRAMES = 65536
@@ -76,7 +79,8 @@ class GatherArgs(C.Structure):
     _fields_ = [("ring", RingDesc), ("frag_slot", C.c_void_p), ("frag_len", C.c_void_p),
                 ("req_first", C.c_void_p), ("n_req", C.c_uint32), ("n_frags", C.c_uint32),
                 ("app", AppDesc), ("offsets_out", C.c_void_p), ("flags", C.c_uint32),
-                ("mtu", C.c_uint32), ("fixed_req_size", C.c_uint64)]
+                ("mtu", C.c_uint32), ("fixed_req_size", C.c_uint64), ("counts", C.c_void_p),
+                ("slot_state", C.c_void_p), ("n_slot_states", C.c_uint32), ("reserved2", C.c_uint32)]
 
 
 class ScatterArgs(C.Structure):
@@ -84,14 +88,17 @@ class ScatterArgs(C.Structure):
                 ("hdr_src_slot", C.c_void_p), ("resp_first", C.c_void_p), ("resp_size", C.c_void_p),
                 ("fixed_resp_size", C.c_uint64), ("n_req", C.c_uint32), ("n_frames", C.c_uint32),
                 ("mtu", C.c_uint32), ("flags", C.c_uint32), ("app", AppDesc),
-                ("offsets_out", C.c_void_p), ("hdr_templates", C.c_void_p), ("req_token", C.c_void_p)]
+                ("offsets_out", C.c_void_p), ("hdr_templates", C.c_void_p), ("req_token", C.c_void_p),
+                ("hdr_src_req", C.c_void_p), ("counts", C.c_void_p), ("slot_state", C.c_void_p),
+                ("n_slot_states", C.c_uint32), ("reserved2", C.c_uint32)]
 
 
 class ReassembleArgs(C.Structure):
     _fields_ = [("ring", RingDesc), ("arrivals", C.c_void_p), ("len_nic", C.c_void_p),
-                ("n_arrivals", C.c_uint32), ("reserved", C.c_uint32), ("req_size", C.c_uint64),
+                ("n_arrivals", C.c_uint32), ("flags", C.c_uint32), ("req_size", C.c_uint64),
                 ("frag_slot", C.c_void_p), ("frag_len", C.c_void_p), ("req_first", C.c_void_p),
-                ("req_token", C.c_void_p)]
+                ("req_token", C.c_void_p), ("req_hdr_slot", C.c_void_p), ("counts_out", C.c_void_p),
+                ("n_arrivals_dev", C.c_void_p)]
 
 
 _lib = None
@@ -129,8 +136,11 @@ def load() -> C.CDLL:
     lib.sg_hip_gather_batch.argtypes = [P, C.POINTER(GatherArgs)]
     lib.sg_hip_scatter_batch.argtypes = [P, C.POINTER(ScatterArgs)]
     lib.sg_hip_gather_batch_static.argtypes = [C.c_int, P, C.POINTER(GatherArgs), P, P]
-    lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32),
-                                      C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+    lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32 * 4)]
+    lib.sg_hip_reassemble_reset.argtypes = [P]
+    lib.sg_hip_reassemble_evict.argtypes = [P, C.c_uint32, C.POINTER(C.c_uint32)]
+    lib.sg_hip_set_slot_index.argtypes = [P, C.c_int, C.c_uint32]
+    lib.sg_hip_get_slot_index.argtypes = [P, C.c_int, C.POINTER(C.c_uint32)]
     lib.sg_hip_set_cursor.argtypes = [P, C.c_int, C.c_uint64]
     lib.sg_hip_get_cursor.argtypes = [P, C.c_int, C.POINTER(C.c_uint64)]
     lib.sg_hip_set_profiling.argtypes = [P, C.c_int]

@@ -22,6 +22,8 @@ constexpr uint32_t kStBadSize = 1u << 2;     // request larger than its destinat
 constexpr uint32_t kStBadFrames = 1u << 3;   // response frame count disagrees with the fragmenting rule
 constexpr uint32_t kStBadTable = 1u << 4;    // CSR table is not a gap-free tiling of the items
 constexpr uint32_t kStNotRule = 1u << 5;     // a fragment's length departs from the fragmenting rule
+constexpr uint32_t kStSlotState = 1u << 6;   // an application slot was not in the state the call expects
+constexpr uint32_t kStPoolFull = 1u << 7;    // more requests in flight than the reassembly pool holds
 constexpr uint32_t kInvalidReq = 0xffffffffu; // owner field of a descriptor the kernels must skip
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -94,10 +94,37 @@ struct PrepArgs {
   // mode 1: where each frame's header comes from, held against the RX ring here
   // so that a bad index refuses the batch before anything is written
   const uint32_t *hdr_src_slot;
+  const uint32_t *hdr_src_req;  // or one header source per request
   uint32_t rx_n_slots;
+  // Counts that live on the device (what sg_hip_reassemble left): [0] requests,
+  // [1] items.  n_req and n_items above are then upper bounds the launch was
+  // sized with.  nullptr: the bounds are the counts.
+  const uint32_t *counts;
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
+
+// The counts a kernel works with: the host's, or the device's held against the
+// host's bounds.  More requests on the device than the launch was sized for is
+// refused by k_finish / the descriptor pass.
+__device__ __forceinline__ uint32_t dev_count(const uint32_t *counts, uint32_t k, uint32_t bound)
+{
+  if (!counts) return bound;
+  const uint32_t v = sload(counts + k);
+  return v < bound ? v : bound;
+}
+
+__device__ __forceinline__ void prep_effective(PrepArgs &a)
+{
+  if (!a.counts) return;
+  const uint32_t n = sload(a.counts);
+  if (n > a.n_req) refuse(a.status, a.status_flag, kStBadSize);
+  a.n_req = n < a.n_req ? n : a.n_req;
+  // gather: the item count comes with the request count; scatter: it is where the frame table ends
+  const uint32_t items = a.mode == 0 ? sload(a.counts + 1) : (a.n_req ? a.first[a.n_req] : 0u);
+  if (a.mode == 0 && items > a.n_items) refuse(a.status, a.status_flag, kStBadSize);
+  a.n_items = items < a.n_items ? items : a.n_items;
+}
 
 // Exclusive scan over the threads of a workgroup of BLOCK threads, built from
 // wavefront scans (DPP/permute shuffles) and one LDS slot per wavefront.
@@ -182,6 +209,7 @@ __device__ __forceinline__ uint32_t prep_range(const PrepArgs &a, uint32_t r, ui
       *f0 = *f1 = 0;
       *size = 0;
     }
+    if (a.hdr_src_req && a.hdr_src_req[r] >= a.rx_n_slots) bad |= kStBadSlot;
   }
   return bad;
 }
@@ -215,7 +243,9 @@ template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void k_prep_block(PrepArgs a)
 {
   __shared__ uint64_t wave_tot[BLOCK / kWave];
+  prep_effective(a);
   const uint32_t r = blockIdx.x;
+  if (r >= a.n_req) return;
   uint32_t f0, f1;
   uint64_t size;
   uint32_t bad = prep_range(a, r, &f0, &f1, &size);
@@ -241,6 +271,7 @@ __global__ __launch_bounds__(BLOCK) void k_prep_block(PrepArgs a)
 // One wavefront per request (requests of at most a few dozen fragments).
 __global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
 {
+  prep_effective(a);
   const uint32_t r = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (r >= a.n_req) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -313,6 +344,7 @@ __device__ __forceinline__ void scan_check_batch(const PrepArgs &a, uint64_t bat
 __global__ __launch_bounds__(kScanBlock) void k_req_scan(PrepArgs a)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  prep_effective(a);
   uint64_t run = *a.cursor % a.cap, batch_bytes = 0;
   for (uint32_t base = 0; base < a.n_req; base += kScanTile) {
     const uint32_t q0 = base + threadIdx.x * kScanPerThread;
@@ -402,18 +434,52 @@ __device__ __forceinline__ uint32_t item_of_wave(bool remap)
 // states where the caller keeps them.  A recorded graph may therefore hold any
 // number of calls.
 struct FinishArgs {
-  uint64_t *cursor;      // advanced by n_req * size modulo cap; nullptr: nothing to advance
+  uint64_t *cursor;       // advanced by n_req * size modulo cap; nullptr: nothing to advance
   uint64_t size;
   uint64_t cap;
-  uint32_t n_req;
+  uint32_t n_req;         // requests of the call, or their upper bound with `counts`
+  const uint32_t *counts; // device-resident request count, or nullptr
+  // Application slot states (the h_state words of the reference's app_rr pool,
+  // src/p2p_rpc_app_rr.h:15-46): the n_req slots from *slot_idx on go from
+  // `expect` to `publish`, and *slot_idx moves on by n_req (modulo n_states).
+  uint32_t *state;        // nullptr: no slot ring
+  uint32_t n_states;
+  uint32_t *slot_idx;
+  uint32_t expect, publish;
+  uint32_t all_or_nothing;  // a refused batch publishes and advances nothing (descriptor pass)
+  uint32_t *status;
+  volatile uint32_t *status_flag;
 };
 
 __global__ __launch_bounds__(kBlock) void k_finish(FinishArgs a)
 {
+  const uint32_t refused = *a.status;  // what earlier kernels left
+  __syncthreads();                     // read by every thread before this kernel adds to it
+  uint32_t n = a.n_req;
+  if (a.counts) {
+    const uint32_t v = sload(a.counts);
+    if (v > n && threadIdx.x == 0) refuse(a.status, a.status_flag, kStBadSize);  // the launch was sized for fewer
+    n = v < n ? v : n;
+  }
+  if (a.all_or_nothing && refused) return;
   if (a.cursor && threadIdx.x == 0) {
     // bump ring with equal sizes: off = (off + size) % capacity, n_req times
     const uint64_t c = *a.cursor;
-    *a.cursor = (c % a.cap + ((uint64_t)a.n_req * a.size) % a.cap) % a.cap;
+    *a.cursor = (c % a.cap + ((uint64_t)n * a.size) % a.cap) % a.cap;
+  }
+  if (a.state) {
+    const uint32_t i0 = *a.slot_idx % a.n_states;
+    uint32_t bad = 0;
+    for (uint32_t k = threadIdx.x; k < n; k += kBlock) {
+      uint32_t s = i0 + k % a.n_states;
+      s = s >= a.n_states ? s - a.n_states : s;
+      // the words may live in pinned host memory, where the worker's loop reads and writes them
+      if (__hip_atomic_load(a.state + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != a.expect) bad = 1;
+      __hip_atomic_store(a.state + s, a.publish, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    if (bad) refuse(a.status, a.status_flag, kStSlotState);
+    __syncthreads();  // every thread has read *slot_idx
+    if (threadIdx.x == 0) *a.slot_idx = (i0 + n % a.n_states) % a.n_states;
   }
 }
 
@@ -448,13 +514,14 @@ struct GatherArgs {
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   uint64_t *cursor;             // packed: wavefront 0 commits *next_cursor unless the batch was refused
   const uint64_t *next_cursor;
+  const uint32_t *counts;       // device-resident counts ([0] requests, [1] items), or nullptr
   AppDev app;
 };
 
 // Descriptor of item `item` from the rule; publishes the request offset and, on
 // the batch's last item, the advanced cursor.  Returns status bits.
 __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &app, uint32_t item,
-                                              uint32_t n_items, uint32_t lane, uint32_t *slot,
+                                              uint32_t n_items, uint32_t n_req, uint32_t lane, uint32_t *slot,
                                               uint32_t *len, uint32_t *off, uint32_t *r,
                                               uint32_t *i, uint64_t *req_off)
 {
@@ -482,7 +549,7 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
       if (item == n_items - 1 && g.offsets_out) {
         uint64_t end = *req_off + g.size;  // size <= capacity
         end = end >= app.cap ? end - app.cap : end;
-        g.offsets_out[g.n_req] = end;
+        g.offsets_out[n_req] = end;
       }
     }
   }
@@ -586,17 +653,22 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   const u32x4 *desc = a.desc;
   const uint64_t *req_off = a.req_off;
   const uint8_t *ring = a.ring;
-  const uint32_t slot_size = a.slot_size, hl = a.hl, n_items = a.n_items, remap = a.remap;
+  const uint32_t slot_size = a.slot_size, hl = a.hl, remap = a.remap;
   const uint32_t pieces = a.pieces;
   const uint32_t *status = a.status;
+  const uint32_t *counts = a.counts;
+  uint32_t n_items = a.n_items;
   SG_PIN(desc); SG_PIN(req_off); SG_PIN(ring); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_items);
-  SG_PIN(remap); SG_PIN(status); SG_PIN(pieces);
+  SG_PIN(remap); SG_PIN(status); SG_PIN(pieces); SG_PIN(counts);
+  if (counts) n_items = dev_count(counts, 1, n_items);
   const uint32_t w = item_of_wave(remap != 0);
   const uint32_t item = LONG ? w / pieces : w;
   const uint32_t piece = LONG ? w - item * pieces : 0;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   // this kernel does not read the cursor: the value the descriptor pass left is committed here
-  if (w == 0 && lane == 0 && a.cursor && !sload(status)) *a.cursor = sload(a.next_cursor);
+  // (a batch of no requests at all has left none)
+  if (w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts)))
+    *a.cursor = sload(a.next_cursor);
   if (item >= n_items) return;
   const u32x4 d = sload_here(desc + item);  // asked for together with the status word
   if (sload_here(status)) return;           // the descriptor pass refused the batch: move nothing
@@ -645,6 +717,7 @@ struct GatherRuleArgs {
   const uint32_t *frag_len;
   const uint32_t *first;
   uint64_t *offsets_out;
+  const uint32_t *counts;     // device-resident counts ([0] requests, [1] fragments), or nullptr
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   AppDev app;  // consulted for several tensor-major buffers only
@@ -662,12 +735,19 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   uint8_t *dst = a.dst;
   const uint64_t *cursor_in = a.cursor;
   const uint64_t size = a.size, cap = a.cap;
-  const uint32_t n_items = a.n_items, per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
+  const uint32_t per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
   const uint32_t hl = a.hl, n_slots = a.n_slots, pieces = a.pieces, opts = a.opts;
   const uint32_t div_mul = a.div_mul, div_shift = a.div_shift;
+  const uint32_t *counts = a.counts;
+  uint32_t n_items = a.n_items, n_req = a.n_req;
   SG_PIN(ring); SG_PIN(frag_slot); SG_PIN(dst); SG_PIN(cursor_in); SG_PIN(size); SG_PIN(cap);
   SG_PIN(n_items); SG_PIN(per_req); SG_PIN(mtu); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_slots);
-  SG_PIN(pieces); SG_PIN(opts); SG_PIN(div_mul); SG_PIN(div_shift);
+  SG_PIN(pieces); SG_PIN(opts); SG_PIN(div_mul); SG_PIN(div_shift); SG_PIN(counts);
+  if (counts) {
+    // counts left on the device by the reassembly: the launch was sized for n_req requests at most
+    n_req = dev_count(counts, 0, n_req);
+    n_items = n_req * per_req;
+  }
 
   const uint32_t w = item_of_wave((opts & kOptRemap) != 0);
   const uint32_t item = LONG ? w / pieces : w;
@@ -697,7 +777,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
       if (i == 0) a.offsets_out[r] = ro;
       if (item == n_items - 1) {
         uint64_t end = ro + size;  // size <= capacity
-        a.offsets_out[a.n_req] = end >= cap ? end - cap : end;
+        a.offsets_out[n_req] = end >= cap ? end - cap : end;
       }
     }
     uint64_t o = ro + off;  // < 2 * capacity
@@ -768,12 +848,15 @@ struct ScatterArgs {
   uint32_t ref64;
   uint32_t flags;
   uint32_t n_items;
+  uint32_t n_req;
   uint32_t remap;
   uint32_t pieces;  // wavefronts per frame
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   uint64_t *cursor;             // descriptor path, packed: wavefront 0 commits *next_cursor
   const uint64_t *next_cursor;
+  const uint32_t *hdr_src_req;  // one header source per request instead of hdr_src_slot per frame
+  const uint32_t *counts;       // device-resident request count, or nullptr
   RuleArgs rule;
   AppDev app;
 };
@@ -797,11 +880,19 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   const uint8_t *hdr_templates = a.hdr_templates, *rx = a.rx;
   uint8_t *tx = a.tx;
   const uint32_t rx_slot_size = a.rx_slot_size, rx_n_slots = a.rx_n_slots, tx_slot_size = a.tx_slot_size;
-  const uint32_t hl = a.hl, n_items = a.n_items, remap = a.remap, n_pieces = a.pieces;
+  const uint32_t hl = a.hl, remap = a.remap, n_pieces = a.pieces;
   const uint32_t *status = a.status;
+  const uint32_t *counts = a.counts, *hdr_src_req = a.hdr_src_req;
+  uint32_t n_items = a.n_items, n_req = a.n_req;
   SG_PIN(desc); SG_PIN(req_off); SG_PIN(first); SG_PIN(hdr_src_slot); SG_PIN(hdr_templates); SG_PIN(rx);
   SG_PIN(tx); SG_PIN(rx_slot_size); SG_PIN(rx_n_slots); SG_PIN(tx_slot_size); SG_PIN(hl); SG_PIN(n_items);
-  SG_PIN(remap); SG_PIN(n_pieces); SG_PIN(status);
+  SG_PIN(remap); SG_PIN(n_pieces); SG_PIN(status); SG_PIN(counts); SG_PIN(hdr_src_req);
+  if (counts) {
+    // the launch was sized for n_req responses at most; the frame table ends where the live ones end
+    n_req = dev_count(counts, 0, n_req);
+    const uint32_t live = FUSED ? n_req * a.rule.per_req : (n_req ? sload(first + n_req) : 0u);
+    n_items = live < n_items ? live : n_items;
+  }
   SG_PIN(a.app.n_tensors); SG_PIN(a.app.arena); SG_PIN(a.app.cap); SG_PIN(a.app.mirrored);
   if (FUSED) {
     SG_PIN(a.rule.item_slot); SG_PIN(a.rule.first); SG_PIN(a.rule.size); SG_PIN(a.rule.mtu);
@@ -813,11 +904,12 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   const uint32_t piece = SPLIT ? w - item * pieces : 0;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   // descriptor path: this kernel does not read the cursor and commits what the descriptor pass left
-  if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status)) *a.cursor = sload(a.next_cursor);
+  if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts)))
+    *a.cursor = sload(a.next_cursor);
   if (item >= n_items) return;
   const bool from_template = hdr_templates != nullptr;
   // independent table reads, asked for together
-  const uint32_t hs = from_template ? 0u : sload_here(hdr_src_slot + item);
+  uint32_t hs = (from_template || hdr_src_req) ? 0u : sload_here(hdr_src_slot + item);
   u32x4 d;
   uint32_t r, f0, nf;
   uint64_t ro;
@@ -831,7 +923,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     ro = a.app.n_tensors == 0 ? sload(req_off + r) : 0;
   } else {
     uint32_t slot_i, len, off, i;
-    const uint32_t bad = rule_desc(a.rule, a.app, item, a.n_items, piece == 0 ? lane : 1u, &slot_i, &len,
+    const uint32_t bad = rule_desc(a.rule, a.app, item, n_items, n_req, piece == 0 ? lane : 1u, &slot_i, &len,
                                    &off, &r, &i, &ro);
     if (bad) {
       if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, bad);
@@ -854,6 +946,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
       hf.token = a.req_token[r];
     }
   } else {
+    if (hdr_src_req) hs = sload(hdr_src_req + r);
     if (hs >= rx_n_slots) {
       // descriptor path: the descriptor pass has refused the batch already and nothing gets here
       if (FUSED && lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
@@ -946,49 +1039,79 @@ __global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, 
 // What the receive thread of the reference does per packet -- look the request
 // up by token (get_rr), file the fragment at its sequence number
 // (rr_emplace_mbuf), hand the request over once complete (is_rr_ready,
-// mark_rx_ready_rr) -- done for a whole burst of arrivals at once:
-//   k_ra_insert  one thread per arrival: open-addressing insert of the token
-//                into a hash table (atomicCAS on the key, linear probing over a
-//                table at least twice the arrivals: every probe makes progress,
-//                nothing waits), fragment count / byte total / last arrival
-//                position per request by atomics
-//   k_ra_flag    the thread of a complete request's LAST arrival flags that
+// mark_rx_ready_rr) -- done for a whole burst of arrivals at once, with the
+// requests that are still incomplete kept on the device from call to call, as
+// rr_cache keeps them (src/p2p_rpc_rr_pool_ng.h:97-119):
+//   request table   token -> cell, open addressing in buckets of kRaBucket
+//                   cells: a lookup reads the whole bucket, so emptying a cell
+//                   (a completed request) never hides another request, and a
+//                   new token claims the lowest empty cell by atomicCAS
+//   record pool     one record per request in flight: SG_MAX_BI_SIZE entries
+//                   {slot, length} indexed by sequence number (p2p_bufs of the
+//                   reference's rr); free records wait in a ring with a head
+//                   and a tail word on the device (the rr pool's free ring,
+//                   src/p2p_rpc_rr_pool_ng.h:121-147: consume_rr / reap_rr)
+//   k_ra_insert  one thread per arrival: find or claim the request's cell (a
+//                claimed cell takes a record off the free ring), add to its
+//                fragment count / byte total, note the arrival's position
+//   k_ra_flag    every arrival files its entry in its request's record; the
+//                thread of a complete request's LAST arrival flags that
 //                position with the request's fragment count; workgroup-local
 //                scan of the packed (requests, fragments) flags
-//   k_ra_scan    one workgroup scans the workgroup totals
+//   k_ra_scan    one workgroup scans the workgroup totals and leaves the counts
+//                on the device and in pinned host memory
 //   k_ra_emit    batch index of a request = number of requests completed before
-//                it (completion order, the order of the rx-ready ring), read
-//                off the scan at its last arrival; every arrival of a complete
-//                request writes its table entry at first + seq_num
-//   k_ra_wipe    empties the cells this call used
+//                it in this call (completion order, the order of the rx-ready
+//                ring); the wavefront of the completing arrival copies the
+//                record into the output tables, empties it, returns it to the
+//                free ring and empties the cell
+// Nothing waits on another thread: every probe and every ring operation makes
+// progress by itself.
+
+constexpr uint32_t kRaBucket = 32;
+constexpr uint32_t kRaNoCell = 0xffffffffu;
+constexpr uint32_t kRaNoRec = 0xffffffffu;
+constexpr int kRaBlock = 1024;
+// device words of the reassembly state
+enum { kRaHead = 0, kRaTail, kRaEpoch, kRaInFlight, kRaClaims, kRaDropped, kRaOverflow, kRaEvicted, kRaWords = 16 };
 
 struct RaArgs {
   const uint8_t *ring;
-  uint32_t n_slots, slot_size, ref64, n;
+  uint32_t n_slots, slot_size, ref64;
+  uint32_t n;             // arrivals of this call, or their upper bound with n_dev
+  const uint32_t *n_dev;  // device-resident arrival count, or nullptr
   const uint32_t *arrivals;
   const uint32_t *len_nic;
   uint64_t req_size;  // REF64 readiness: bytes == req_size; BL58: fragments == num_frags
-  uint32_t hmask;     // table size - 1
-  uint32_t max_req;
-  // hash table
+  uint32_t bmask;     // buckets - 1
+  uint32_t rmask;     // records - 1
+  uint32_t max_req, max_frag;  // room in the output tables
+  // request table: cells
   unsigned long long *keys;
-  uint32_t *cnt, *last, *want;
   unsigned long long *bytes;
-  // per arrival
+  uint32_t *cnt, *want, *last, *rec, *seen;
+  // record pool
+  unsigned long long *tab;  // records x SG_MAX_BI_SIZE entries: slot | length << 32
+  uint32_t *free_ring;
+  uint32_t *words;          // kRa* above
+  // per arrival of this call
   uint32_t *arr_cell, *arr_len, *arr_fidx;
   unsigned long long *arr_pack;  // (1 << 32 | fragments) at the completing arrival, else 0; then its local scan
-  unsigned long long *blk;       // workgroup totals, then their scan; blk[n_blocks] = grand total
+  unsigned long long *blk;       // workgroup totals, then their scan
   uint32_t n_blocks;
   // outputs
-  uint32_t *frag_slot, *frag_len, *req_first;
+  uint32_t *frag_slot, *frag_len, *req_first, *req_hdr_slot;
   uint64_t *req_token;
-  volatile uint32_t *counts;  // pinned host memory: [0] requests, [1] fragments
+  uint32_t *counts_out;            // device: requests, fragments, arrivals dropped, requests in flight
+  volatile uint32_t *counts_host;  // the same four, pinned host memory
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
 
-constexpr uint32_t kRaNoCell = 0xffffffffu;
-constexpr int kRaBlock = 1024;
+__device__ __forceinline__ uint32_t ra_n(const RaArgs &a)
+{
+  return dev_count(a.n_dev, 0, a.n);
+}
 
 __device__ __forceinline__ uint32_t ra_hash(unsigned long long k)
 {
@@ -998,18 +1121,67 @@ __device__ __forceinline__ uint32_t ra_hash(unsigned long long k)
   return (uint32_t)k;
 }
 
-// Find or claim the hash cell of `token`: linear probing from its hash; a plain
-// read first, since nearly every arrival finds its request already present.
-__device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long long token)
+__device__ __forceinline__ unsigned long long ra_key(const unsigned long long *p)
 {
-  uint32_t c = ra_hash(token) & a.hmask;
-  for (uint32_t probe = 0; probe <= a.hmask; probe++) {
-    unsigned long long old = __hip_atomic_load(&a.keys[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (old == 0ull) old = atomicCAS(&a.keys[c], 0ull, token);
-    if (old == 0ull || old == token) return c;
-    c = (c + 1) & a.hmask;
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Find or claim the cell of `token`.  The whole bucket is read first: the
+// request may sit behind cells that have emptied since it came in.  Only then
+// is the lowest empty cell claimed; a thread walking the bucket tries every
+// empty cell it meets, so two threads that bring the same new token end up in
+// the same cell whatever else is claimed around them.
+__device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long long token, bool *claimed)
+{
+  const uint32_t b = (ra_hash(token) & a.bmask) * kRaBucket;
+  *claimed = false;
+#pragma unroll 1
+  for (uint32_t h = 0; h < kRaBucket; h += 16) {
+    unsigned long long k[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) k[j] = ra_key(a.keys + b + h + j);
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+      if (k[j] == token) return b + h + j;
   }
-  return kRaNoCell;
+#pragma unroll 1
+  for (uint32_t j = 0; j < kRaBucket; j++) {
+    unsigned long long k = ra_key(a.keys + b + j);
+    if (k == 0ull) {
+      k = atomicCAS(&a.keys[b + j], 0ull, token);
+      if (k == 0ull) {
+        *claimed = true;
+        return b + j;
+      }
+    }
+    if (k == token) return b + j;
+  }
+  return kRaNoCell;  // bucket full
+}
+
+// A record off the free ring, or kRaNoRec.  The tail does not move during the
+// kernel that takes records (returns happen in k_ra_emit), so the head may
+// advance up to the tail read here; the compare-and-swap never takes a record
+// that is not there.
+__device__ __forceinline__ uint32_t ra_take_record(const RaArgs &a)
+{
+  const uint32_t tail = a.words[kRaTail];
+  uint32_t h = __hip_atomic_load(&a.words[kRaHead], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while ((int32_t)(tail - h) > 0) {
+    const uint32_t old = atomicCAS(&a.words[kRaHead], h, h + 1);
+    if (old == h) return a.free_ring[h & a.rmask];
+    h = old;  // somebody else took that one: progress was made
+  }
+  return kRaNoRec;
+}
+
+// A newly claimed cell: take a record and stamp the cell.
+__device__ __forceinline__ void ra_open_cell(const RaArgs &a, uint32_t c)
+{
+  const uint32_t r = ra_take_record(a);
+  a.rec[c] = r;
+  atomicAdd(&a.words[kRaClaims], 1u);
+  if (r == kRaNoRec) refuse(a.status, a.status_flag, kStPoolFull);
 }
 
 // Fragments of one request tend to arrive together, so the lanes of a
@@ -1021,9 +1193,11 @@ constexpr int kRaRounds = 4;
 
 __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
 {
+  const uint32_t n = ra_n(a);
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  const bool in_range = i < a.n;
+  const bool in_range = i < n;
+  const uint32_t epoch = a.words[kRaEpoch];  // advanced by k_ra_scan, behind this kernel
   uint32_t cell = kRaNoCell, len = 0, fidx = 0, want = 0;
   unsigned long long token = 0;
   bool pending = false;
@@ -1064,12 +1238,15 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
     const uint32_t g_bytes = wave_sum(mine ? len : 0u);
     uint32_t c = kRaNoCell;
     if ((int)lane == first) {
-      c = ra_find_cell(a, t);
+      bool claimed;
+      c = ra_find_cell(a, t, &claimed);
       if (c != kRaNoCell) {
+        if (claimed) ra_open_cell(a, c);
         atomicAdd(&a.cnt[c], (uint32_t)__popcll(group));
         atomicAdd(&a.bytes[c], (unsigned long long)g_bytes);
         atomicMax(&a.last[c], i - lane + (63u - (uint32_t)__clzll((long long)group)));
         if (!a.ref64) a.want[c] = want;  // every fragment of a request says the same
+        a.seen[c] = epoch;
       }
     }
     c = (uint32_t)__shfl((int)c, first, kWave);
@@ -1079,19 +1256,26 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
     }
   }
   if (pending) {
-    cell = ra_find_cell(a, token);
+    bool claimed;
+    cell = ra_find_cell(a, token, &claimed);
     if (cell != kRaNoCell) {
+      if (claimed) ra_open_cell(a, cell);
       atomicAdd(&a.cnt[cell], 1u);
       atomicAdd(&a.bytes[cell], (unsigned long long)len);
       atomicMax(&a.last[cell], i);
       if (!a.ref64) a.want[cell] = want;
+      a.seen[cell] = epoch;
     }
   }
   if (in_range) {
     a.arr_cell[i] = cell;
     a.arr_len[i] = len;
     a.arr_fidx[i] = fidx;
+    if (cell == kRaNoCell && token != 0) refuse(a.status, a.status_flag, kStPoolFull);  // bucket full
   }
+  // arrivals that belong to no request: token 0, refused, no room
+  const unsigned long long lost = __ballot(in_range && cell == kRaNoCell);
+  if (lane == 0 && lost) atomicAdd(&a.words[kRaDropped], (uint32_t)__popcll(lost));
 }
 
 __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell)
@@ -1102,87 +1286,172 @@ __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell)
 __global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
 {
   __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  const uint32_t n = ra_n(a);
   const uint32_t i = blockIdx.x * kRaBlock + threadIdx.x;
   unsigned long long pack = 0;
-  if (i < a.n) {
+  if (i < n) {
     const uint32_t cell = a.arr_cell[i];
-    if (cell != kRaNoCell && a.last[cell] == i && ra_complete(a, cell))
-      pack = (1ull << 32) | a.cnt[cell];
+    const uint32_t r = cell != kRaNoCell ? a.rec[cell] : kRaNoRec;
+    if (r != kRaNoRec) {
+      const uint32_t fidx = a.arr_fidx[i];
+      if (fidx < SG_MAX_BI_SIZE) {
+        // rr_emplace_mbuf: the entry goes where its sequence number says
+        a.tab[(size_t)r * SG_MAX_BI_SIZE + fidx] = (unsigned long long)a.arrivals[i] | ((unsigned long long)a.arr_len[i] << 32);
+      } else {
+        refuse(a.status, a.status_flag, kStBadTable);  // beyond what a request's tables hold (src/p2p_bufs.h:10)
+      }
+      const uint32_t cnt = a.cnt[cell];
+      if (a.last[cell] == i && ra_complete(a, cell)) {
+        if (cnt <= SG_MAX_BI_SIZE) pack = (1ull << 32) | cnt;
+        else refuse(a.status, a.status_flag, kStBadTable);
+      }
+    }
   }
   uint64_t tot;
   const uint64_t ex = block_exclusive_scan<kRaBlock>(pack, wave_tot, &tot);
-  if (i < a.n) a.arr_pack[i] = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
+  if (i < n) a.arr_pack[i] = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
   if (threadIdx.x == 0) a.blk[blockIdx.x] = tot;
 }
 
 __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
 {
   __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  const uint32_t n = ra_n(a);
+  const uint32_t n_blocks = (n + kRaBlock - 1) / kRaBlock;
   uint64_t run = 0;
-  for (uint32_t base = 0; base < a.n_blocks; base += kRaBlock) {
+  for (uint32_t base = 0; base < n_blocks; base += kRaBlock) {
     const uint32_t b = base + threadIdx.x;
-    const uint64_t v = b < a.n_blocks ? a.blk[b] : 0;
+    const uint64_t v = b < n_blocks ? a.blk[b] : 0;
     uint64_t tot;
     const uint64_t ex = block_exclusive_scan<kRaBlock>(v, wave_tot, &tot);
-    if (b < a.n_blocks) a.blk[b] = run + ex;
+    if (b < n_blocks) a.blk[b] = run + ex;
     run += tot;
   }
   if (threadIdx.x == 0) {
-    a.blk[a.n_blocks] = run;
-    const uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
-    a.counts[0] = n_req;  // straight into pinned host memory: nothing to copy back
-    a.counts[1] = n_frag;
-    if (n_req <= a.max_req) a.req_first[n_req] = n_frag;
-    else refuse(a.status, a.status_flag, kStBadTable);
-  }
-}
-
-// Every arrival of a complete request writes its table entry.  The request's
-// rank and first fragment index hang on its LAST arrival (arr_pack there, plus
-// the scanned total of that arrival's workgroup); that arrival also writes the
-// request's row of req_first / req_token.
-__global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
-{
-  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i < a.n) {
-    const uint32_t cell = a.arr_cell[i];
-    if (cell != kRaNoCell) {
-      const uint32_t last = a.last[cell];
-      const unsigned long long p = a.arr_pack[last];
-      if (p >> 63) {  // the request completed among these arrivals
-        const unsigned long long v = (p & ~(1ull << 63)) + a.blk[last / kRaBlock];
-        const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v;
-        if (r < a.max_req) {  // else refused by k_ra_scan
-          const uint32_t n = a.cnt[cell];
-          const uint32_t fidx = a.arr_fidx[i];
-          if (fidx < n) {
-            a.frag_slot[first + fidx] = a.arrivals[i];
-            a.frag_len[first + fidx] = a.arr_len[i];
-          } else {
-            refuse(a.status, a.status_flag, kStBadTable);  // a sequence number beyond the request's fragments
-          }
-          if (i == last) {
-            a.req_first[r] = first;
-            if (a.req_token) a.req_token[r] = a.keys[cell];
-          }
-        }
-      }
+    uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
+    uint32_t overflow = 0;
+    if (n_req > a.max_req || n_frag > a.max_frag) {
+      // the output tables cannot take what completed: nothing is emitted, the requests stay parked
+      refuse(a.status, a.status_flag, kStBadTable);
+      overflow = 1;
+      n_req = n_frag = 0;
+    }
+    a.words[kRaOverflow] = overflow;
+    a.req_first[n_req] = n_frag;
+    const uint32_t in_flight = a.words[kRaInFlight] + a.words[kRaClaims] - n_req;
+    const uint32_t dropped = a.words[kRaDropped];
+    a.words[kRaInFlight] = in_flight;
+    a.words[kRaClaims] = 0;
+    a.words[kRaDropped] = 0;
+    a.words[kRaEpoch] += 1;
+    const uint32_t c[4] = {n_req, n_frag, dropped, in_flight};
+    for (int k = 0; k < 4; k++) {
+      if (a.counts_out) a.counts_out[k] = c[k];
+      a.counts_host[k] = c[k];  // straight into pinned host memory: nothing to copy back
     }
   }
 }
 
-// Wipes the cells this call used, so that the table is empty for the next one.
-__global__ __launch_bounds__(256) void k_ra_wipe(RaArgs a)
+// The wavefront of a completing arrival hands the request over: its record goes
+// into the output tables in sequence order, the record is emptied and returned
+// to the free ring, the cell is emptied.  The request's rank and first fragment
+// index hang on that arrival (arr_pack there plus its workgroup's scanned total).
+__global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
 {
+  const uint32_t n = ra_n(a);
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= a.n) return;
-  const uint32_t cell = a.arr_cell[i];
-  if (cell == kRaNoCell) return;
-  a.keys[cell] = 0;
-  a.cnt[cell] = 0;
-  a.bytes[cell] = 0;
-  a.last[cell] = 0;
-  a.want[cell] = 0;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const bool overflow = a.words[kRaOverflow] != 0;
+  uint32_t cell = kRaNoCell;
+  unsigned long long v = 0;
+  bool completes = false;
+  if (i < n) {
+    cell = a.arr_cell[i];
+    const unsigned long long p = a.arr_pack[i];
+    completes = cell != kRaNoCell && (p >> 63) && !overflow;
+    if (completes) v = (p & ~(1ull << 63)) + a.blk[i / kRaBlock];
+    // the position of a request's last arrival counts per call
+    if (cell != kRaNoCell && !completes) a.last[cell] = 0;
+  }
+  unsigned long long todo = __ballot(completes);
+  while (todo) {
+    const int l = __ffsll((long long)todo) - 1;
+    todo &= todo - 1;
+    const uint32_t c = (uint32_t)__shfl((int)cell, l, kWave);
+    const uint32_t r = (uint32_t)__shfl((int)(uint32_t)(v >> 32), l, kWave);
+    const uint32_t first = (uint32_t)__shfl((int)(uint32_t)v, l, kWave);
+    const uint32_t rc = a.rec[c], cnt = a.cnt[c];
+    unsigned long long *t = a.tab + (size_t)rc * SG_MAX_BI_SIZE;
+    for (uint32_t j = lane; j < cnt; j += kWave) {
+      const unsigned long long e = t[j];
+      a.frag_slot[first + j] = (uint32_t)e;
+      a.frag_len[first + j] = (uint32_t)(e >> 32);
+      t[j] = 0;  // a fresh request finds an empty record
+      if (j == 0) {
+        a.req_first[r] = first;
+        if (a.req_token) a.req_token[r] = a.keys[c];
+        if (a.req_hdr_slot) a.req_hdr_slot[r] = (uint32_t)e;  // the slot whose header the responses answer
+      }
+    }
+    if (lane == 0) {
+      // reap_rr: the record goes back to the free ring, the token leaves the table
+      const uint32_t tl = atomicAdd(&a.words[kRaTail], 1u);
+      a.free_ring[tl & a.rmask] = rc;
+      a.cnt[c] = 0;
+      a.bytes[c] = 0;
+      a.last[c] = 0;
+      a.want[c] = 0;
+      a.rec[c] = kRaNoRec;
+      __hip_atomic_store(&a.keys[c], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// Empties the table: every cell, every record, all records back in the ring.
+__global__ __launch_bounds__(256) void k_ra_reset(RaArgs a, uint32_t cells, uint32_t records)
+{
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < cells) {
+    a.keys[i] = 0;
+    a.bytes[i] = 0;
+    a.cnt[i] = a.want[i] = a.last[i] = a.seen[i] = 0;
+    a.rec[i] = kRaNoRec;
+  }
+  if (i < records) a.free_ring[i] = (uint32_t)i;
+  if (i < (size_t)records * SG_MAX_BI_SIZE) a.tab[i] = 0;
+  if (i < kRaWords) a.words[i] = i == kRaTail ? records : 0u;
+}
+
+// Drops the requests no fragment has come in for during the last max_age calls
+// (a lost fragment parks its request for good in the reference,
+// src/p2p_rpc_rr_pool_ng.h:57-64; here the caller can clear such requests out).
+// One wavefront per cell.
+__global__ __launch_bounds__(256) void k_ra_evict(RaArgs a, uint32_t cells, uint32_t max_age)
+{
+  const uint32_t c = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  if (c >= cells) return;
+  if (a.keys[c] == 0ull) return;
+  if (a.words[kRaEpoch] - a.seen[c] <= max_age) return;
+  const uint32_t rc = a.rec[c];
+  if (rc != kRaNoRec) {
+    unsigned long long *t = a.tab + (size_t)rc * SG_MAX_BI_SIZE;
+    for (uint32_t j = lane; j < SG_MAX_BI_SIZE; j += kWave) t[j] = 0;
+  }
+  if (lane == 0) {
+    if (rc != kRaNoRec) {
+      const uint32_t tl = atomicAdd(&a.words[kRaTail], 1u);
+      a.free_ring[tl & a.rmask] = rc;
+    }
+    a.cnt[c] = 0;
+    a.bytes[c] = 0;
+    a.last[c] = 0;
+    a.want[c] = 0;
+    a.rec[c] = kRaNoRec;
+    a.keys[c] = 0;
+    atomicSub(&a.words[kRaInFlight], 1u);
+    atomicAdd(&a.words[kRaEvicted], 1u);
+  }
 }
 
 // Sets `n` 32-bit words to zero (a fill kernel rather than a memset node, so
@@ -1232,6 +1501,7 @@ struct Scratch {
   // descriptor pass stages for the copy kernel to commit
   uint64_t *cursor[2] = {nullptr, nullptr};
   uint64_t *next_cursor[2] = {nullptr, nullptr};
+  uint32_t *slot_idx[2] = {nullptr, nullptr};  // next slot of the application ring to fill / to serve
   uint32_t *status = nullptr;
   volatile uint32_t *flag = nullptr;  // raised with every refusal (pinned host memory in a context)
 };
@@ -1263,8 +1533,9 @@ struct sg_hip_ctx {
   uint64_t prof_n[6] = {0, 0, 0, 0, 0, 0};
   // reassembly scratch, allocated by the first sg_hip_reassemble call
   void *ra_mem = nullptr;
-  uint32_t ra_cells = 0;  // hash table size (power of two >= 2 * max_frames)
-  uint32_t *h_counts = nullptr;  // pinned: requests, fragments (written by k_ra_scan itself)
+  uint32_t ra_cells = 0;    // cells of the request table (power of two >= 4 * max_reqs)
+  uint32_t ra_records = 0;  // records of the pool (power of two >= max_reqs)
+  uint32_t *h_counts = nullptr;  // pinned: requests, fragments, dropped, in flight (written by k_ra_scan itself)
   char err[512] = {0};
 };
 
@@ -1407,7 +1678,7 @@ int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs
     k_prep_block<1024><<<p.n_req, 1024, 0, st>>>(p);
   }
   if (p.packed && !p.fixed_offsets) {
-    if (p.n_req <= 2 * kScanTile) {
+    if (p.n_req <= 2 * kScanTile || p.counts) {  // counts on the device: one workgroup walks whatever is there
       k_req_scan<<<1, kScanBlock, 0, st>>>(p);
     } else {
       const uint32_t n_tiles = (p.n_req + kScanTile - 1) / kScanTile;
@@ -1418,15 +1689,29 @@ int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs
   return prof_end(c);
 }
 
-// Behind the copy kernel of a single-kernel call on a packed arena.
-void launch_finish(hipStream_t st, uint64_t *cursor, uint64_t size, uint64_t cap, uint32_t n_req)
+// Behind the copy kernel: advance the cursor (single-kernel calls on a packed
+// arena) and publish slot states (where the caller keeps a slot ring).
+void launch_finish(const Scratch &sc, hipStream_t st, uint64_t *cursor, uint64_t size, uint64_t cap, uint32_t n_req,
+                   const uint32_t *counts, uint32_t *state, uint32_t n_states, int which, bool all_or_nothing)
 {
+  if (!cursor && !state) return;
   FinishArgs f;
   memset(&f, 0, sizeof f);
   f.cursor = cursor;
   f.size = size;
   f.cap = cap;
   f.n_req = n_req;
+  f.counts = counts;
+  f.state = state;
+  f.n_states = n_states;
+  f.slot_idx = sc.slot_idx[which];
+  // gather fills FREE slots and publishes RX_COMPLETE; scatter serves WORK_COMPLETE slots and
+  // frees them (src/splitrpc_server/p2p_rpc_dpdk_server.cc:130,175; states src/p2p_rpc_app_ctx.h:22)
+  f.expect = which == 0 ? SG_SLOT_FREE : SG_SLOT_WORK_COMPLETE;
+  f.publish = which == 0 ? SG_SLOT_RX_COMPLETE : SG_SLOT_FREE;
+  f.all_or_nothing = all_or_nothing ? 1u : 0u;
+  f.status = sc.status;
+  f.status_flag = sc.flag;
   k_finish<<<1, kBlock, 0, st>>>(f);
 }
 
@@ -1496,9 +1781,9 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->tile_tot, sizeof(uint64_t) * ((size_t)c->max_reqs / kScanTile + 2)));
-  HIP_TRY(nullptr, hipMalloc(&c->cursors, 4 * sizeof(uint64_t)));
+  HIP_TRY(nullptr, hipMalloc(&c->cursors, 5 * sizeof(uint64_t)));  // [4]: the two slot indices
   HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
-  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 4 * sizeof(uint64_t), c->stream));
+  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 5 * sizeof(uint64_t), c->stream));
   HIP_TRY(nullptr, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
   c->h_runs_cap = 8192;
   HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
@@ -1518,6 +1803,8 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   sc.cursor[1] = c->cursors + 1;
   sc.next_cursor[0] = c->cursors + 2;
   sc.next_cursor[1] = c->cursors + 3;
+  sc.slot_idx[0] = reinterpret_cast<uint32_t *>(c->cursors + 4);
+  sc.slot_idx[1] = sc.slot_idx[0] + 1;
   sc.status = c->status;
   sc.flag = c->h_flag;
   return SG_OK;
@@ -1578,13 +1865,15 @@ int sg_hip_sync(sg_hip_ctx *c)
     HIP_TRY(c, hipStreamSynchronize(c->stream));
     *c->h_flag = 0;
     const uint32_t st = c->h_status[0];
-    return fail(c, SG_E_DATA, "kernel refused input:%s%s%s%s%s%s",
+    return fail(c, SG_E_DATA, "kernel refused input:%s%s%s%s%s%s%s%s",
                 (st & kStBadSlot) ? " slot index beyond ring;" : "",
                 (st & kStBadLen) ? " fragment longer than a slot holds;" : "",
                 (st & kStBadSize) ? " request larger than its destination;" : "",
                 (st & kStBadFrames) ? " frame count disagrees with size/mtu;" : "",
                 (st & kStBadTable) ? " CSR table does not tile the items;" : "",
-                (st & kStNotRule) ? " a fragment's length departs from the fragmenting rule;" : "");
+                (st & kStNotRule) ? " a fragment's length departs from the fragmenting rule;" : "",
+                (st & kStSlotState) ? " an application slot was not in the state the call expects;" : "",
+                (st & kStPoolFull) ? " more requests in flight than the reassembly pool holds;" : "");
   }
   return SG_OK;
 }
@@ -1604,6 +1893,24 @@ int sg_hip_get_cursor(sg_hip_ctx *c, int which, uint64_t *value)
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
   HIP_TRY(c, hipMemcpy(value, c->cursors + which, sizeof *value, hipMemcpyDeviceToHost));
+  return SG_OK;
+}
+
+int sg_hip_set_slot_index(sg_hip_ctx *c, int which, uint32_t value)
+{
+  if (!c || which < 0 || which > 1) return fail(c, SG_E_INVAL, "slot index %d", which);
+  DeviceGuard g(c->device);
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  HIP_TRY(c, hipMemcpy(c->sc.slot_idx[which], &value, sizeof value, hipMemcpyHostToDevice));
+  return SG_OK;
+}
+
+int sg_hip_get_slot_index(sg_hip_ctx *c, int which, uint32_t *value)
+{
+  if (!c || !value || which < 0 || which > 1) return fail(c, SG_E_INVAL, "slot index %d", which);
+  DeviceGuard g(c->device);
+  HIP_TRY(c, hipStreamSynchronize(c->stream));
+  HIP_TRY(c, hipMemcpy(value, c->sc.slot_idx[which], sizeof *value, hipMemcpyDeviceToHost));
   return SG_OK;
 }
 
@@ -1740,6 +2047,9 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
   rc = check_app(c, a->app, &app, &max_req_bytes);
   if (rc != SG_OK) return rc;
   const bool packed = app.n_tensors == 0;
+  if (a->slot_state && a->n_slot_states == 0) return fail(c, SG_E_INVAL, "a slot ring of no slots");
+  if (a->slot_state && a->n_req > a->n_slot_states)
+    return fail(c, SG_E_INVAL, "%u requests do not fit a ring of %u application slots", a->n_req, a->n_slot_states);
   // a batch larger than the arena would lap itself and its wavefronts would race for the same bytes
   if (packed && a->fixed_req_size && (uint64_t)a->n_req * a->fixed_req_size > app.cap)
     return fail(c, SG_E_INVAL, "%u requests of %llu bytes do not fit an arena of %llu bytes", a->n_req,
@@ -1751,8 +2061,11 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     if (!a->fixed_req_size || !a->mtu) return fail(c, SG_E_INVAL, "SG_F_RULE_FRAGS needs fixed_req_size and mtu");
     if ((uint64_t)a->mtu + hl0 > a->ring.slot_size) return fail(c, SG_E_INVAL, "mtu %u + %u header bytes does not fit a %u-byte slot", a->mtu, hl0, a->ring.slot_size);
     const uint64_t per = (a->fixed_req_size + a->mtu - 1) / a->mtu;
-    if (per * a->n_req != a->n_frags) return fail(c, SG_E_INVAL, "%u requests of %llu bytes at mtu %u are %llu fragments, not %u", a->n_req, (unsigned long long)a->fixed_req_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frags);
-    if (a->n_frags >= (1u << 27)) return fail(c, SG_E_INVAL, "%u fragments in one call: the limit is 2^27 - 1", a->n_frags);
+    // with the counts on the device n_req and n_frags are bounds: the launch covers per * n_req fragments
+    if (a->counts ? per * a->n_req > sc.max_frames : per * a->n_req != a->n_frags)
+      return fail(c, SG_E_INVAL, "%u requests of %llu bytes at mtu %u are %llu fragments, not %u", a->n_req, (unsigned long long)a->fixed_req_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frags);
+    const uint32_t n_items = (uint32_t)(per * a->n_req);
+    if (n_items >= (1u << 27)) return fail(c, SG_E_INVAL, "%u fragments in one call: the limit is 2^27 - 1", n_items);
     if (a->fixed_req_size > 0xffffffffull || (packed ? a->fixed_req_size > app.cap : a->fixed_req_size > max_req_bytes))
       return fail(c, SG_E_INVAL, "request size %llu does not fit its destination", (unsigned long long)a->fixed_req_size);
     GatherRuleArgs ga;
@@ -1763,7 +2076,8 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     ga.cursor = sc.cursor[0];
     ga.size = a->fixed_req_size;
     ga.cap = packed ? app.cap : 0;
-    ga.n_items = a->n_frags;
+    ga.n_items = n_items;
+    ga.counts = a->counts;
     ga.per_req = (uint32_t)per;
     magic_div(per, &ga.div_mul, &ga.div_shift);
     ga.mtu = a->mtu;
@@ -1779,7 +2093,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     ga.app = app;
     ga.pieces = pieces_for(a->mtu);
     uint32_t grid, remap;
-    geometry((uint64_t)a->n_frags * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
+    geometry((uint64_t)n_items * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
               (app.n_tensors > 1 ? kOptMultiTensor : 0u) |
               ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
@@ -1789,7 +2103,8 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     else k_gather_rule<false><<<grid, kBlock, 0, st>>>(ga);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
-    if (packed) launch_finish(st, sc.cursor[0], a->fixed_req_size, app.cap, a->n_req);
+    launch_finish(sc, st, packed ? sc.cursor[0] : nullptr, a->fixed_req_size, app.cap, a->n_req, a->counts,
+                  a->slot_state, a->n_slot_states, 0, false);
     return finish(c, a->flags);
   }
 
@@ -1816,6 +2131,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
   p.cursor = sc.cursor[0];
   p.next_cursor = sc.next_cursor[0];
   p.offsets_out = packed ? a->offsets_out : nullptr;
+  p.counts = a->counts;
   p.status = sc.status;
   p.status_flag = sc.flag;
   rc = launch_prep(c, sc, st, p);
@@ -1837,6 +2153,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
       ga.cursor = sc.cursor[0];
       ga.next_cursor = sc.next_cursor[0];
     }
+    ga.counts = a->counts;
     ga.app = app;
     ga.pieces = pieces_for(p.slot_size - p.hl);
     uint32_t grid;
@@ -1848,6 +2165,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }
+  launch_finish(sc, st, nullptr, 0, 0, a->n_req, a->counts, a->slot_state, a->n_slot_states, 0, true);
   return finish(c, a->flags);
 }
 
@@ -1868,7 +2186,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
   if (a->n_req == 0) return SG_OK;
   if (a->n_req > sc.max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u", a->n_req, sc.max_reqs);
   if (a->n_frames > sc.max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u", a->n_frames, sc.max_frames);
-  if (!a->resp_first || (a->n_frames && (!a->tx_slot || (!a->hdr_src_slot && !a->hdr_templates))))
+  if (!a->resp_first || (a->n_frames && (!a->tx_slot || (!a->hdr_src_slot && !a->hdr_src_req && !a->hdr_templates))))
     return fail(c, SG_E_INVAL, "null frame tables");
   const uint32_t hl = hdr_len_of(a->tx.hdr_profile);
   if (a->mtu == 0 || (uint64_t)a->mtu + hl > a->tx.slot_size)
@@ -1879,13 +2197,18 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
   rc = check_app(c, a->app, &app, &max_req_bytes);
   if (rc != SG_OK) return rc;
   const bool packed = app.n_tensors == 0;
+  if (a->slot_state && a->n_slot_states == 0) return fail(c, SG_E_INVAL, "a slot ring of no slots");
+  if (a->slot_state && a->n_req > a->n_slot_states)
+    return fail(c, SG_E_INVAL, "%u responses do not fit a ring of %u application slots", a->n_req, a->n_slot_states);
 
   const bool fused = a->resp_size == nullptr && !(a->flags & SG_F_NO_FUSE);
   if (fused) {
     if (a->fixed_resp_size == 0 || a->fixed_resp_size > 0xffffffffull)
       return fail(c, SG_E_INVAL, "fixed response size %llu out of range", (unsigned long long)a->fixed_resp_size);
     const uint64_t per = (a->fixed_resp_size + a->mtu - 1) / a->mtu;
-    if (per * a->n_req != a->n_frames) return fail(c, SG_E_INVAL, "%u responses of %llu bytes at mtu %u are %llu frames, not %u", a->n_req, (unsigned long long)a->fixed_resp_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frames);
+    if (a->counts ? per * a->n_req > a->n_frames : per * a->n_req != a->n_frames)
+      return fail(c, SG_E_INVAL, "%u responses of %llu bytes at mtu %u are %llu frames, not %u", a->n_req, (unsigned long long)a->fixed_resp_size, a->mtu, (unsigned long long)(per * a->n_req), a->n_frames);
+    const uint32_t n_items = (uint32_t)(per * a->n_req);
     if (app.n_tensors == 0 ? a->fixed_resp_size > app.cap : a->fixed_resp_size > max_req_bytes)
       return fail(c, SG_E_INVAL, "response size %llu does not fit its source", (unsigned long long)a->fixed_resp_size);
     ScatterArgs sa;
@@ -1901,7 +2224,10 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.hl = hl;
     sa.ref64 = a->tx.hdr_profile == SG_HDR_REF64;
     sa.flags = a->flags & 0xfu;
-    sa.n_items = a->n_frames;
+    sa.n_items = n_items;
+    sa.n_req = a->n_req;
+    sa.counts = a->counts;
+    sa.hdr_src_req = a->hdr_templates ? nullptr : a->hdr_src_req;
     sa.status = sc.status;
     sa.status_flag = sc.flag;
     sa.app = app;
@@ -1917,14 +2243,15 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.rule.offsets_out = packed ? a->offsets_out : nullptr;
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
-    geometry((uint64_t)a->n_frames * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
+    geometry((uint64_t)n_items * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
              !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
     launch_scatter<true>(st, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
-    if (packed) launch_finish(st, sc.cursor[1], a->fixed_resp_size, app.cap, a->n_req);
+    launch_finish(sc, st, packed ? sc.cursor[1] : nullptr, a->fixed_resp_size, app.cap, a->n_req, a->counts,
+                  a->slot_state, a->n_slot_states, 1, false);
     return finish(c, a->flags);
   }
 
@@ -1952,9 +2279,11 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
   p.next_cursor = sc.next_cursor[1];
   p.offsets_out = packed ? a->offsets_out : nullptr;
   if (!a->hdr_templates) {
-    p.hdr_src_slot = a->hdr_src_slot;
+    if (a->hdr_src_req) p.hdr_src_req = a->hdr_src_req;
+    else p.hdr_src_slot = a->hdr_src_slot;
     p.rx_n_slots = a->rx.n_slots;
   }
+  p.counts = a->counts;
   p.status = sc.status;
   p.status_flag = sc.flag;
   rc = launch_prep(c, sc, st, p);
@@ -1978,6 +2307,9 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.ref64 = a->tx.hdr_profile == SG_HDR_REF64;
     sa.flags = a->flags & 0xfu;
     sa.n_items = a->n_frames;
+    sa.n_req = a->n_req;
+    sa.counts = a->counts;
+    sa.hdr_src_req = a->hdr_templates ? nullptr : a->hdr_src_req;
     sa.status = sc.status;
     sa.status_flag = sc.flag;
     if (packed) {
@@ -1995,6 +2327,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }
+  launch_finish(sc, st, nullptr, 0, 0, a->n_req, a->counts, a->slot_state, a->n_slot_states, 1, true);
   return finish(c, a->flags);
 }
 
@@ -2059,6 +2392,8 @@ int sg_hip_gather_batch_static(int device_id, void *stream, const sg_gather_args
   sc.next_cursor[1] = nullptr;
   sc.status = status ? status : w32;
   sc.flag = w32 + 1;
+  sc.slot_idx[0] = w32 + 2;  // the array's own producer index, for callers that pass a slot ring
+  sc.slot_idx[1] = w32 + 3;
   // descriptors, request totals, offsets and the staged cursor are written by this call's own
   // kernels before they are read; the array's own status word would carry the last call's refusals
   if (!status) k_zero_words<<<1, kBlock, 0, st>>>(w32, 2);
@@ -2067,87 +2402,149 @@ int sg_hip_gather_batch_static(int device_id, void *stream, const sg_gather_args
 
 // ---- reassembly ----------------------------------------------------------------
 
-int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *n_req_out, uint32_t *n_frags_out,
-                      uint32_t *n_left_out)
+namespace {
+
+uint32_t pow2_at_least(uint64_t v)
+{
+  uint32_t p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// Carves the reassembly state out of c->ra_mem (allocating it first where needed).
+int ra_state(sg_hip_ctx *c, RaArgs *r, bool *fresh)
+{
+  const uint32_t n_max = c->max_frames;
+  const uint32_t cells = pow2_at_least(4ull * c->max_reqs < 2 * kRaBucket ? 2 * kRaBucket : 4ull * c->max_reqs);
+  const uint32_t records = pow2_at_least(c->max_reqs);
+  const size_t n_blk = (n_max + kRaBlock - 1) / kRaBlock + 1;
+  const size_t bytes = (size_t)cells * (8 + 8 + 5 * 4) + (size_t)records * SG_MAX_BI_SIZE * 8 + (size_t)records * 4 +
+                       kRaWords * 4 + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 256;
+  *fresh = false;
+  if (!c->ra_mem) {
+    HIP_TRY(c, hipMalloc(&c->ra_mem, bytes));
+    HIP_TRY(c, hipHostMalloc((void **)&c->h_counts, 4 * sizeof(uint32_t), hipHostMallocDefault));
+    memset(c->h_counts, 0, 4 * sizeof(uint32_t));
+    c->ra_cells = cells;
+    c->ra_records = records;
+    *fresh = true;
+  }
+  memset(r, 0, sizeof *r);
+  uint8_t *m = static_cast<uint8_t *>(c->ra_mem);
+  r->keys = reinterpret_cast<unsigned long long *>(m); m += (size_t)cells * 8;
+  r->bytes = reinterpret_cast<unsigned long long *>(m); m += (size_t)cells * 8;
+  r->tab = reinterpret_cast<unsigned long long *>(m); m += (size_t)records * SG_MAX_BI_SIZE * 8;
+  r->arr_pack = reinterpret_cast<unsigned long long *>(m); m += (size_t)n_max * 8;
+  r->blk = reinterpret_cast<unsigned long long *>(m); m += n_blk * 8;
+  r->cnt = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
+  r->want = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
+  r->last = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
+  r->rec = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
+  r->seen = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
+  r->free_ring = reinterpret_cast<uint32_t *>(m); m += (size_t)records * 4;
+  r->words = reinterpret_cast<uint32_t *>(m); m += kRaWords * 4;
+  r->arr_cell = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
+  r->arr_len = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
+  r->arr_fidx = reinterpret_cast<uint32_t *>(m);
+  r->bmask = cells / kRaBucket - 1;
+  r->rmask = records - 1;
+  r->counts_host = c->h_counts;
+  r->status = c->status;
+  r->status_flag = c->h_flag;
+  return SG_OK;
+}
+
+void ra_launch_reset(sg_hip_ctx *c, const RaArgs &r)
+{
+  const size_t items = (size_t)c->ra_records * SG_MAX_BI_SIZE > c->ra_cells ? (size_t)c->ra_records * SG_MAX_BI_SIZE
+                                                                            : c->ra_cells;
+  k_ra_reset<<<(uint32_t)((items + 255) / 256), 256, 0, c->stream>>>(r, c->ra_cells, c->ra_records);
+}
+
+}  // namespace
+
+int sg_hip_reassemble_reset(sg_hip_ctx *c)
+{
+  if (!c) return SG_E_INVAL;
+  DeviceGuard g(c->device);
+  RaArgs r;
+  bool fresh;
+  int rc = ra_state(c, &r, &fresh);
+  if (rc != SG_OK) return rc;
+  ra_launch_reset(c, r);
+  return finish(c, 0);
+}
+
+int sg_hip_reassemble_evict(sg_hip_ctx *c, uint32_t max_age_calls, uint32_t *n_evicted_out)
+{
+  if (!c) return SG_E_INVAL;
+  if (n_evicted_out) *n_evicted_out = 0;
+  if (!c->ra_mem) return SG_OK;  // nothing has come in yet
+  DeviceGuard g(c->device);
+  RaArgs r;
+  bool fresh;
+  int rc = ra_state(c, &r, &fresh);
+  if (rc != SG_OK) return rc;
+  k_zero_words<<<1, kBlock, 0, c->stream>>>(r.words + kRaEvicted, 1);
+  k_ra_evict<<<(c->ra_cells + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, c->stream>>>(r, c->ra_cells, max_age_calls);
+  rc = finish(c, 0);
+  if (rc != SG_OK) return rc;
+  uint32_t n = 0;
+  HIP_TRY(c, hipMemcpy(&n, r.words + kRaEvicted, sizeof n, hipMemcpyDeviceToHost));
+  if (n_evicted_out) *n_evicted_out = n;
+  return SG_OK;
+}
+
+int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *counts_host_out)
 {
   if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
   int rc = check_ring(c, a->ring, "rx");
   if (rc != SG_OK) return rc;
-  if (n_req_out) *n_req_out = 0;
-  if (n_frags_out) *n_frags_out = 0;
-  if (n_left_out) *n_left_out = 0;
-  if (a->n_arrivals == 0) return SG_OK;
+  if (counts_host_out) memset(counts_host_out, 0, 4 * sizeof(uint32_t));
   if (a->n_arrivals > c->max_frames) return fail(c, SG_E_INVAL, "n_arrivals %u > max_frames %u of this context", a->n_arrivals, c->max_frames);
-  if (!a->arrivals || !a->frag_slot || !a->frag_len || !a->req_first) return fail(c, SG_E_INVAL, "null tables");
+  if ((a->n_arrivals && !a->arrivals) || !a->frag_slot || !a->frag_len || !a->req_first) return fail(c, SG_E_INVAL, "null tables");
   const bool ref64 = a->ring.hdr_profile == SG_HDR_REF64;
   if (ref64 && (!a->len_nic || !a->req_size)) return fail(c, SG_E_INVAL, "REF64 headers need len_nic and the server-wide request size");
   DeviceGuard g(c->device);
 
-  const uint32_t n_max = c->max_frames;
-  if (!c->ra_mem) {
-    uint32_t cells = 2;
-    while (cells < 2 * n_max) cells <<= 1;
-    // keys u64, bytes u64, cnt/last/want u32 per cell;
-    // arr_cell/arr_len/arr_fidx u32 + arr_pack u64 per arrival; blk u64 per workgroup
-    const size_t n_blk = (n_max + kRaBlock - 1) / kRaBlock + 1;
-    const size_t bytes = (size_t)cells * (8 + 8 + 3 * 4) + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 64;
-    HIP_TRY(c, hipMalloc(&c->ra_mem, bytes));
-    HIP_TRY(c, hipMemsetAsync(c->ra_mem, 0, bytes, c->stream));
-    c->ra_cells = cells;
-    HIP_TRY(c, hipHostMalloc((void **)&c->h_counts, 4 * sizeof(uint32_t), hipHostMallocDefault));
-  }
   RaArgs r;
-  memset(&r, 0, sizeof r);
+  bool fresh;
+  rc = ra_state(c, &r, &fresh);
+  if (rc != SG_OK) return rc;
+  if (fresh) ra_launch_reset(c, r);
   r.ring = static_cast<const uint8_t *>(a->ring.base);
   r.n_slots = a->ring.n_slots;
   r.slot_size = a->ring.slot_size;
   r.ref64 = ref64;
   r.n = a->n_arrivals;
+  r.n_dev = a->n_arrivals_dev;
   r.arrivals = a->arrivals;
   r.len_nic = a->len_nic;
   r.req_size = a->req_size;
-  // a table at least twice the arrivals of THIS call keeps probes short and the touched memory small
-  uint32_t cells = 2;
-  while (cells < 2 * a->n_arrivals) cells <<= 1;
-  r.hmask = cells - 1;
   r.max_req = c->max_reqs;
-  const size_t C = c->ra_cells;
-  uint8_t *m = static_cast<uint8_t *>(c->ra_mem);
-  r.keys = reinterpret_cast<unsigned long long *>(m); m += C * 8;
-  r.bytes = reinterpret_cast<unsigned long long *>(m); m += C * 8;
-  r.cnt = reinterpret_cast<uint32_t *>(m); m += C * 4;
-  r.last = reinterpret_cast<uint32_t *>(m); m += C * 4;
-  r.want = reinterpret_cast<uint32_t *>(m); m += C * 4;
-  r.arr_pack = reinterpret_cast<unsigned long long *>(m); m += (size_t)n_max * 8;
-  r.blk = reinterpret_cast<unsigned long long *>(m); m += ((n_max + kRaBlock - 1) / kRaBlock + 1) * 8;
-  r.arr_cell = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
-  r.arr_len = reinterpret_cast<uint32_t *>(m); m += (size_t)n_max * 4;
-  r.arr_fidx = reinterpret_cast<uint32_t *>(m);
+  r.max_frag = c->max_frames;
   r.n_blocks = (a->n_arrivals + kRaBlock - 1) / kRaBlock;
   r.frag_slot = a->frag_slot;
   r.frag_len = a->frag_len;
   r.req_first = a->req_first;
   r.req_token = a->req_token;
-  r.counts = c->h_counts;
-  r.status = c->status;
-  r.status_flag = c->h_flag;
+  r.req_hdr_slot = a->req_hdr_slot;
+  r.counts_out = a->counts_out;
 
   const uint32_t g256 = (a->n_arrivals + 255) / 256;
   rc = prof_begin(c, 5);
   if (rc != SG_OK) return rc;
-  k_ra_insert<<<g256, 256, 0, c->stream>>>(r);
-  k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
-  k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);
-  k_ra_emit<<<g256, 256, 0, c->stream>>>(r);
-  k_ra_wipe<<<g256, 256, 0, c->stream>>>(r);
+  if (a->n_arrivals) {
+    k_ra_insert<<<g256, 256, 0, c->stream>>>(r);
+    k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
+  }
+  k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);  // an empty burst still leaves its counts
+  if (a->n_arrivals) k_ra_emit<<<g256, 256, 0, c->stream>>>(r);
   rc = prof_end(c);
   if (rc != SG_OK) return rc;
-  rc = finish(c, 0);
-  if (rc != SG_OK) return rc;
-  if (n_req_out) *n_req_out = c->h_counts[0];
-  if (n_frags_out) *n_frags_out = c->h_counts[1];
-  // every arrival either belongs to a request that completed or is left out
-  if (n_left_out) *n_left_out = a->n_arrivals - c->h_counts[1];
+  rc = finish(c, a->flags);
+  if (rc != SG_OK || (a->flags & SG_F_ASYNC)) return rc;
+  if (counts_host_out) memcpy(counts_host_out, c->h_counts, 4 * sizeof(uint32_t));
   return SG_OK;
 }
 

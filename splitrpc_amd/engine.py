@@ -137,7 +137,8 @@ class SgContext:
     def gather_args(ring: RingRef, frag_slot: torch.Tensor, frag_len: Optional[torch.Tensor],
                     req_first: torch.Tensor, n_req: int, n_frags: int, app: AppRef,
                     offsets_out: Optional[torch.Tensor] = None, flags: int = 0,
-                    fixed_req_size: int = 0, mtu: int = 0) -> capi.GatherArgs:
+                    fixed_req_size: int = 0, mtu: int = 0, counts: Optional[torch.Tensor] = None,
+                    slot_state: Optional[torch.Tensor] = None) -> capi.GatherArgs:
         a = capi.GatherArgs()
         a.ring = ring.desc()
         a.frag_slot = frag_slot.data_ptr()
@@ -150,6 +151,10 @@ class SgContext:
         a.flags = flags
         a.fixed_req_size = int(fixed_req_size)
         a.mtu = int(mtu)
+        a.counts = counts.data_ptr() if counts is not None else None
+        if slot_state is not None:
+            a.slot_state = slot_state.data_ptr()
+            a.n_slot_states = int(slot_state.numel())
         return a
 
     def gather_batch(self, *args, **kw) -> None:
@@ -169,12 +174,14 @@ class SgContext:
                      n_frames: int, mtu: int, app: AppRef,
                      offsets_out: Optional[torch.Tensor] = None, flags: int = 0,
                      hdr_templates: Optional[torch.Tensor] = None,
-                     req_token: Optional[torch.Tensor] = None) -> capi.ScatterArgs:
+                     req_token: Optional[torch.Tensor] = None, hdr_src_req: Optional[torch.Tensor] = None,
+                     counts: Optional[torch.Tensor] = None,
+                     slot_state: Optional[torch.Tensor] = None) -> capi.ScatterArgs:
         a = capi.ScatterArgs()
         a.rx = rx.desc()
         a.tx = tx.desc()
         a.tx_slot = tx_slot.data_ptr()
-        a.hdr_src_slot = hdr_src_slot.data_ptr()
+        a.hdr_src_slot = hdr_src_slot.data_ptr() if hdr_src_slot is not None else None
         a.resp_first = resp_first.data_ptr()
         a.resp_size = resp_size.data_ptr() if resp_size is not None else None
         a.fixed_resp_size = int(fixed_resp_size)
@@ -186,6 +193,11 @@ class SgContext:
         a.offsets_out = offsets_out.data_ptr() if offsets_out is not None else None
         a.hdr_templates = hdr_templates.data_ptr() if hdr_templates is not None else None
         a.req_token = req_token.data_ptr() if req_token is not None else None
+        a.hdr_src_req = hdr_src_req.data_ptr() if hdr_src_req is not None else None
+        a.counts = counts.data_ptr() if counts is not None else None
+        if slot_state is not None:
+            a.slot_state = slot_state.data_ptr()
+            a.n_slot_states = int(slot_state.numel())
         return a
 
     def scatter_batch(self, *args, **kw) -> None:
@@ -198,26 +210,61 @@ class SgContext:
         if rc != capi.SG_OK:
             self._check(rc)
 
-    def reassemble(self, ring: RingRef, arrivals: torch.Tensor, n_arrivals: int, frag_slot: torch.Tensor,
-                   frag_len: torch.Tensor, req_first: torch.Tensor, req_token: Optional[torch.Tensor] = None,
-                   len_nic: Optional[torch.Tensor] = None, req_size: int = 0):
-        """Sort a burst of arrivals into requests on the device; returns
-        (requests, fragments, arrivals left out)."""
+    @staticmethod
+    def reassemble_args(ring: RingRef, arrivals: torch.Tensor, n_arrivals: int, frag_slot: torch.Tensor,
+                        frag_len: torch.Tensor, req_first: torch.Tensor, req_token: Optional[torch.Tensor] = None,
+                        len_nic: Optional[torch.Tensor] = None, req_size: int = 0,
+                        req_hdr_slot: Optional[torch.Tensor] = None, counts_out: Optional[torch.Tensor] = None,
+                        n_arrivals_dev: Optional[torch.Tensor] = None, flags: int = 0) -> capi.ReassembleArgs:
         a = capi.ReassembleArgs()
         a.ring = ring.desc()
         a.arrivals = arrivals.data_ptr()
         a.len_nic = len_nic.data_ptr() if len_nic is not None else None
         a.n_arrivals = n_arrivals
+        a.flags = flags
         a.req_size = int(req_size)
         a.frag_slot = frag_slot.data_ptr()
         a.frag_len = frag_len.data_ptr()
         a.req_first = req_first.data_ptr()
         a.req_token = req_token.data_ptr() if req_token is not None else None
-        n_req, n_frag, n_left = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
-        self._after_torch()
-        self._check(self.lib.sg_hip_reassemble(self.h, C.byref(a), C.byref(n_req), C.byref(n_frag),
-                                               C.byref(n_left)))
-        return int(n_req.value), int(n_frag.value), int(n_left.value)
+        a.req_hdr_slot = req_hdr_slot.data_ptr() if req_hdr_slot is not None else None
+        a.counts_out = counts_out.data_ptr() if counts_out is not None else None
+        a.n_arrivals_dev = n_arrivals_dev.data_ptr() if n_arrivals_dev is not None else None
+        return a
+
+    def reassemble_raw(self, a: capi.ReassembleArgs):
+        """Returns (requests completed, their fragments, arrivals dropped,
+        requests still in flight); all zero for an SG_F_ASYNC call."""
+        counts = (C.c_uint32 * 4)()
+        if not (a.flags & capi.F_ASYNC):
+            self._after_torch()
+        rc = self.lib.sg_hip_reassemble(self.h, C.byref(a), C.byref(counts))
+        if rc != capi.SG_OK:
+            self._check(rc)
+        return tuple(int(x) for x in counts)
+
+    def reassemble(self, *args, **kw):
+        """Sort a burst of arrivals into requests on the device; incomplete
+        requests stay on the device for later calls.  Returns (requests
+        completed, their fragments, requests still in flight)."""
+        n_req, n_frag, self.last_dropped, in_flight = self.reassemble_raw(self.reassemble_args(*args, **kw))
+        return n_req, n_frag, in_flight
+
+    def reassemble_reset(self) -> None:
+        self._check(self.lib.sg_hip_reassemble_reset(self.h))
+
+    def reassemble_evict(self, max_age_calls: int) -> int:
+        n = C.c_uint32(0)
+        self._check(self.lib.sg_hip_reassemble_evict(self.h, max_age_calls, C.byref(n)))
+        return int(n.value)
+
+    def set_slot_index(self, which: int, value: int) -> None:
+        self._check(self.lib.sg_hip_set_slot_index(self.h, which, value))
+
+    def get_slot_index(self, which: int) -> int:
+        v = C.c_uint32(0)
+        self._check(self.lib.sg_hip_get_slot_index(self.h, which, C.byref(v)))
+        return int(v.value)
 
     # -- per request ---------------------------------------------------------
     def copy_runs(self, src: Sequence[int], dst: Sequence[int], lens: Sequence[int],

@@ -1,0 +1,302 @@
+"""The receive -> gather -> scatter pipeline with its bookkeeping on the device:
+requests that straddle bursts (the reference's rr_cache across rr_recv_ng
+bursts, src/transport/dpdk_transport_ng.h:176-218), counts that never visit
+the host, application slot states published by the device
+(src/splitrpc_server/p2p_rpc_dpdk_server.cc:130,175), and the whole step
+recorded into one HIP graph."""
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from splitrpc_amd import capi, synth
+from splitrpc_amd.engine import AppRef, DeviceWorkload, RingRef, SgContext, SgError, to_dev
+
+from helpers import first_diff
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FREE, RX, WORK = capi.SLOT_FREE, capi.SLOT_RX_COMPLETE, capi.SLOT_WORK_COMPLETE
+
+
+class Tables:
+    """Output tables of the device reassembly, sized for the context."""
+
+    def __init__(self, max_reqs, max_frames):
+        self.fs = torch.zeros(max_frames, dtype=torch.int32, device=DEV)
+        self.fl = torch.zeros(max_frames, dtype=torch.int32, device=DEV)
+        self.rf = torch.zeros(max_reqs + 1, dtype=torch.int32, device=DEV)
+        self.tok = torch.zeros(max_reqs, dtype=torch.int64, device=DEV)
+        self.hdr = torch.zeros(max_reqs, dtype=torch.int32, device=DEV)
+        self.counts = torch.zeros(4, dtype=torch.int32, device=DEV)
+
+    def take(self, n_req, n_frag):
+        u32 = lambda t: t.cpu().numpy().view(np.uint32)
+        return (u32(self.fs[:n_frag]), u32(self.fl[:n_frag]), u32(self.rf[:n_req + 1]),
+                self.tok[:n_req].cpu().numpy().view(np.uint64), u32(self.hdr[:n_req]))
+
+
+def _feed_in_bursts(ctx, w, order, burst, tabs, len_nic=None, req_size=0):
+    rx = RingRef(torch.from_numpy(w.ring).to(DEV), w.n_slots, w.slot_size, w.profile)
+    arr = to_dev(np.ascontiguousarray(order, np.uint32), DEV)
+    ln = to_dev(len_nic, DEV) if len_nic is not None else None
+    fs, fl, first, tok, hdr = [], [], [0], [], []
+    peak = 0
+    for b in range(0, len(order), burst):
+        n = min(burst, len(order) - b)
+        n_req, n_frag, in_flight = ctx.reassemble(rx, arr[b:b + n], n, tabs.fs, tabs.fl, tabs.rf, tabs.tok,
+                                                  ln, req_size, req_hdr_slot=tabs.hdr, counts_out=tabs.counts)
+        assert tabs.counts.cpu().tolist() == [n_req, n_frag, ctx.last_dropped, in_flight]
+        peak = max(peak, in_flight)
+        s, l, f, t, h = tabs.take(n_req, n_frag)
+        assert f[0] == 0 and f[-1] == n_frag
+        fs.append(s), fl.append(l), tok.append(t), hdr.append(h)
+        first.extend(int(x) + first[-1] for x in np.diff(f.astype(np.int64)))
+    assert in_flight == 0
+    return np.concatenate(fs), np.concatenate(fl), np.array(first, np.uint32), np.concatenate(tok), \
+        np.concatenate(hdr), peak
+
+
+@pytest.mark.parametrize("order_kind", ["as generated", "shuffled across requests"])
+def test_resnet_sized_requests_arrive_in_bursts_of_64(order_kind):
+    """Config 2 at full size, 64 arrivals per call as a NIC burst brings them:
+    every 431-fragment request straddles many calls; the calls' outputs laid end
+    to end are what the oracle makes of the whole stream."""
+    w = synth.make_workload(2)
+    order = w.arrivals if order_kind == "as generated" else np.random.default_rng(3).permutation(w.arrivals)
+    print(f"case bursts cfg=2 arrivals={len(order)} order={order_kind}", flush=True)
+    ctx = SgContext(0, max_reqs=64, max_frames=8192)
+    ctx.reassemble_reset()
+    tabs = Tables(64, 8192)
+    fs, fl, first, tok, hdr, peak = _feed_in_bursts(ctx, w, order, 64, tabs)
+    efs, efl, erf, etok = oracle.reassemble(w, arrivals=order)
+    assert np.array_equal(tok, etok)
+    assert np.array_equal(first, erf)
+    assert np.array_equal(fs, efs)
+    assert np.array_equal(fl, efl)
+    assert np.array_equal(hdr, efs[erf[:-1]])
+    assert peak >= (1 if order_kind == "as generated" else w.n_req)
+    ctx.close()
+
+
+def test_bursts_with_the_reference_header_and_nic_lengths():
+    """REF64: a request is complete when its bytes add up to the server-wide
+    size; the running total is carried from call to call."""
+    w = synth.make_workload(1, 20, profile=synth.HDR_REF64)
+    len_nic = np.zeros(w.n_slots, np.uint32)
+    len_nic[w.frag_slot] = w.frag_len
+    order = np.random.default_rng(8).permutation(w.arrivals)
+    ctx = SgContext(0, max_reqs=32, max_frames=256)
+    tabs = Tables(32, 256)
+    size = int(w.req_sizes[0])
+    fs, fl, first, tok, hdr, peak = _feed_in_bursts(ctx, w, order, 7, tabs, len_nic=len_nic, req_size=size)
+    efs, efl, erf, etok = oracle.reassemble(w, arrivals=order, req_size=size, frag_len_nic=len_nic)
+    assert np.array_equal(tok, etok) and np.array_equal(first, erf)
+    assert np.array_equal(fs, efs) and np.array_equal(fl, efl)
+    assert peak > 3
+    ctx.close()
+
+
+def test_pool_exhaustion_eviction_and_reset():
+    """More requests in flight than the pool has records: refused, the rest
+    goes on.  Eviction clears out what has been idle; afterwards the table is
+    as good as new."""
+    w = synth.make_custom([4200] * 9, [64] * 9, seed=41)
+    ctx = SgContext(0, max_reqs=4, max_frames=64)
+    tabs = Tables(4, 64)
+    rx = RingRef(torch.from_numpy(w.ring).to(DEV), w.n_slots, w.slot_size, w.profile)
+    firsts = np.ascontiguousarray(w.frag_slot[w.req_first[:6]], np.uint32)  # fragment 0 of six requests
+    with pytest.raises(SgError) as e:
+        ctx.reassemble(rx, to_dev(firsts, DEV), 6, tabs.fs, tabs.fl, tabs.rf, tabs.tok)
+    assert e.value.code == capi.SG_E_DATA and "in flight" in str(e.value)
+    # nothing idle yet at age 5; everything parked goes at age 0
+    assert ctx.reassemble_evict(5) == 0
+    assert ctx.reassemble_evict(0) == 6
+    n_req, n_frag, in_flight = ctx.reassemble(rx, to_dev(w.arrivals[:1], DEV), 0, tabs.fs, tabs.fl, tabs.rf, tabs.tok)
+    assert (n_req, n_frag, in_flight) == (0, 0, 0)
+    # four requests at a time fit
+    for lo in (0, 4):
+        sel = np.concatenate([w.frag_slot[w.req_first[r]:w.req_first[r + 1]] for r in range(lo, min(lo + 4, 9))])
+        n_req, n_frag, in_flight = ctx.reassemble(rx, to_dev(sel.astype(np.uint32), DEV), len(sel), tabs.fs, tabs.fl,
+                                                  tabs.rf, tabs.tok)
+        assert (n_req, n_frag, in_flight) == (4, 12, 0)
+        assert np.array_equal(tabs.take(n_req, n_frag)[0], sel)
+    # a parked request, then a reset
+    ctx.reassemble(rx, to_dev(firsts[:2], DEV), 2, tabs.fs, tabs.fl, tabs.rf, tabs.tok)
+    ctx.reassemble_reset()
+    n_req, n_frag, in_flight = ctx.reassemble(rx, to_dev(firsts[:1], DEV), 0, tabs.fs, tabs.fl, tabs.rf, tabs.tok)
+    assert in_flight == 0
+    ctx.close()
+
+
+def _sub(w, fs, fl, rf, resp_rows, tx_slots, hdr_slots, resp_size):
+    """A workload holding just the requests of one call, for the oracle."""
+    n = len(rf) - 1
+    per = synth.num_frames(resp_size, w.mtu)
+    return dataclasses.replace(
+        w, frag_slot=fs, frag_len=fl, req_first=rf.astype(np.uint32),
+        req_sizes=np.full(n, int(w.req_sizes[0]), np.uint64), resp_sizes=np.full(n, resp_size, np.uint64),
+        resp_first=(np.arange(n + 1) * per).astype(np.uint32), tx_slot=tx_slots[:n * per].astype(np.uint32),
+        hdr_src_slot=np.repeat(hdr_slots, per).astype(np.uint32), resp_payload=resp_rows, req_ids=np.zeros(n, np.uint64))
+
+
+def test_slot_states_published_by_the_device():
+    """gather: FREE -> RX_COMPLETE for the slots it filled; scatter: WORK_COMPLETE
+    -> FREE; both indices advance on the device and wrap; a slot in the wrong
+    state is reported."""
+    w = synth.make_custom([4200] * 5, [3000] * 5, seed=51, flags=synth.F_UDP_CSUM_PSEUDO)
+    dw = DeviceWorkload(w)
+    ctx = SgContext(0)
+    n_states = 7
+    states = torch.zeros(n_states, dtype=torch.int32, device=DEV)
+    ctx.set_slot_index(0, 5)
+    ctx.set_slot_index(1, 5)
+    for mode in ("rule", "scan"):
+        ga = ctx.gather_args(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app, dw.req_offsets,
+                             flags=capi.F_RULE_FRAGS if mode == "rule" else 0,
+                             fixed_req_size=4200 if mode == "rule" else 0, mtu=w.mtu, slot_state=states)
+        pi = ctx.get_slot_index(0)
+        ctx.gather_batch_raw(ga)
+        want = np.zeros(n_states, np.int32)
+        want[(pi + np.arange(5)) % n_states] = RX
+        assert np.array_equal(states.cpu().numpy(), want), mode
+        assert ctx.get_slot_index(0) == (pi + 5) % n_states
+        # the TX side finds them not yet worked on: reported, and (as documented) freed all the same
+        sa = ctx.scatter_args(dw.rx, dw.tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first,
+                              None if mode == "rule" else dw.resp_size, 3000 if mode == "rule" else 0, dw.n_req,
+                              dw.n_frames, w.mtu, dw.resp_app, dw.resp_offsets, w.flags, slot_state=states)
+        if mode == "rule":
+            with pytest.raises(SgError) as e:
+                ctx.scatter_batch_raw(sa)
+            assert e.value.code == capi.SG_E_DATA and "slot" in str(e.value)
+            assert not states.cpu().numpy().any()
+            ctx.set_slot_index(1, pi)
+            states.copy_(torch.from_numpy(want))
+        states[states == RX] = WORK  # the worker
+        ctx.scatter_batch_raw(sa)
+        assert not states.cpu().numpy().any(), mode
+        assert ctx.get_slot_index(1) == (pi + 5) % n_states
+    # a refused descriptor-pass batch publishes nothing and advances nothing
+    bad = w.frag_slot.copy()
+    bad[2] = w.n_slots + 1
+    bad_dev = to_dev(bad, DEV)
+    ga = ctx.gather_args(dw.rx, bad_dev, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app, dw.req_offsets,
+                         slot_state=states)
+    pi = ctx.get_slot_index(0)
+    with pytest.raises(SgError):
+        ctx.gather_batch_raw(ga)
+    assert not states.cpu().numpy().any()
+    assert ctx.get_slot_index(0) == pi
+    # more requests than the ring has slots: refused by the host
+    small = torch.zeros(3, dtype=torch.int32, device=DEV)
+    ga = ctx.gather_args(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app, slot_state=small)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch_raw(ga)
+    assert e.value.code == capi.SG_E_INVAL
+    ctx.close()
+
+
+@pytest.mark.parametrize("use_graph", [False, True], ids=["eager", "one-graph"])
+def test_bursts_through_reassembly_gather_and_scatter_without_the_host(use_graph):
+    """One step = reassemble + gather + scatter, three calls, none of which
+    waits for the host: the counts go from call to call in device memory.  With
+    use_graph the three calls (an odd number per arena) are recorded ONCE and
+    replayed for every burst; the burst's arrivals and their number are written
+    into device buffers between replays.  Every step is held against the oracle:
+    request arena, TX ring, bump-ring cursors, slot indices and slot states."""
+    n_reqs, burst, resp_size, n_states = 24, 16, 3000, 17
+    w = synth.make_custom([4200] * n_reqs, [resp_size] * n_reqs, seed=61,
+                          flags=synth.F_UDP_CSUM_PSEUDO | synth.F_IPV4_CSUM)
+    order = np.random.default_rng(4).permutation(w.arrivals)
+    efs, efl, erf, etok = oracle.reassemble(w, arrivals=order)
+    slot_req = {int(s): r for r in range(n_reqs) for s in efs[erf[r]:erf[r + 1]]}
+    per_req, per_resp = 3, synth.num_frames(resp_size, w.mtu)
+    s = torch.cuda.Stream()
+    ctx = SgContext(0, max_reqs=64, max_frames=4096, stream=s.cuda_stream)
+    ctx.reassemble_reset()
+    tabs = Tables(64, 4096)
+    rx_ring = torch.from_numpy(w.ring).to(DEV)
+    rx = RingRef(rx_ring, w.n_slots, w.slot_size, w.profile)
+    tx_slots = np.random.default_rng(5).permutation(burst * per_resp).astype(np.uint32)
+    tx_init = np.random.default_rng(6).integers(0, 256, burst * per_resp * w.slot_size, dtype=np.uint8)
+    tx_ring = torch.from_numpy(tx_init).to(DEV)
+    tx = RingRef(tx_ring, burst * per_resp, w.slot_size, w.profile)
+    req_cap, resp_cap = 17 * 4200 + 100, 7 * resp_size + 50  # the request arena holds a whole burst's worth
+    req_arena = torch.zeros(req_cap, dtype=torch.uint8, device=DEV)
+    resp_np = np.random.default_rng(7).integers(0, 256, resp_cap, dtype=np.uint8)
+    resp_arena = torch.from_numpy(resp_np).to(DEV)
+    states = torch.zeros(n_states, dtype=torch.int32, device=DEV)
+    arr_buf = torch.zeros(burst, dtype=torch.int32, device=DEV)
+    n_arr = torch.zeros(1, dtype=torch.int32, device=DEV)
+    tx_slot_dev = to_dev(tx_slots, DEV)
+    resp_first = to_dev((np.arange(burst + 1) * per_resp).astype(np.uint32), DEV)
+
+    A = capi.F_ASYNC
+    ra = ctx.reassemble_args(rx, arr_buf, burst, tabs.fs, tabs.fl, tabs.rf, tabs.tok, req_hdr_slot=tabs.hdr,
+                             counts_out=tabs.counts, n_arrivals_dev=n_arr, flags=A)
+    ga = ctx.gather_args(rx, tabs.fs, None, tabs.rf, burst, burst * per_req, AppRef(arena=req_arena, cap=req_cap),
+                         None, flags=A | capi.F_RULE_FRAGS, fixed_req_size=4200, mtu=w.mtu, counts=tabs.counts,
+                         slot_state=states)
+    sa = ctx.scatter_args(rx, tx, tx_slot_dev, None, resp_first, None, resp_size, burst, burst * per_resp, w.mtu,
+                          AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A, hdr_src_req=tabs.hdr,
+                          counts=tabs.counts, slot_state=states)
+
+    def step():
+        ctx.reassemble_raw(ra)
+        ctx.gather_batch_raw(ga)
+        with torch.cuda.stream(s):
+            states.copy_(torch.where(states == RX, torch.full_like(states, WORK), states))  # the worker
+        ctx.scatter_batch_raw(sa)
+
+    ctx.set_cursor(0, req_cap - 5000)
+    ctx.set_cursor(1, 0)
+    ctx.set_slot_index(0, n_states - 3)
+    ctx.set_slot_index(1, n_states - 3)
+    torch.cuda.synchronize()
+    g = None
+    if use_graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            step()
+    want_req = np.zeros(req_cap, np.uint8)
+    want_tx = tx_init.copy()
+    cur0, cur1, done, idx = req_cap - 5000, 0, 0, n_states - 3
+    pos_done = np.zeros(n_reqs, int)  # fragments seen per request (in completion-order numbering)
+    for b in range(0, len(order), burst):
+        part = order[b:b + burst]
+        arr_buf[:len(part)] = to_dev(np.ascontiguousarray(part, np.uint32), DEV)
+        n_arr.fill_(len(part))
+        torch.cuda.synchronize()
+        if use_graph:
+            g.replay()
+        else:
+            step()
+        torch.cuda.synchronize()
+        ctx.sync()
+        for sl in part:
+            pos_done[slot_req[int(sl)]] += 1
+        now = int((pos_done == per_req).sum())
+        r0, r1 = done, now
+        counts = tabs.counts.cpu().tolist()
+        assert counts[:2] == [r1 - r0, (r1 - r0) * per_req], f"burst at {b}: {counts}"
+        assert counts[3] == int(((pos_done > 0) & (pos_done < per_req)).sum())
+        if r1 > r0:
+            fs = efs[erf[r0]:erf[r1]]
+            sub = _sub(w, fs, efl[erf[r0]:erf[r1]], erf[r0:r1 + 1] - erf[r0], None, tx_slots, efs[erf[r0:r1]],
+                       resp_size)
+            want_req, _, cur0 = oracle.gather(sub, arena_cap=req_cap, cursor=cur0, out=want_req)
+            sub.tx_n_slots = burst * per_resp
+            _, cur1 = oracle.scatter(sub, w.ring, want_tx, resp_np, arena_cap=resp_cap, cursor=cur1)
+        done = now
+        idx = (idx + (r1 - r0)) % n_states
+        got = req_arena.cpu().numpy()
+        assert np.array_equal(got, want_req), f"burst at {b}: " + first_diff(got, want_req)
+        got = tx_ring.cpu().numpy()
+        assert np.array_equal(got, want_tx), f"burst at {b}: " + first_diff(got, want_tx)
+        assert ctx.get_cursor(0) == cur0 and ctx.get_cursor(1) == cur1
+        assert ctx.get_slot_index(0) == idx and ctx.get_slot_index(1) == idx
+        assert not states.cpu().numpy().any()
+    assert done == n_reqs
+    ctx.close()

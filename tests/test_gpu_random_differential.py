@@ -83,6 +83,13 @@ def test_random_workload(ctx, seed):
         per = (w.req_first[1:] - w.req_first[:-1]).astype(np.int64)
         live = per > 0
         assert got == (int(live.sum()), w.n_frags, 0)
+        # the oracle's replay of the receive path on the same arrivals
+        efs, efl, erf, etok = oracle.reassemble(w, req_size=int(w.req_sizes[0]) if ref64 else 0,
+                                                frag_len_nic=ln if (ref64 or seed % 2) else None)
+        assert np.array_equal(fs.cpu().numpy().view(np.uint32), efs)
+        assert np.array_equal(fl.cpu().numpy().view(np.uint32), efl)
+        assert np.array_equal(rf.cpu().numpy().view(np.uint32)[:len(erf)], erf)
+        assert np.array_equal(tok.cpu().numpy().view(np.uint64)[:len(etok)], etok)
         assert np.array_equal(fs.cpu().numpy().view(np.uint32), w.frag_slot.astype(np.uint32))
         assert np.array_equal(fl.cpu().numpy().view(np.uint32), w.frag_len.astype(np.uint32))
         want_first = np.concatenate([[0], np.cumsum(per[live])]).astype(np.uint32)

@@ -13,11 +13,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def device_reassemble(ctx, w, arrivals, len_nic=None, req_size=0, ring=None, max_reqs=8192):
+def device_reassemble(ctx, w, arrivals, len_nic=None, req_size=0, ring=None, max_reqs=8192, reset=True):
     n = len(arrivals)
+    if reset:
+        ctx.reassemble_reset()  # the context is shared: nothing of an earlier case may still be in flight
     rx = RingRef(torch.from_numpy(w.ring if ring is None else ring).to(DEV), w.n_slots, w.slot_size, w.profile)
-    fs = torch.zeros(max(n, 1), dtype=torch.int32, device=DEV)
-    fl = torch.zeros(max(n, 1), dtype=torch.int32, device=DEV)
+    # room for the fragments that earlier calls left in flight as well
+    fs = torch.zeros(n + 4096, dtype=torch.int32, device=DEV)
+    fl = torch.zeros(n + 4096, dtype=torch.int32, device=DEV)
     rf = torch.zeros(max_reqs + 1, dtype=torch.int32, device=DEV)
     tok = torch.zeros(max_reqs, dtype=torch.int64, device=DEV)
     ln = to_dev(len_nic, DEV) if len_nic is not None else None
@@ -53,8 +56,8 @@ def test_reassembly_ref64_by_request_size(ctx):
 
 
 def test_lost_fragments_and_token_zero(ctx):
-    """A lost fragment parks its request; token 0 is dropped; the rest goes
-    through, and the table is clean for the next call."""
+    """A lost fragment parks its request until the fragment comes; token 0 is
+    dropped; the rest goes through."""
     w = synth.make_workload(1, 10)
     ring = w.ring.copy().reshape(w.n_slots, w.slot_size)
     zero_slot = int(w.frag_slot[int(w.req_first[3])])       # a fragment of request 3 loses its token
@@ -67,8 +70,14 @@ def test_lost_fragments_and_token_zero(ctx):
     for g, e in zip(got[:4], want):
         assert np.array_equal(g, e)
     assert len(got[3]) == 8
-    assert got[4] == 3 + 2  # request 3: token-0 packet + its two orphans; request 6: two fragments waiting
-    # a second, clean burst right after
+    assert got[4] == 2            # requests 3 and 6 stay in flight, each one fragment short
+    assert ctx.last_dropped == 1  # the token-0 packet
+    # the missing fragment of request 6 comes with the next burst: the request completes there
+    late = np.array([w.frag_slot[int(w.req_first[6]) + 1]], np.uint32)
+    got = device_reassemble(ctx, w2, late, ring=w2.ring, reset=False)
+    assert len(got[3]) == 1 and got[3][0] == w.req_ids[6] and got[4] == 1
+    assert np.array_equal(got[0], w.frag_slot[int(w.req_first[6]):int(w.req_first[7])])
+    # a clean burst after a reset
     got = device_reassemble(ctx, w, w.arrivals)
     want = oracle.reassemble(w)
     for g, e in zip(got[:4], want):
@@ -120,6 +129,7 @@ def test_client_requests_served_on_the_device_end_to_end(ctx, kind):
     fs = torch.zeros(w.n_frags, dtype=torch.int32, device=dev)
     fl = torch.zeros(w.n_frags, dtype=torch.int32, device=dev)
     rf = torch.zeros(8193, dtype=torch.int32, device=dev)
+    ctx.reassemble_reset()
     n_req, n_frag, n_left = ctx.reassemble(dw.rx, dw.arrivals, w.n_frags, fs, fl, rf, len_nic=to_dev(ln, dev),
                                            req_size=size)
     assert (n_req, n_frag, n_left) == (w.n_req, w.n_frags, 0)
