@@ -6,6 +6,13 @@
  * GPU the context was created on (hipMalloc, VMM mapping, or pinned host
  * memory); the library never allocates or frees payload memory.
  *
+ * Reads around a run.  The copy kernels load 16-byte chunks at 16-byte aligned
+ * addresses whatever the address of a run (a fragment's payload, a piece of a
+ * tensor): up to 15 bytes before the first and after the last byte of a run are
+ * read, and discarded, when they share such a chunk with bytes of the run.  A
+ * chunk never spans a page, so whatever memory holds the run holds every byte
+ * that is read; nothing outside a run is ever written.
+ *
  * Return convention: 0 on success, a negative SG_E_* code on failure (the
  * reference's sg_on_gpu returns 1/0, src/transport/g_copy_ng.cu:169-223; the
  * C++ engine above this ABI keeps that convention for its callers).

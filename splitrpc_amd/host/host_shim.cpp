@@ -8,6 +8,7 @@
 #include <thread>
 #include <vector>
 
+#include "sg_app_ctx.h"
 #include "sg_app_rr.h"
 #include "sg_engine.h"
 #include "sg_rr.h"
@@ -194,10 +195,14 @@ int sgh_ring_stress(uint32_t n_threads, uint32_t per_thread, uint32_t capacity)
 // 117-189) on one GPU: file the arrivals under their requests, take a slot of
 // the application ring per ready request, gather, and -- for the responses the
 // caller describes -- set up the response buffers, rewrite their headers and
-// scatter.  per_request != 0 uses the reference's one-request calls, else the
-// batched gather.  The request arena (n_done * req_size bytes) and the TX ring
-// are copied back for inspection.  Fixed-size requests (req_size) as in the
-// reference.  Returns completed requests or a negative error.
+// scatter.  per_request == 1 uses the reference's one-request calls; 0 the
+// batched gather with per-request TX; 2 the batched gather and the batched TX
+// (headers from the connections' templates, written by the scatter kernel),
+// with the application slots' state words published by the device and walked
+// by the worker's batching window on the host.  The request arena
+// (n_done * req_size bytes) and the TX ring are copied back for inspection.
+// Fixed-size requests (req_size) as in the reference.  Returns completed
+// requests or a negative error.
 int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots, uint32_t slot_size,
                       uint32_t profile, const uint32_t *arrivals, uint32_t n_arr, const uint32_t *len_nic,
                       uint64_t req_size, uint64_t resp_size, uint32_t mtu, uint32_t flags, int per_request,
@@ -254,23 +259,64 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
       app.arena = app_pool.rr_mem_pool->get_req_addr_range();
       app.arena_cap = app_pool.rr_mem_pool->get_req_addr_pool_size();
       app.arena_mirrored = app_pool.rr_mem_pool->mirrored();
+      uint32_t *states = per_request == 2 ? (uint32_t *)app_pool.rr_mem_pool->get_doorbells_device() : nullptr;
       if (engine.gather_batch(ready.data(), (uint32_t)ready.size(), view, app, nullptr, req_size,
-                              len_nic ? 0 : mtu, 0) != SG_OK)
+                              len_nic ? 0 : mtu, 0, states, states ? (uint32_t)n_app : 0) != SG_OK)
         return -11;
-      for (auto *s : slots) *s->h_state = RX_COMPLETE;
+      if (states) {
+        // RX_COMPLETE was published by the device, behind the copy
+        for (auto *s : slots)
+          if (*s->h_state != RX_COMPLETE) return -14;
+      } else {
+        for (auto *s : slots) *s->h_state = RX_COMPLETE;
+      }
     }
     for (size_t k = 0; k < ready.size(); k++)
       (void)hipMemcpy(req_out + k * req_size, slots[k]->h_stub->req, req_size, hipMemcpyDeviceToHost);
 
     // ---- the model: responses land in the slots' resp buffers ----
-    for (size_t k = 0; k < ready.size(); k++) {
+    for (size_t k = 0; k < ready.size(); k++)
       (void)hipMemcpy(slots[k]->h_stub->resp, resp_host + k * resp_size, resp_size, hipMemcpyHostToDevice);
-      *slots[k]->h_state = WORK_COMPLETE;
+    if (per_request == 2) {
+      // the worker's window over the very words the device wrote
+      SgBatchWindow win;
+      if (win.collect(&app_pool, (int)ready.size()) != (int)ready.size()) return -15;
+      win.complete(&app_pool);
+    } else {
+      for (size_t k = 0; k < ready.size(); k++) *slots[k]->h_state = WORK_COMPLETE;
     }
 
     // ---- TX half: response buffers, headers, scatter ----
     const uint32_t per = (uint32_t)((resp_size + mtu - 1) / mtu);
-    for (size_t k = 0; k < ready.size(); k++) {
+    if (per_request == 2) {
+      for (size_t k = 0; k < ready.size(); k++) {
+        // rr_alloc_mbufs: fresh response buffers take the place of the request's
+        P2pRpcRr *r = ready[k];
+        r->transport_mbufs->num_items = r->hdr_bufs->num_items = r->payload_bufs->num_items = 0;
+        r->payload_size = 0;
+        size_t rem = resp_size;
+        for (uint32_t i = 0; i < per; i++) {
+          uint8_t *slot = d_tx + (size_t)tx_slot[(uint32_t)k * per + i] * slot_size;
+          const size_t cur = rem <= mtu ? rem : mtu;
+          rem -= cur;
+          r->rr_append_mbuf((uintptr_t)slot, (uintptr_t)slot, (uintptr_t)(slot + hl), cur);
+        }
+      }
+      SgRingView txv{sg_ring_desc{d_tx, tx_n_slots, slot_size, profile, 0}};
+      sg_app_desc rapp;
+      std::memset(&rapp, 0, sizeof rapp);
+      rapp.arena = app_pool.rr_mem_pool->get_resp_addr_range();
+      rapp.arena_cap = app_pool.rr_mem_pool->get_resp_addr_pool_size();
+      rapp.arena_mirrored = app_pool.rr_mem_pool->mirrored();
+      uint32_t *states = (uint32_t *)app_pool.rr_mem_pool->get_doorbells_device();
+      if (!ready.empty() &&
+          engine.scatter_batch(ready.data(), (uint32_t)ready.size(), txv, rapp, mtu, flags, states, (uint32_t)n_app) != SG_OK)
+        return -16;
+      for (auto *s : slots)
+        if (*s->h_state != FREE) return -17;  // freed by the device, behind the copy
+      for (auto *r : ready) pool.reap_rr(r);
+    }
+    for (size_t k = 0; per_request != 2 && k < ready.size(); k++) {
       P2pRpcRr *r = ready[k];
       r->transport_mbufs->num_items = r->hdr_bufs->num_items = r->payload_bufs->num_items = 0;
       r->payload_size = 0;
@@ -331,6 +377,61 @@ int64_t sgh_window_replay(int device_id, int pool_size, const int32_t *ops, uint
     }
   }
   return n_win;
+}
+
+// P2pRpcSgZcEngine (src/p2p_rpc_sg_engine.h:109-134): gather hands out the
+// first payload pointer as request and response buffer, scatter does nothing.
+// Returns 1 when it behaves so.
+int sgh_zc_engine(uint64_t payload_ptr)
+{
+  P2pRpcSgEngine *e = new P2pRpcSgZcEngine();
+  P2pRpcRr rr;
+  rr.rr_append_mbuf(payload_ptr - 64, payload_ptr - 64, payload_ptr, 1024);
+  g_params stub{nullptr, nullptr};
+  e->gather(&rr, &stub);
+  const bool ok = (uint64_t)(uintptr_t)stub.req == payload_ptr && (uint64_t)(uintptr_t)stub.resp == payload_ptr;
+  g_params before = stub;
+  e->scatter(&rr, &stub);
+  e->gather(&rr, (uint8_t *)nullptr);
+  e->scatter(&rr, (uint8_t *)nullptr);
+  const bool same = stub.req == before.req && stub.resp == before.resp && e->num_instances == 1;
+  delete e;
+  return ok && same ? 1 : 0;
+}
+
+// The reference's copy context and its C entry points (CopyCtx,
+// sg_on_gpu_entry, sg_on_gpu; src/transport/g_copy_ng.cuh:21-37) moving one
+// run on the device, its doorbell in a BufItemPool object
+// (src/p2p_buf_pool.h:12-78).  Returns a bit per step that went as it should.
+int sgh_copy_ctx_gpu(int device_id, uint64_t src, uint64_t dst, uint64_t len)
+{
+  if (hipSetDevice(device_id) != hipSuccess) return -1;
+  int ok = 0;
+  CopyCtx c;
+  c.device_id = device_id;
+  c.door_bell = BufItemPool<uint32_t>::create_buf_item_pool(1, device_id);
+  if (!c.door_bell) return -2;
+  c.d_door_bell = BufItemPool<uint32_t>::get_dev_ptr(c.door_bell);
+  if (c.d_door_bell) ok |= 1;
+  g_copy_params *skb = BufItemPool<g_copy_params>::create_buf_item_pool(1);  // host memory
+  if (BufItemPool<g_copy_params>::get_dev_ptr(skb) == skb) ok |= 2;          // "no dev mapping": the host pointer
+  if (sg_on_gpu_entry(&c) == 1) ok |= 4;
+  skb->i_buf[0] = src;
+  skb->o_buf[0] = dst;
+  skb->len[0] = len;
+  skb->num_items = 1;
+  if (sg_on_gpu(&c, skb) == 1) ok |= 8;
+  c.ResetAppRunStatus();
+  if (!c.IsAppRunComplete()) ok |= 16;
+  c.AppCompleteNotify(1);
+  c.WaitForAppRunComplete();
+  if (c.IsAppRunComplete()) ok |= 32;
+  c.AppRunNotify(1);  // the doorbell holds 1 already: returns at once
+  sg_on_gpu_exit(&c);
+  BufItemPool<g_copy_params>::delete_buf_item_pool(skb);
+  BufItemPool<uint32_t>::delete_buf_item_pool(c.door_bell, device_id);
+  if (BufItemPool<uint32_t>::get_dev_ptr(c.door_bell) == nullptr) ok |= 64;
+  return ok;
 }
 
 // A double-mapped arena for callers outside C++ (the tests): the request

@@ -17,6 +17,8 @@
 #include <cstring>
 #include <vector>
 
+#include <hip/hip_runtime.h>
+
 #include "sg_hip.h"
 #include "sg_rr.h"
 #include "sg_tables.h"
@@ -118,10 +120,20 @@ struct SgRingView {
 
 class P2pRpcSgHipEngine : public P2pRpcSgEngine {
   sg_hip_ctx *ctx;
-  // pinned staging + device copies of the CSR tables of the batched calls
-  uint32_t *h_tab = nullptr, *d_tab = nullptr;
-  size_t tab_cap = 0;
   uint32_t max_reqs, max_frames;
+
+  // Tables of a batched call are built in pinned host memory and copied to the
+  // device on the engine's stream.  Two such stages take turns, each with an
+  // event behind its last call, so a call waits only if the stage it is about
+  // to overwrite is still being read -- not for everything queued.
+  struct Stage {
+    uint32_t *h = nullptr, *d = nullptr;
+    size_t cap = 0;  // 32-bit words
+    hipEvent_t ev = nullptr;
+    bool busy = false;
+  };
+  Stage stage[2];
+  int turn = 0;
 
   void fail(const char *what, int rc) const
   {
@@ -129,16 +141,52 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
     std::printf("P2pRpcSgHipEngine: %s failed (%d): %s\n", what, rc, sg_hip_last_error(ctx));
   }
 
-  bool tables(size_t words)
+  hipStream_t stream() const { return static_cast<hipStream_t>(sg_hip_stream(ctx)); }
+
+  struct OnDevice {
+    int prev = -1;
+    explicit OnDevice(int dev)
+    {
+      if (hipGetDevice(&prev) != hipSuccess || prev == dev) prev = -1;
+      else (void)hipSetDevice(dev);
+    }
+    ~OnDevice()
+    {
+      if (prev >= 0) (void)hipSetDevice(prev);
+    }
+  };
+
+  Stage *take_stage(size_t words)
   {
-    if (words <= tab_cap) return true;
-    if (h_tab) (void)hipHostFree(h_tab);
-    if (d_tab) (void)hipFree(d_tab);
-    tab_cap = 0;
-    if (hipHostMalloc((void **)&h_tab, words * 4, hipHostMallocDefault) != hipSuccess) return false;
-    if (hipMalloc((void **)&d_tab, words * 4) != hipSuccess) return false;
-    tab_cap = words;
-    return true;
+    Stage &s = stage[turn];
+    turn ^= 1;
+    if (s.busy) {
+      (void)hipEventSynchronize(s.ev);
+      s.busy = false;
+    }
+    if (words > s.cap) {
+      if (s.h) (void)hipHostFree(s.h);
+      if (s.d) (void)hipFree(s.d);
+      s.h = s.d = nullptr;
+      s.cap = 0;
+      const size_t want = words + words / 2 + 64;
+      if (hipHostMalloc((void **)&s.h, want * 4, hipHostMallocDefault) != hipSuccess) return nullptr;
+      if (hipMalloc((void **)&s.d, want * 4) != hipSuccess) return nullptr;
+      s.cap = want;
+    }
+    if (!s.ev && hipEventCreateWithFlags(&s.ev, hipEventDisableTiming) != hipSuccess) return nullptr;
+    return &s;
+  }
+
+  bool send_stage(Stage *s, size_t words)
+  {
+    return hipMemcpyAsync(s->d, s->h, words * 4, hipMemcpyHostToDevice, stream()) == hipSuccess;
+  }
+
+  void stage_in_use(Stage *s)
+  {
+    if (hipEventRecord(s->ev, stream()) == hipSuccess) s->busy = true;
+    else (void)hipStreamSynchronize(stream());
   }
 
  public:
@@ -160,12 +208,18 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
 
   ~P2pRpcSgHipEngine() override
   {
-    if (h_tab) (void)hipHostFree(h_tab);
-    if (d_tab) (void)hipFree(d_tab);
+    OnDevice on(device_id);
+    (void)sg_hip_sync(ctx);
+    for (Stage &s : stage) {
+      if (s.h) (void)hipHostFree(s.h);
+      if (s.d) (void)hipFree(s.d);
+      if (s.ev) (void)hipEventDestroy(s.ev);
+    }
     sg_hip_destroy(ctx);
   }
 
   sg_hip_ctx *context() { return ctx; }
+  int sync() { return last_rc = sg_hip_sync(ctx); }
 
   // ---- the reference's four calls: one request, synchronous ----
   inline void gather(P2pRpcRr *rpc_rr, g_params *app_stub) override { gather(rpc_rr, app_stub->req); }
@@ -206,21 +260,50 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
   }
 
   // ---- batched: every ready request in one call ----
+  // With tables that are on the device already (what reassemble() leaves there).
+  int gather_batch(const sg_gather_args *a)
+  {
+    last_rc = sg_hip_gather_batch(ctx, a);
+    if (last_rc != SG_OK) fail("gather_batch", last_rc);
+    return last_rc;
+  }
+  int scatter_batch(const sg_scatter_args *a)
+  {
+    last_rc = sg_hip_scatter_batch(ctx, a);
+    if (last_rc != SG_OK) fail("scatter_batch", last_rc);
+    return last_rc;
+  }
+
+  // The receive thread's per-packet work for one burst, on the device
+  // (rr_recv_ng + get_rr + rr_emplace_mbuf + is_rr_ready,
+  // src/transport/dpdk_transport_ng.h:176-218): requests that the burst
+  // completes come out as tables gather_batch(const sg_gather_args *) takes;
+  // the others stay on the device for later bursts.  counts (4 words or
+  // nullptr): requests, fragments, arrivals dropped, requests in flight.
+  int reassemble(const sg_reassemble_args *a, uint32_t *counts)
+  {
+    last_rc = sg_hip_reassemble(ctx, a, counts);
+    if (last_rc != SG_OK) fail("reassemble", last_rc);
+    return last_rc;
+  }
+
   // Gathers n requests whose payload pointers lie in `ring` into `app`
   // (consecutive bump-ring positions or tensor-major buffers), in the order
   // given.  fixed_req_size / rule_mtu as in sg_gather_args.  Returns SG_OK or
-  // the error; `flags` may carry SG_F_ASYNC.
+  // the error; `flags` may carry SG_F_ASYNC.  slot_state (or nullptr) and
+  // n_slot_states as in sg_gather_args.
   int gather_batch(P2pRpcRr *const *rrs, uint32_t n, const SgRingView &ring, const sg_app_desc &app,
-                   uint64_t *offsets_out_dev, uint64_t fixed_req_size, uint32_t rule_mtu, uint32_t flags)
+                   uint64_t *offsets_out_dev, uint64_t fixed_req_size, uint32_t rule_mtu, uint32_t flags,
+                   uint32_t *slot_state = nullptr, uint32_t n_slot_states = 0)
   {
     size_t n_frags = 0;
     for (uint32_t r = 0; r < n; r++) n_frags += rrs[r]->payload_bufs->num_items;
     if (n > max_reqs || n_frags > max_frames) return last_rc = SG_E_INVAL;
-    // the staging tables are reused: what the previous call enqueued must have read them
-    if ((last_rc = sg_hip_sync(ctx)) != SG_OK) return last_rc;
+    OnDevice on(device_id);
     const size_t words = 2 * n_frags + n + 1;
-    if (!tables(words)) return last_rc = SG_E_NOMEM;
-    uint32_t *slot = h_tab, *len = h_tab + n_frags, *first = h_tab + 2 * n_frags;
+    Stage *st = take_stage(words);
+    if (!st) return last_rc = SG_E_NOMEM;
+    uint32_t *slot = st->h, *len = st->h + n_frags, *first = st->h + 2 * n_frags;
     size_t f = 0;
     for (uint32_t r = 0; r < n; r++) {
       const p2p_bufs *b = rrs[r]->payload_bufs;
@@ -233,14 +316,13 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
       }
     }
     first[n] = (uint32_t)f;
-    hipStream_t st = static_cast<hipStream_t>(sg_hip_stream(ctx));
-    if (hipMemcpyAsync(d_tab, h_tab, words * 4, hipMemcpyHostToDevice, st) != hipSuccess) return last_rc = SG_E_HIP;
+    if (!send_stage(st, words)) return last_rc = SG_E_HIP;
     sg_gather_args a;
     std::memset(&a, 0, sizeof a);
     a.ring = ring.desc;
-    a.frag_slot = d_tab;
-    a.frag_len = d_tab + n_frags;
-    a.req_first = d_tab + 2 * n_frags;
+    a.frag_slot = st->d;
+    a.frag_len = st->d + n_frags;
+    a.req_first = st->d + 2 * n_frags;
     a.n_req = n;
     a.n_frags = (uint32_t)n_frags;
     a.app = app;
@@ -248,8 +330,77 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
     a.flags = flags | (rule_mtu && fixed_req_size ? SG_F_RULE_FRAGS : 0u);
     a.mtu = rule_mtu;
     a.fixed_req_size = fixed_req_size;
+    a.slot_state = slot_state;
+    a.n_slot_states = n_slot_states;
     last_rc = sg_hip_gather_batch(ctx, &a);
+    stage_in_use(st);
     if (last_rc != SG_OK) fail("gather_batch", last_rc);
+    return last_rc;
+  }
+
+  // The TX half for n requests at once (src/splitrpc_server/p2p_rpc_dpdk_server.cc:158-189 for
+  // every WORK_COMPLETE slot): the response of rrs[k] is read from `app` (next bump-ring positions
+  // or tensor-major buffers), cut at `mtu` into the response buffers rrs[k]->payload_bufs names
+  // (rr_alloc_mbufs has put them there; they lie in `tx`), and every frame's header is written
+  // from the request's connection template with its token, sequence number, lengths and the sums
+  // `flags` asks for (rr_set_hdr, src/transport/dpdk_transport_ng.h:113-141) -- payload and
+  // headers in one kernel.  The response size of a request is what its buffers add up to.
+  int scatter_batch(P2pRpcRr *const *rrs, uint32_t n, const SgRingView &tx, const sg_app_desc &app, uint32_t mtu,
+                    uint32_t flags, uint32_t *slot_state = nullptr, uint32_t n_slot_states = 0)
+  {
+    size_t n_frames = 0;
+    for (uint32_t r = 0; r < n; r++) n_frames += rrs[r]->payload_bufs->num_items;
+    if (n > max_reqs || n_frames > max_frames) return last_rc = SG_E_INVAL;
+    if (n == 0) return last_rc = SG_OK;
+    OnDevice on(device_id);
+    // u32 tx_slot[n_frames], u32 first[n + 1], pad to 8 bytes, u64 token[n], u64 size[n], u8 template[64 n]
+    const size_t w32 = (n_frames + n + 1 + 1) & ~(size_t)1;
+    const size_t words = w32 + 2 * n + 2 * n + 16 * n;
+    Stage *st = take_stage(words);
+    if (!st) return last_rc = SG_E_NOMEM;
+    uint32_t *slot = st->h, *first = st->h + n_frames;
+    uint64_t *token = reinterpret_cast<uint64_t *>(st->h + w32), *size = token + n;
+    uint8_t *tmpl = reinterpret_cast<uint8_t *>(size + n);
+    size_t f = 0;
+    bool one_size = true;
+    for (uint32_t r = 0; r < n; r++) {
+      const p2p_bufs *b = rrs[r]->payload_bufs;
+      first[r] = (uint32_t)f;
+      uint64_t total = 0;
+      for (int i = 0; i < b->num_items; i++, f++) {
+        const int64_t s = tx.slot_of_payload(b->burst_items[i]);
+        if (s < 0) return last_rc = SG_E_INVAL;
+        slot[f] = (uint32_t)s;
+        total += b->item_size[i];
+      }
+      size[r] = total;
+      one_size = one_size && total == size[0];
+      token[r] = rrs[r]->req_token;
+      std::memcpy(tmpl + 64 * (size_t)r, &rrs[r]->_client_conn_info.hdr_template, 64);
+    }
+    first[n] = (uint32_t)f;
+    if (!send_stage(st, words)) return last_rc = SG_E_HIP;
+    sg_scatter_args a;
+    std::memset(&a, 0, sizeof a);
+    a.rx = tx.desc;  // headers come from templates: no request ring is read
+    a.tx = tx.desc;
+    a.tx_slot = st->d;
+    a.resp_first = st->d + n_frames;
+    const uint64_t *d64 = reinterpret_cast<const uint64_t *>(st->d + w32);
+    a.req_token = d64;
+    a.resp_size = one_size ? nullptr : d64 + n;
+    a.fixed_resp_size = one_size ? size[0] : 0;
+    a.hdr_templates = reinterpret_cast<const uint8_t *>(d64 + 2 * n);
+    a.n_req = n;
+    a.n_frames = (uint32_t)n_frames;
+    a.mtu = mtu;
+    a.flags = flags;
+    a.app = app;
+    a.slot_state = slot_state;
+    a.n_slot_states = n_slot_states;
+    last_rc = sg_hip_scatter_batch(ctx, &a);
+    stage_in_use(st);
+    if (last_rc != SG_OK) fail("scatter_batch", last_rc);
     return last_rc;
   }
 };

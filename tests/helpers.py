@@ -46,11 +46,16 @@ def first_diff(a: np.ndarray, b: np.ndarray) -> str:
     return f"{idx.size} bytes differ, first at {i}: got {a[i]} want {b[i]}"
 
 
-def conn_templates(w, seed=0):
+def conn_templates(w, seed=0, server=None, first_slots=None):
     """Per-request connection templates the way the reference builds them: a
     server-side template (gen_*_header_template) pointed at the client by
     set_conn_info with the request's first packet.  Returns (n_req x 64 uint8,
-    n_req uint64 tokens read from those packets)."""
+    n_req uint64 tokens read from those packets).  ``server`` = (mac bytes,
+    ip, port) fixes the server's identity as initialize_src_conn_info does
+    (src/p2p_rpc_conn_info.h:50-70: both MACs the server's, destination
+    0.0.0.0:0); otherwise identities are random.  ``first_slots[r]`` names the
+    packet of request r that reached the server first (the one set_conn_info
+    sees); default: fragment 0."""
     import ctypes as C
     L = oracle.lib()
     rng = np.random.default_rng(seed)
@@ -60,12 +65,16 @@ def conn_templates(w, seed=0):
     for r in range(w.n_req):
         if w.req_first[r + 1] == w.req_first[r]:
             continue
-        slot = int(w.frag_slot[w.req_first[r]])
+        slot = int(first_slots[r]) if first_slots is not None else int(w.frag_slot[w.req_first[r]])
         recv = np.ascontiguousarray(w.ring[slot * w.slot_size: slot * w.slot_size + 64])
-        sm, dm = rng.integers(0, 256, 6, dtype=np.uint8), rng.integers(0, 256, 6, dtype=np.uint8)
         t = np.zeros(64, np.uint8)
-        L.sgo_gen_hdr_template(pp(t), pp(sm), pp(dm), int(rng.integers(0, 2 ** 32)), int(rng.integers(0, 2 ** 32)),
-                               int(rng.integers(0, 65536)), int(rng.integers(0, 65536)))
+        if server is not None:
+            sm = dm = np.frombuffer(bytes(server[0]), np.uint8).copy()
+            L.sgo_gen_hdr_template(pp(t), pp(sm), pp(dm), int(server[1]), 0, int(server[2]), 0)
+        else:
+            sm, dm = rng.integers(0, 256, 6, dtype=np.uint8), rng.integers(0, 256, 6, dtype=np.uint8)
+            L.sgo_gen_hdr_template(pp(t), pp(sm), pp(dm), int(rng.integers(0, 2 ** 32)), int(rng.integers(0, 2 ** 32)),
+                                   int(rng.integers(0, 65536)), int(rng.integers(0, 65536)))
         L.sgo_set_conn_info(pp(t), pp(recv), w.profile)
         tm[r] = t
         tk[r] = recv[42:50].view(np.uint64)[0]

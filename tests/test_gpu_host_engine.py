@@ -10,7 +10,7 @@ import pytest
 import oracle
 from splitrpc_amd import build, synth
 
-from helpers import first_diff
+from helpers import conn_templates, first_diff
 
 pytestmark = pytest.mark.gpu
 
@@ -24,6 +24,8 @@ def host():
                                 C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32, C.c_int, C.c_int,
                                 C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
                                 C.POINTER(C.c_int)]
+    h.sgh_copy_ctx_gpu.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64]
+    h.sgh_zc_engine.argtypes = [C.c_uint64]
     h.sgh_window_replay.restype = C.c_int64
     h.sgh_window_replay.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_uint32, C.c_void_p]
     h.sgh_mempool_create.restype = C.c_void_p
@@ -43,13 +45,15 @@ def p(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
 
-@pytest.mark.parametrize("per_request", [1, 0], ids=["per-request", "batched"])
+@pytest.mark.parametrize("per_request", [1, 0, 2], ids=["per-request", "batched", "batched-tx"])
 @pytest.mark.parametrize("mirror", [1, 0], ids=["mirrored", "plain"])
 @pytest.mark.parametrize("cfg,n,profile", [(1, 12, synth.HDR_BL58), (2, 3, synth.HDR_BL58),
                                            (2, 2, synth.HDR_REF64), (5, 1, synth.HDR_BL58)])
 def test_one_burst_of_the_shunter(host, cfg, n, profile, mirror, per_request):
     w = synth.make_workload(cfg, n, profile=profile)
     flags = w.flags & ~synth.F_UDP_CSUM_FULL  # a header-only rewrite cannot see the payload
+    if per_request == 2:
+        flags = w.flags                           # the batched TX writes headers with the payload in hand
     print(f"case serve cfg={cfg} n={n} profile={profile} mirror={mirror} per_request={per_request}", flush=True)
     req_size, resp_size = int(w.req_sizes[0]), int(w.resp_sizes[0])
     len_nic = None
@@ -69,8 +73,41 @@ def test_one_burst_of_the_shunter(host, cfg, n, profile, mirror, per_request):
     exp, _, _ = oracle.gather(w)
     assert np.array_equal(req_out, exp), first_diff(req_out, exp)
     exp_tx = w.tx_ring_init.copy()
-    oracle.scatter(w, w.ring, exp_tx, w.resp_payload, flags=flags)
+    if per_request == 2:
+        # fresh response buffers: headers from the connections' templates (rr_set_hdr), the server
+        # identity being the one the host layer was started with
+        import socket
+        import struct
+        server = (bytes.fromhex("b8cef6cc6a52"), struct.unpack("!I", socket.inet_aton("192.168.25.1"))[0], 50051)
+        # set_conn_info sees the packet of a request that ARRIVES first, whatever its sequence number
+        req_of_slot = np.full(w.n_slots, -1, np.int64)
+        req_of_slot[w.frag_slot] = np.repeat(np.arange(w.n_req), np.diff(w.req_first.astype(np.int64)))
+        first_slots = np.zeros(w.n_req, np.int64)
+        for s in arr[::-1]:
+            first_slots[req_of_slot[s]] = s
+        tm, tk = conn_templates(w, server=server, first_slots=first_slots)
+        oracle.scatter(w, w.ring, exp_tx, w.resp_payload, flags=flags, templates=tm, tokens=tk)
+    else:
+        oracle.scatter(w, w.ring, exp_tx, w.resp_payload, flags=flags)
     assert np.array_equal(tx, exp_tx), first_diff(tx, exp_tx)
+
+
+def test_copy_context_entry_points_and_small_object_pool(host):
+    """CopyCtx + sg_on_gpu_entry + sg_on_gpu (the reference's C entry points)
+    move a run; the doorbell sits in a BufItemPool object both sides reach."""
+    import torch
+    src = torch.arange(5000, dtype=torch.int32, device="cuda").view(torch.uint8)
+    dst = torch.zeros(20000 + 64, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    got = host.sgh_copy_ctx_gpu(0, src.data_ptr() + 3, dst.data_ptr() + 7, 19990)
+    assert got == 127, f"steps {got:#x}"
+    torch.cuda.synchronize()
+    assert torch.equal(dst[7:7 + 19990], src[3:3 + 19990])
+    assert not bool(dst[:7].any()) and not bool(dst[7 + 19990:].any())
+
+
+def test_zero_copy_engine_hands_out_the_packet_buffer(host):
+    assert host.sgh_zc_engine(0x7f0000001040) == 1
 
 
 @pytest.mark.parametrize("mode", ["scan", "rule"])
