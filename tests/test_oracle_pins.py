@@ -411,23 +411,51 @@ def test_tring_closed_form():
 
 # ---------------------------------------------------------------- reassembly
 
-def _py_reassemble(w, arrivals):
-    """Brute force: group slots by token in arrival order, index by frag_idx,
-    complete when num_frags fragments are in."""
+def _py_reassemble(w, arrivals, len_nic=None, req_size=0):
+    """Brute force: group slots by token in arrival order, index by the
+    fragment's sequence number.  BL58: complete when num_frags fragments are in.
+    REF64 (the reference's header: seq_num at byte 58, no count, no length):
+    lengths come per slot as from the NIC and a request is complete when its
+    bytes add up to the server-wide request size (src/p2p_rpc_rr_ng.h:107-110)."""
     ring = w.ring.reshape(w.n_slots, w.slot_size)
     live, done = {}, []
     for s in arrivals:
         h = ring[s]
         tok = int.from_bytes(bytes(h[42:50]), "little")
-        idx = int.from_bytes(bytes(h[50:52]), "little")
-        nf = int.from_bytes(bytes(h[52:54]), "little")
-        ln = int.from_bytes(bytes(h[54:58]), "little")
+        if tok == 0:
+            continue
+        if w.profile == synth.HDR_REF64:
+            idx = int.from_bytes(bytes(h[58:60]), "little")
+            ln = int(len_nic[s])
+        else:
+            idx = int.from_bytes(bytes(h[50:52]), "little")
+            nf = int.from_bytes(bytes(h[52:54]), "little")
+            ln = int.from_bytes(bytes(h[54:58]), "little")
         d = live.setdefault(tok, {})
         d[idx] = (int(s), ln)
-        if len(d) == nf:
-            done.append((tok, [d[i] for i in range(nf)]))
+        ready = (sum(l for _, l in d.values()) == req_size) if w.profile == synth.HDR_REF64 else (len(d) == nf)
+        if ready:
+            done.append((tok, [d[i] for i in range(len(d))]))
             del live[tok]
     return done
+
+
+@pytest.mark.parametrize("cfg,n", [(1, 8), (2, 2), (5, 2)])
+def test_reassembly_by_request_size_against_brute_force(cfg, n):
+    """The REF64 completion rule of the oracle, against the brute force above,
+    in generated order and shuffled."""
+    w = synth.make_workload(cfg, n, profile=synth.HDR_REF64)
+    len_nic = np.zeros(w.n_slots, np.uint32)
+    len_nic[w.frag_slot] = w.frag_len
+    size = int(w.req_sizes[0])
+    for arr in (w.arrivals, np.random.default_rng(cfg).permutation(w.arrivals)):
+        fs, fl, rf, tok = oracle.reassemble(w, arrivals=arr, req_size=size, frag_len_nic=len_nic)
+        want = _py_reassemble(w, arr, len_nic, size)
+        assert len(want) == n
+        assert tok.tolist() == [t for t, _ in want]
+        assert fs.tolist() == [s for _, fr in want for s, _ in fr]
+        assert fl.tolist() == [l for _, fr in want for _, l in fr]
+        assert rf.tolist() == np.concatenate([[0], np.cumsum([len(fr) for _, fr in want])]).tolist()
 
 
 @pytest.mark.parametrize("cfg,n", [(1, 8), (2, 2), (3, 40), (4, 60), (5, 2)])
@@ -573,10 +601,11 @@ def _py_scatter(w, rx, tx0, streams, flags):
     return tx.reshape(-1)
 
 
+@pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64], ids=["bl58", "ref64"])
 @pytest.mark.parametrize("cfg,n", [(1, 5), (2, 2), (3, 6), (5, 1)])
 @pytest.mark.parametrize("extra", [0, synth.F_REF_QUIRKS, synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL])
-def test_scatter_composite_against_brute_force(cfg, n, extra):
-    w = synth.make_workload(cfg, n)
+def test_scatter_composite_against_brute_force(cfg, n, extra, profile):
+    w = synth.make_workload(cfg, n, profile=profile)
     flags = w.flags | extra
     per = w.resp_payload.size // w.n_req
     streams = [w.resp_payload[r * per:(r + 1) * per] for r in range(w.n_req)]
