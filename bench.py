@@ -36,6 +36,14 @@ MEASURED_TRAFFIC = {(2, 32, "k_gather"): 652.2e6}
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 
+def _log(msg: str) -> None:
+    """Progress on stderr: a long run shows where it is."""
+    print(f"[bench {time.perf_counter() - _T0:7.1f}s] {msg}", file=sys.stderr, flush=True)
+
+
+_T0 = time.perf_counter()
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -53,6 +61,8 @@ def parse():
                          "the 58-byte benchmark header")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-remap", action="store_true", help="disable the XCD-aware launch order")
+    ap.add_argument("--no-small", action="store_true",
+                    help="one wavefront per frame even for short frames (SG_F_NO_SMALL)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 512 MiB device copy a few times (a kernel of known "
                          "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -303,12 +313,14 @@ def main() -> int:
         print("bench.py needs a GPU (cuda:0)", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
-    extra = capi.F_NO_XCD_REMAP if a.no_remap else 0
+    extra = (capi.F_NO_XCD_REMAP if a.no_remap else 0) | (capi.F_NO_SMALL if a.no_small else 0)
     bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
     prof = synth.HDR_REF64 if a.ref64 else synth.HDR_BL58
     w = synth.make_workload(a.workload, profile=prof)
     ctx = SgContext(0, max_reqs=max(4096, w.n_req * bpl), max_frames=max(65536, max(w.n_frags, w.n_resp_frames) * bpl))
+    _log(f"staging {w.name} x {bpl} batches per launch")
     pool = Pool(w, bpl, a.rotate_mb, extra, rule=not a.general)
+    _log(f"{len(pool.items)} ring copies staged")
 
     if a.calib_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").fill_(3)
@@ -319,6 +331,7 @@ def main() -> int:
         del src, dst
 
     sec = timed(ctx, pool, a.steps, a.warmup)
+    _log(f"timed: {sec * 1e6:.1f} us per step")
     kt = kernel_times(ctx, pool, min(a.steps, 100))
     total_bytes = pool.gather_bytes + pool.scatter_bytes
     value = total_bytes / sec / 1e9
@@ -328,6 +341,7 @@ def main() -> int:
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     b2b = back_to_back(ctx, pool, dom, min(a.steps, 100))
 
+    _log("kernel times and back-to-back done; reassembly")
     # request reassembly on the device for the same call's arrivals (synchronous: counts come back)
     dw0 = pool.items[0]
     n_arr = int(dw0.arrivals.numel())
@@ -352,6 +366,7 @@ def main() -> int:
                   "tables_match_pre_staged": bool(got[0] == pool.n_req and torch.equal(ra_fs, dw0.frag_slot))}
     del ra_fs, ra_fl, ra_rf
 
+    _log("reassembly done; single-batch call")
     # the single-batch call of the same workload, for the record
     single = None
     if bpl != 1:
@@ -369,6 +384,7 @@ def main() -> int:
         single["hip_graph_ms_per_step"] = round(sg * 1e3, 5)
         single["hip_graph_requests_per_sec"] = round(w.n_req / sg, 1)
 
+    _log("per-request calls")
     per_req = per_request_calls(ctx, pool.items[0]) if not w.in_tensor_sizes else None
     rps = {WORKLOAD_NAMES[a.workload]: round(pool.n_req / sec, 1)}
     sweep = {}
@@ -378,6 +394,7 @@ def main() -> int:
                 continue
             wc = synth.make_workload(cfg)
             b = DEFAULT_BPL[cfg]
+            _log(f"sweep: {wc.name} x {b}")
             c2 = SgContext(0, max_reqs=max(4096, wc.n_req * b),
                            max_frames=max(65536, max(wc.n_frags, wc.n_resp_frames) * b))
             pc = Pool(wc, b, a.rotate_mb, extra, rule=not a.general)

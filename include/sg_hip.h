@@ -70,6 +70,9 @@ extern "C" {
                                           kernel could derive the descriptors (for experiments) */
 #define SG_F_ASYNC (1u << 16)          /* enqueue only; completion through sg_hip_sync() */
 #define SG_F_NO_XCD_REMAP (1u << 17)   /* launch-order = item order (for experiments) */
+#define SG_F_NO_SMALL (1u << 18)       /* one wavefront per frame even for short frames (for experiments) */
+#define SG_F_FORCE_SMALL (1u << 19)    /* short remainder frames always go several to a wavefront, also where
+                                          the call is too small for the extra launch to pay (for tests) */
 
 /* States of an application slot (APP_RR_STATUS, src/p2p_rpc_app_ctx.h:22). */
 #define SG_SLOT_FREE 0u

@@ -29,6 +29,8 @@ F_RULE_FRAGS = 1 << 4
 F_NO_FUSE = 1 << 5
 F_ASYNC = 1 << 16
 F_NO_XCD_REMAP = 1 << 17
+F_NO_SMALL = 1 << 18
+F_FORCE_SMALL = 1 << 19
 
 MAX_BI_SIZE = 1024
 MAX_TENSORS = 4

@@ -434,4 +434,222 @@ __device__ __forceinline__ uint32_t hdr_rewrite(const uint8_t *__restrict__ in, 
   return hdr_finish(hdr_fetch(in, lane, f.hl), lane, f, payload_sum);
 }
 
+
+// ---- short frames: several frames per wavefront -----------------------------
+// A frame of a few hundred bytes does not fill a wavefront: most lanes idle
+// while the wavefront pays the full price in instructions and round trips.
+// The functions below give a frame to a GROUP of L = 16 or 32 consecutive
+// lanes, so that a wavefront moves 64 / L frames at once.  Everything a group
+// works with (addresses, lengths, indices) lives in vector registers, the same
+// value on every lane of the group; nothing here is wavefront-uniform.
+
+// Sum over the 16 lanes of a row, left in every lane of the row: DPP adds, no LDS.
+__device__ __forceinline__ uint32_t row_sum(uint32_t v)
+{
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xb1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4e, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false);  // row_half_mirror
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false);  // row_mirror
+  return v;
+}
+
+// Sum over the L lanes of a group.
+template <int L>
+__device__ __forceinline__ uint32_t group_sum(uint32_t v)
+{
+  v = row_sum(v);
+  if (L == 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+
+// One run in the hands of a group of L lanes: the scheme of RunState above with
+// L aligned source chunks per step yielding L - 1 destination chunks (the
+// group's last lane has no upper neighbour of its own: the wave shift hands it
+// a foreign lane's chunk, which it does not use).  Lanes 0..15 of the group
+// carry one head byte and one tail byte each.
+template <int L>
+struct GroupRun {
+  const uint8_t *sa;
+  uint8_t *d;
+  uint8_t *dst;
+  uint32_t body, lim, p;
+  uint32_t head_b, tail_b, tail_off;
+  bool has_head, has_tail;
+  u32x4 v0, v1;
+};
+
+template <int L>
+__device__ __forceinline__ void group_run_begin(GroupRun<L> &r, const uint8_t *src, uint8_t *dst, uint32_t len,
+                                                uint32_t gl)
+{
+  uint32_t head = (uint32_t)(-(uintptr_t)dst) & 15u;
+  head = head < len ? head : len;
+  const uint32_t body = (len - head) >> 4;
+  const uint32_t tail = (len - head) & 15u;
+  r.dst = dst;
+  r.body = body;
+  r.has_head = gl < head;
+  r.has_tail = gl < tail;
+  r.tail_off = head + (body << 4) + gl;
+  r.head_b = r.has_head ? src[gl] : 0u;
+  r.tail_b = r.has_tail ? src[r.tail_off] : 0u;
+  const uint8_t *s = src + head;
+  r.d = dst + head;
+  r.p = (uint32_t)(uintptr_t)s & 15u;
+  r.sa = s - r.p;
+  r.lim = r.p ? body : body - 1;  // body == 0: lim wraps, guarded below
+  r.v0 = (u32x4){0, 0, 0, 0};
+  r.v1 = (u32x4){0, 0, 0, 0};
+  if (body) {
+    if (gl <= r.lim) r.v0 = load16_aligned(r.sa + ((size_t)gl << 4));
+    if ((L - 1) + gl <= r.lim) r.v1 = load16_aligned(r.sa + ((size_t)((L - 1) + gl) << 4));
+  }
+}
+
+// Returns this lane's share of the little-endian 16-bit word sum with CSUM.
+// Every lane of the wavefront has to call this (the realignment shifts values
+// across lanes); a group without a run passes body = 0 and no edge bytes.
+template <int L, bool CSUM>
+__device__ __forceinline__ uint32_t group_run_end(GroupRun<L> &r, uint32_t gl)
+{
+  uint32_t acc = 0;
+  // the phase differs from group to group: realign() switches on it per lane
+  const u32x4 o0 = realign(r.v0, r.p);
+  const u32x4 o1 = realign(r.v1, r.p);
+  if (gl < L - 1 && gl < r.body) {
+    store16_aligned(r.d + ((size_t)gl << 4), o0);
+    if (CSUM) acc += words_sum(o0);
+  }
+  if (gl < L - 1 && (L - 1) + gl < r.body) {
+    store16_aligned(r.d + ((size_t)((L - 1) + gl) << 4), o1);
+    if (CSUM) acc += words_sum(o1);
+  }
+  // longer runs: the wavefront keeps stepping while any of its groups has chunks left
+  for (uint32_t base = 2 * (L - 1); __any(base < r.body); base += 2 * (L - 1)) {
+    const uint32_t c0 = base + gl, c1 = base + (L - 1) + gl;
+    u32x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+    if (c0 <= r.lim && base < r.body) v0 = load16_aligned(r.sa + ((size_t)c0 << 4));
+    if (c1 <= r.lim && base < r.body) v1 = load16_aligned(r.sa + ((size_t)c1 << 4));
+    const u32x4 q0 = realign(v0, r.p);
+    const u32x4 q1 = realign(v1, r.p);
+    if (gl < L - 1 && c0 < r.body) {
+      store16_aligned(r.d + ((size_t)c0 << 4), q0);
+      if (CSUM) acc += words_sum(q0);
+    }
+    if (gl < L - 1 && c1 < r.body) {
+      store16_aligned(r.d + ((size_t)c1 << 4), q1);
+      if (CSUM) acc += words_sum(q1);
+    }
+  }
+  if (r.has_head) {
+    r.dst[gl] = (uint8_t)r.head_b;
+    if (CSUM) acc += ((uintptr_t)(r.dst + gl) & 1u) ? (r.head_b << 8) : r.head_b;
+  }
+  if (r.has_tail) {
+    r.dst[r.tail_off] = (uint8_t)r.tail_b;
+    if (CSUM) acc += ((uintptr_t)(r.dst + r.tail_off) & 1u) ? (r.tail_b << 8) : r.tail_b;
+  }
+  return acc;
+}
+
+// Response header of one frame on the first 16 lanes of a group, two 16-bit
+// words per lane: lane j holds header bytes 4j .. 4j+3.  Every field of the
+// header is a whole number of 16-bit words at an even offset, so the rewrite
+// of hdr_finish above becomes word moves: word h comes from word hdr_src_word(h)
+// of the incoming header (MACs, addresses, ports exchanged) or from word h of a
+// template, length / routing / checksum words are overridden, and the sums run
+// over the words as they lie in memory (little-endian), which yields the
+// network-order checksums.  Same fields and flags as HdrFields.
+__device__ __forceinline__ uint32_t hdr_src_word(uint32_t h)
+{
+  if (h < 3) return h + 3;
+  if (h < 6) return h - 3;
+  if (h == 13 || h == 14) return h + 2;
+  if (h == 15 || h == 16) return h - 2;
+  if (h == 17) return 18;
+  if (h == 18) return 17;
+  return h;
+}
+
+struct SmallHdr {
+  uint32_t w0, w1;  // words 2j and 2j+1 as fetched
+};
+
+__device__ __forceinline__ SmallHdr small_hdr_fetch(const uint8_t *in, uint32_t j, uint32_t hl, bool swap, bool live)
+{
+  SmallHdr h{0u, 0u};
+  const uint32_t n_words = hl >> 1;
+  const uint16_t *w = reinterpret_cast<const uint16_t *>(in);  // rings and templates start at even addresses
+  if (live && 2 * j < n_words) h.w0 = w[swap ? hdr_src_word(2 * j) : 2 * j];
+  if (live && 2 * j + 1 < n_words) h.w1 = w[swap ? hdr_src_word(2 * j + 1) : 2 * j + 1];
+  return h;
+}
+
+__device__ __forceinline__ uint32_t bswap16(uint32_t v) { return ((v & 0xffu) << 8) | ((v >> 8) & 0xffu); }
+
+// One header word's final value.
+__device__ __forceinline__ uint32_t small_hdr_word(uint32_t v, uint32_t h, const HdrFields &f, uint32_t tot, uint32_t ulen)
+{
+  if (h == 8) v = bswap16(tot);
+  if (h == 19) v = bswap16(ulen);
+  if (!f.from_template && (h == 12 || h == 20)) v = 0;  // swap_eth_hdr zeroes both sums
+  if (f.set_token && h >= 21 && h < 25) v = (uint32_t)(f.token >> (16u * (h - 21u))) & 0xffffu;
+  if (f.ref64) {
+    if (h == 25 || h == 26) v = 0;  // sock_perf_header &= 0xFFFFFFFF00000000
+    if (h == 29) v = f.frag_idx & 0xffffu;
+  } else {
+    if (h == 25) v = f.frag_idx & 0xffffu;
+    if (h == 26) v = f.num_frags & 0xffffu;
+    if (h == 27) v = f.payload_len & 0xffffu;
+    if (h == 28) v = f.payload_len >> 16;
+  }
+  return v;
+}
+
+// Finishes and stores the header of the group's frame at `out`.  `j` is the
+// lane's index in its group; lanes 16.. of a 32-lane group take part in the
+// sums only.  `live` says whether the group has a frame at all; payload_sum is
+// the group-wide sum of the payload's little-endian words (full UDP checksum).
+template <int L>
+__device__ __forceinline__ void small_hdr_finish(SmallHdr s, uint8_t *out, uint32_t j, const HdrFields &f,
+                                                 uint32_t payload_sum, bool live)
+{
+  const uint32_t n_words = f.hl >> 1;
+  const uint32_t Lx = (f.hl - 42u) + f.payload_len;
+  const uint32_t tot = (28u + Lx) & 0xffffu, ulen = (8u + Lx) & 0xffffu;
+  const uint32_t h0 = 2 * j, h1 = 2 * j + 1;
+  const bool on0 = live && j < 16 && h0 < n_words, on1 = live && j < 16 && h1 < n_words;
+  uint32_t v0 = on0 ? small_hdr_word(s.w0, h0, f, tot, ulen) : 0u;
+  uint32_t v1 = on1 ? small_hdr_word(s.w1, h1, f, tot, ulen) : 0u;
+  const uint32_t kAnyCsum = 0x7u;  // IPV4 | PSEUDO | FULL
+  if (f.flags & kAnyCsum) {
+    auto in = [](uint32_t h, uint32_t a, uint32_t b) { return h >= a && h < b; };
+    const uint32_t s_ip = group_sum<L>((in(h0, 7, 17) && h0 != 12 ? v0 : 0u) + (in(h1, 7, 17) && h1 != 12 ? v1 : 0u));
+    const uint32_t s_addr = group_sum<L>((in(h0, 13, 17) ? v0 : 0u) + (in(h1, 13, 17) ? v1 : 0u));
+    // word 7 = bytes 14, 15 (version/ihl first); word 11 = bytes 22, 23 (protocol second)
+    const uint32_t pick = group_sum<L>((h1 == 7 ? (v1 & 0xffu) : 0u) + (h1 == 11 ? (v1 & 0xff00u) : 0u));
+    const uint32_t b14 = pick & 0xffu, proto = pick >> 8;
+    uint32_t udp = 0xffffffffu, ipc = 0xffffffffu;
+    if (f.flags & (1u << 1)) {  // raw pseudo sum, reference style
+      const uint32_t hdr_bytes = (f.flags & (1u << 3)) ? (b14 >> 4) * 4u : (b14 & 0xfu) * 4u;
+      const uint32_t l = (tot - hdr_bytes) & 0xffffu;
+      udp = fold16(s_addr + (proto << 8) + bswap16(l));
+    }
+    if (f.flags & (1u << 2)) {  // finished UDP checksum
+      const uint32_t s_l4 = group_sum<L>(((in(h0, 17, 20) || in(h0, 21, n_words)) ? v0 : 0u) +
+                                         ((in(h1, 17, 20) || in(h1, 21, n_words)) ? v1 : 0u));
+      uint32_t t = s_addr + (proto << 8) + bswap16(ulen) + s_l4;
+      t = fold16(fold16(t) + fold16(payload_sum));
+      udp = (~t) & 0xffffu;
+      if (udp == 0) udp = 0xffffu;
+    }
+    if (f.flags & (1u << 0)) ipc = (~fold16(s_ip)) & 0xffffu;
+    if (h0 == 20 && udp != 0xffffffffu) v0 = udp;
+    if (h0 == 12 && ipc != 0xffffffffu) v0 = ipc;
+  }
+  uint16_t *w = reinterpret_cast<uint16_t *>(out);
+  if (on0) w[h0] = (uint16_t)v0;
+  if (on1) w[h1] = (uint16_t)v1;
+}
+
 }  // namespace sg

@@ -497,6 +497,11 @@ struct RuleArgs {
   uint32_t n_req;
   uint32_t n_slots;
   uint32_t single_wrap;  // n_req * size <= capacity: a request offset wraps at most once
+  // A short last frame per response goes to k_scatter_small: this kernel then takes
+  // per_launch = per_req - 1 frames of every response (else per_launch == per_req).
+  uint32_t per_launch;
+  uint32_t div_mul, div_shift;  // item / per_req == (item * div_mul) >> div_shift for item < 2^27
+  uint32_t lmul, lshift;        // the same for per_launch
   const uint64_t *cursor;  // read only here; k_finish advances it behind this kernel
   uint64_t *offsets_out;
 };
@@ -642,6 +647,39 @@ __device__ __forceinline__ bool plain_target(const AppDev &app, uint64_t req_off
   return false;
 }
 
+// Where byte `pos` of request r's stream lives, whatever the layout (the slow
+// way, for the rare frame that straddles an arena end or a tensor boundary).
+__device__ __forceinline__ uint8_t *app_byte(const AppDev &app, uint64_t req_off, uint32_t r, uint64_t pos)
+{
+  if (app.n_tensors == 0) return app.arena + (req_off + pos) % app.cap;
+  uint64_t t0 = 0;
+  for (uint32_t t = 0; t < app.n_tensors; t++) {
+    if (pos < t0 + app.tensor_size[t]) return app.tensor_base[t] + (uint64_t)r * app.tensor_size[t] + (pos - t0);
+    t0 += app.tensor_size[t];
+  }
+  return nullptr;
+}
+
+// [off, off+len) of request r's byte stream when it starts in one tensor-major
+// buffer and ends in the next: the two pieces.  False for anything else.
+__device__ __forceinline__ bool two_tensor_target(const AppDev &app, uint32_t r, uint32_t off, uint32_t len,
+                                                  uint8_t **to_a, uint32_t *len_a, uint8_t **to_b)
+{
+  uint64_t t0 = 0;
+  for (uint32_t t = 0; t + 1 < app.n_tensors; t++) {
+    const uint64_t t1 = t0 + app.tensor_size[t];
+    if (off < t1) {
+      if ((uint64_t)off + len <= t1 || (uint64_t)off + len > t1 + app.tensor_size[t + 1]) return false;
+      *to_a = app.tensor_base[t] + (uint64_t)r * app.tensor_size[t] + (off - t0);
+      *len_a = (uint32_t)(t1 - off);
+      *to_b = app.tensor_base[t + 1] + (uint64_t)r * app.tensor_size[t + 1];
+      return true;
+    }
+    t0 = t1;
+  }
+  return false;
+}
+
 // Gather from descriptors written by the descriptor pass.  One wavefront per
 // fragment piece: a fragment longer than kPieceChunks chunks is spread over
 // `pieces` consecutive wavefronts.  (Several fragments per wavefront were
@@ -706,6 +744,11 @@ struct GatherRuleArgs {
   uint32_t n_items;
   uint32_t per_req;
   uint32_t div_mul, div_shift;  // item / per_req == (item * div_mul) >> div_shift for item < 2^27
+  // A short last fragment per request goes to k_gather_small: this kernel then takes
+  // per_launch = per_req - 1 fragments of every request (else per_launch == per_req);
+  // lmul / lshift divide by per_launch as div_mul / div_shift divide by per_req.
+  uint32_t per_launch, lmul, lshift;
+  uint32_t period, pmul, pshift;  // wavefronts per turn of full and remainder work, and the division by it
   uint32_t mtu;
   uint32_t slot_size;
   uint32_t hl;
@@ -726,8 +769,16 @@ constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
 // slots start at 16-byte aligned addresses: the header's length field can be read as part of
 // the aligned chunk at byte 48 (a ring only has to start at an even address)
 constexpr uint32_t kOptHdrChunk = 16u;
+constexpr uint32_t kOptSmallLast = 32u;  // the last fragment of every request is left to k_gather_small
 
-template <bool LONG>
+template <int L>
+__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave);
+
+// SMALL: lanes per remainder fragment (16 or 32) when the last fragment of every
+// request is short -- the wavefronts behind those of the full fragments then move
+// 64 / SMALL remainder fragments each, in the same launch (a launch of their own
+// would be all latency: tens of megabytes at most); 0: no such wavefronts.
+template <bool LONG, int SMALL>
 __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
 {
   const uint8_t *ring = a.ring;
@@ -749,17 +800,39 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     n_items = n_req * per_req;
   }
 
-  const uint32_t w = item_of_wave((opts & kOptRemap) != 0);
-  const uint32_t item = LONG ? w / pieces : w;
+  uint32_t w = item_of_wave((opts & kOptRemap) != 0);
+  const uint32_t pl = a.per_launch;
+  if (SMALL) {
+    // Wavefronts of the two kinds are dealt in turns: after the period - 1 wavefronts of the full
+    // fragments of 64 / SMALL requests comes the one that moves those requests' remainders.  The
+    // short-fragment wavefronts are bound by their arithmetic, the others by memory: side by side
+    // on a CU they overlap, one kind after the other they would not.
+    const uint32_t blk = (uint32_t)(((uint64_t)w * a.pmul) >> a.pshift);
+    const uint32_t j = w - blk * a.period;
+    if (j == a.period - 1) {
+      gather_small_wave<(SMALL ? SMALL : 16)>(a, blk);
+      return;
+    }
+    w = blk * (a.period - 1) + j;
+    if (w >= n_req * pl * (LONG ? pieces : 1u)) return;
+  }
+  uint32_t item = LONG ? w / pieces : w;
   const uint32_t piece = LONG ? w - item * pieces : 0;
-  if (item >= n_items) return;
+  // division by the fragments per request as a multiplication the host prepared (a division of
+  // two scalars is some twenty scalar instructions, and the scalar unit is the busiest here)
+  uint32_t r, i;
+  if (SMALL) {
+    r = (uint32_t)(((uint64_t)item * a.lmul) >> a.lshift);
+    i = item - r * pl;
+    item = r * per_req + i;
+  } else {
+    if (item >= n_items) return;
+    r = (uint32_t)(((uint64_t)item * div_mul) >> div_shift);
+    i = item - r * per_req;
+  }
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t slot = sload(frag_slot + item);
   uint64_t c0 = cap ? sload(cursor_in) : 0;
-  // division by the fragments per request as a multiplication the host prepared (a division of
-  // two scalars is some twenty scalar instructions, and the scalar unit is the busiest here)
-  const uint32_t r = (uint32_t)(((uint64_t)item * div_mul) >> div_shift);
-  const uint32_t i = item - r * per_req;
   const uint32_t off = i * mtu;
   const uint32_t rem = (uint32_t)size - off;  // sizes are below 4 GiB (checked by the host)
   const uint32_t len = rem <= mtu ? rem : mtu;
@@ -815,9 +888,22 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   uint32_t sub_off = 0, sub_len = len;
   if (LONG && plain) sub_run(to, len, piece, &sub_off, &sub_len);
   if (plain && sub_len) run_begin(rs, pkt + hl + sub_off, to + sub_off, sub_len, lane);
+  // a fragment that runs from one tensor into the next: two runs, both in flight at once
+  uint8_t *to_a = nullptr, *to_b = nullptr;
+  uint32_t len_a = 0;
+  const bool two = !plain && (opts & kOptMultiTensor) && piece == 0 &&
+                   two_tensor_target(a.app, r, off, len, &to_a, &len_a, &to_b);
+  RunState rb;
+  if (two) {
+    run_begin(rs, pkt + hl, to_a, len_a, lane);
+    run_begin(rb, pkt + hl + len_a, to_b, len - len_a, lane);
+  }
   asm volatile("" ::"v"(hc), "v"(hv));  // consumed only after the payload loads are under way
   if (plain) {
     if (sub_len) run_end<false>(rs, lane);
+  } else if (two) {
+    run_end<false>(rs, lane);
+    run_end<false>(rb, lane);
   } else if (piece == 0) {
     move_run<true, false>(a.app, ro, r, off, pkt + hl, len, lane);
   }
@@ -830,6 +916,99 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     if (i == 0 && sload(a.first + r) != item) bad |= kStBadTable;
     if (bad && lane == 0) refuse(a.status, a.status_flag, bad);
   }
+}
+
+// Gather of SHORT fragments, 64 / L fragments per wavefront (L = 16 or 32 lanes
+// per fragment): the rule form of the gather for fragments of a few hundred
+// bytes -- every fragment of the call (per_launch == per_req) or the last
+// fragment of every request (the remainder; the full fragments then go through
+// k_gather_rule).  Addressing is per lane.
+template <int L>
+__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave)
+{
+  constexpr uint32_t G = kWave / L;
+  const uint32_t lane = threadIdx.x & (kWave - 1), gl = lane & (L - 1);
+  const uint32_t per_req = a.per_req, mtu = a.mtu, hl = a.hl;
+  const uint32_t n_req = dev_count(a.counts, 0, a.n_req);
+  const bool last_only = (a.opts & kOptSmallLast) != 0;
+  const uint32_t n_frags = last_only ? n_req : n_req * per_req;
+  if (wave * G >= n_frags) return;  // the whole wavefront
+  const uint32_t fi = wave * G + lane / L;
+  bool live = fi < n_frags;
+  uint32_t r = 0, i = 0, item = 0;
+  if (live) {
+    if (last_only) {
+      r = fi;
+      i = per_req - 1;
+      item = r * per_req + i;
+    } else {
+      item = fi;
+      r = (uint32_t)(((uint64_t)item * a.div_mul) >> a.div_shift);
+      i = item - r * per_req;
+    }
+  }
+  const uint32_t off = i * mtu;
+  const uint32_t rem = (uint32_t)a.size - off;  // sizes are below 4 GiB (checked by the host)
+  const uint32_t len = live ? (rem <= mtu ? rem : mtu) : 0u;
+  const uint32_t slot = live ? a.frag_slot[item] : 0u;
+  const uint32_t first_r = live && i == 0 ? a.first[r] : item;
+  uint32_t bad = 0;
+  if (slot >= a.n_slots) bad |= kStBadSlot;
+  if (first_r != item) bad |= kStBadTable;
+  // offsets depend on the item, the size and the cursor only: they are out before a bad fragment is dropped
+  uint64_t ro = 0;
+  if (a.cap) {
+    uint64_t c0 = sload(a.cursor);
+    if (c0 >= a.cap) c0 %= a.cap;  // only after a set_cursor beyond the capacity
+    ro = c0 + (uint64_t)r * a.size;
+    ro = ro >= a.cap ? ro - a.cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
+    if (live && gl == 0 && a.offsets_out) {
+      if (i == 0) a.offsets_out[r] = ro;
+      if (item == n_req * per_req - 1) {
+        const uint64_t end = ro + a.size;  // size <= capacity
+        a.offsets_out[n_req] = end >= a.cap ? end - a.cap : end;
+      }
+    }
+  }
+  if (live && (bad & kStBadSlot)) {
+    if (gl == 0) refuse(a.status, a.status_flag, kStBadSlot);
+    live = false;
+  }
+  const uint8_t *pkt = a.ring + (size_t)(live ? slot : 0u) * a.slot_size;
+  // the fragment's real length, fetched with the payload
+  uint32_t hdr_len = len;
+  if (live && gl == 0) hdr_len = a.frag_len ? a.frag_len[item] : load32_any(pkt + 54);
+  uint8_t *to = nullptr;
+  bool plain = false;
+  if (live && len) {
+    if (a.cap) {
+      // the packed arena, walked through the AppDev view the host filled in for this kernel
+      plain = plain_target(a.app, ro, r, off, len, &to);
+    } else if (a.opts & kOptMultiTensor) {
+      plain = plain_target(a.app, 0, r, off, len, &to);
+    } else {
+      to = a.dst + (uint64_t)r * a.size + off;
+      plain = true;
+    }
+  }
+  GroupRun<L> run;
+  group_run_begin<L>(run, pkt + hl, to, plain ? len : 0u, gl);
+  group_run_end<L, false>(run, gl);
+  if (live && len && !plain) {
+    // across an arena end or a tensor boundary: byte by byte
+    for (uint32_t k = gl; k < len; k += L) *app_byte(a.app, ro, r, (uint64_t)off + k) = pkt[hl + k];
+  }
+  if (live && gl == 0) {
+    if (hdr_len != len) bad |= kStNotRule;
+    if (bad) refuse(a.status, a.status_flag, bad);
+  }
+}
+
+// Every fragment of the call is short.
+template <int L>
+__global__ __launch_bounds__(kBlock) void k_gather_small(GatherRuleArgs a)
+{
+  gather_small_wave<L>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
 }
 
 struct ScatterArgs {
@@ -900,12 +1079,21 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   }
   const uint32_t w = item_of_wave(remap != 0);
   const uint32_t pieces = SPLIT ? n_pieces : 1u;
-  const uint32_t item = SPLIT ? w / pieces : w;
-  const uint32_t piece = SPLIT ? w - item * pieces : 0;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   // descriptor path: this kernel does not read the cursor and commits what the descriptor pass left
   if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts)))
     *a.cursor = sload(a.next_cursor);
+  uint32_t item = SPLIT ? w / pieces : w;
+  const uint32_t piece = SPLIT ? w - item * pieces : 0;
+  if (FUSED && a.rule.per_launch != a.rule.per_req) {
+    // the short remainder frame of every response is k_scatter_small's (a launch of its own: with
+    // both kinds of wavefront in one kernel, in turns or one kind after the other, the full frames
+    // lost more than the second launch costs): this launch counts the other frames only
+    const uint32_t pl = a.rule.per_launch;
+    if (item >= n_req * pl) return;
+    const uint32_t rr = (uint32_t)(((uint64_t)item * a.rule.lmul) >> a.rule.lshift);
+    item = rr * a.rule.per_req + (item - rr * pl);
+  }
   if (item >= n_items) return;
   const bool from_template = hdr_templates != nullptr;
   // independent table reads, asked for together
@@ -991,6 +1179,110 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   // the payload went past the header only, so a TX slot that is the header's own
   // source still held the request header when it was fetched above
   if (lane < hl) slot[lane] = (uint8_t)hb;
+}
+
+// Scatter of SHORT frames, 64 / L frames per wavefront (L = 16 or 32 lanes per
+// frame): the fused form of k_scatter -- responses of one size cut by the
+// fragmenting rule -- for frames of a few hundred bytes, where one wavefront per
+// frame spends most of its time on addressing and header arithmetic that 48 of
+// its 64 lanes take no part in.  Either every frame of the call (rule.per_launch
+// == rule.per_req) or the last frame of every response (the remainder; the full
+// frames then go through k_scatter).  Addressing is per lane, the header is two
+// 16-bit words per lane, sums are row reductions.
+template <int L, bool FULL_CSUM>
+__device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_t wave)
+{
+  constexpr uint32_t G = kWave / L;
+  const uint32_t lane = threadIdx.x & (kWave - 1), gl = lane & (L - 1);
+  const uint32_t per_req = a.rule.per_req, mtu = a.rule.mtu, hl = a.hl;
+  const uint32_t n_req = dev_count(a.counts, 0, a.n_req);
+  const bool last_only = a.rule.per_launch != per_req;
+  const uint32_t n_frames = last_only ? n_req : n_req * per_req;
+  if (wave * G >= n_frames) return;  // the whole wavefront
+  const uint32_t fi = wave * G + lane / L;
+  bool live = fi < n_frames;
+  uint32_t r = 0, i = 0, item = 0;
+  if (live) {
+    if (last_only) {
+      r = fi;
+      i = per_req - 1;
+      item = r * per_req + i;
+    } else {
+      item = fi;
+      r = (uint32_t)(((uint64_t)item * a.rule.div_mul) >> a.rule.div_shift);
+      i = item - r * per_req;
+    }
+  }
+  const uint32_t off = i * mtu;
+  const uint32_t rem = (uint32_t)a.rule.size - off;  // response sizes are below 4 GiB (checked by the host)
+  const uint32_t len = live ? (rem <= mtu ? rem : mtu) : 0u;
+  const bool from_template = a.hdr_templates != nullptr;
+  // tables: independent reads
+  uint32_t bad = 0;
+  const uint32_t tslot = live ? a.rule.item_slot[item] : 0u;
+  const uint32_t first_r = live ? a.rule.first[r] : 0u;
+  uint32_t hs = 0;
+  if (live && !from_template) hs = a.hdr_src_req ? a.hdr_src_req[r] : a.hdr_src_slot[item];
+  if (tslot >= a.rule.n_slots) bad |= kStBadSlot;
+  if (i == 0 && first_r != item) bad |= kStBadTable;
+  if (hs >= a.rx_n_slots) bad |= kStBadSlot;
+  if (live && bad && gl == 0) refuse(a.status, a.status_flag, bad);
+  // offsets depend on the item, the size and the cursor only: they are out before a bad frame is dropped
+  uint64_t ro = 0;
+  if (a.app.n_tensors == 0) {
+    uint64_t c0 = sload(a.rule.cursor);
+    if (c0 >= a.app.cap) c0 %= a.app.cap;  // only after a set_cursor beyond the capacity
+    uint64_t o = c0 + (uint64_t)r * a.rule.size;
+    if (a.rule.single_wrap) o = o >= a.app.cap ? o - a.app.cap : o;
+    else o %= a.app.cap;
+    ro = o;
+    if (live && gl == 0 && a.rule.offsets_out) {
+      if (i == 0) a.rule.offsets_out[r] = ro;
+      if (item == n_req * per_req - 1) {
+        const uint64_t end = ro + a.rule.size;  // size <= capacity
+        a.rule.offsets_out[n_req] = end >= a.app.cap ? end - a.app.cap : end;
+      }
+    }
+  }
+  live = live && !bad;
+  uint8_t *slot = a.tx + (size_t)tslot * a.tx_slot_size;
+  HdrFields hf{hl, a.ref64, a.flags, i, per_req, len, 0, 0, 0};
+  const uint8_t *hin;
+  if (from_template) {
+    hin = a.hdr_templates + (size_t)r * 64;
+    hf.from_template = 1;
+    if (a.req_token) {
+      hf.set_token = 1;
+      hf.token = live ? a.req_token[r] : 0;
+    }
+  } else {
+    hin = a.rx + (size_t)hs * a.rx_slot_size;
+  }
+  // header words and payload chunks are fetched together; a TX slot that is its own header
+  // source still holds the request header then (the payload goes past the header only)
+  const SmallHdr sh = small_hdr_fetch(hin, gl, hl, !from_template, live && gl < 16);
+  uint8_t *from = nullptr;
+  const bool plain = live && len != 0 && plain_target(a.app, ro, r, off, len, &from);
+  GroupRun<L> run;
+  group_run_begin<L>(run, from, slot + hl, plain ? len : 0u, gl);
+  uint32_t acc = group_run_end<L, FULL_CSUM>(run, gl);
+  if (live && len != 0 && !plain) {
+    // across an arena end or a tensor boundary: byte by byte
+    for (uint32_t k = gl; k < len; k += L) {
+      const uint32_t b = *app_byte(a.app, ro, r, (uint64_t)off + k);
+      slot[hl + k] = (uint8_t)b;
+      if (FULL_CSUM) acc += ((uintptr_t)(slot + hl + k) & 1u) ? (b << 8) : b;
+    }
+  }
+  const uint32_t psum = FULL_CSUM ? group_sum<L>(acc) : 0u;
+  small_hdr_finish<L>(sh, slot, gl, hf, psum, live);
+}
+
+// Every frame of the call is short.
+template <int L, bool FULL_CSUM>
+__global__ __launch_bounds__(kBlock) void k_scatter_small(ScatterArgs a)
+{
+  scatter_small_wave<L, FULL_CSUM>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
 }
 
 // ---------------------------------------------------------------------------
@@ -1128,25 +1420,30 @@ __device__ __forceinline__ unsigned long long ra_key(const unsigned long long *p
 
 // Find or claim the cell of `token`.  The whole bucket is read first: the
 // request may sit behind cells that have emptied since it came in.  Only then
-// is the lowest empty cell claimed; a thread walking the bucket tries every
-// empty cell it meets, so two threads that bring the same new token end up in
-// the same cell whatever else is claimed around them.
+// is an empty cell claimed, walking up from the lowest one seen empty and
+// trying every empty cell on the way; cells below that one were taken when
+// they were read and stay taken while arrivals are being filed, so two threads
+// that bring the same new token end up in the same cell whatever else is
+// claimed around them.
 __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long long token, bool *claimed)
 {
   const uint32_t b = (ra_hash(token) & a.bmask) * kRaBucket;
   *claimed = false;
+  uint32_t first_empty = kRaBucket;
 #pragma unroll 1
   for (uint32_t h = 0; h < kRaBucket; h += 16) {
     unsigned long long k[16];
 #pragma unroll
     for (int j = 0; j < 16; j++) k[j] = ra_key(a.keys + b + h + j);
 #pragma unroll
-    for (int j = 0; j < 16; j++)
+    for (int j = 0; j < 16; j++) {
       if (k[j] == token) return b + h + j;
+      if (k[j] == 0ull && first_empty == kRaBucket) first_empty = h + j;
+    }
   }
 #pragma unroll 1
-  for (uint32_t j = 0; j < kRaBucket; j++) {
-    unsigned long long k = ra_key(a.keys + b + j);
+  for (uint32_t j = first_empty; j < kRaBucket; j++) {
+    unsigned long long k = j == first_empty ? 0ull : ra_key(a.keys + b + j);
     if (k == 0ull) {
       k = atomicCAS(&a.keys[b + j], 0ull, token);
       if (k == 0ull) {
@@ -1159,29 +1456,32 @@ __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long 
   return kRaNoCell;  // bucket full
 }
 
-// A record off the free ring, or kRaNoRec.  The tail does not move during the
-// kernel that takes records (returns happen in k_ra_emit), so the head may
-// advance up to the tail read here; the compare-and-swap never takes a record
-// that is not there.
-__device__ __forceinline__ uint32_t ra_take_record(const RaArgs &a)
+// Records for the cells the lanes of this wavefront have just claimed: one
+// addition to the ring's head for the whole wavefront (an addition per claim, let
+// alone a compare-and-swap loop, would queue every new request of a burst on
+// one word).  The tail does not move during the kernel that takes records
+// (returns happen in k_ra_emit), so a position at or beyond the tail read here
+// means the pool is exhausted: the cell then gets no record, the call is
+// refused, and k_ra_scan puts the head back to the tail.
+__device__ __forceinline__ void ra_open_cells(const RaArgs &a, bool claimed, uint32_t cell, uint32_t lane)
 {
-  const uint32_t tail = a.words[kRaTail];
-  uint32_t h = __hip_atomic_load(&a.words[kRaHead], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  while ((int32_t)(tail - h) > 0) {
-    const uint32_t old = atomicCAS(&a.words[kRaHead], h, h + 1);
-    if (old == h) return a.free_ring[h & a.rmask];
-    h = old;  // somebody else took that one: progress was made
+  const unsigned long long cl = __ballot(claimed);
+  if (!cl) return;
+  const uint32_t n = (uint32_t)__popcll(cl);
+  const int leader = __ffsll((long long)cl) - 1;
+  uint32_t base = 0;
+  if ((int)lane == leader) {
+    base = atomicAdd(&a.words[kRaHead], n);
+    atomicAdd(&a.words[kRaClaims], n);
   }
-  return kRaNoRec;
-}
-
-// A newly claimed cell: take a record and stamp the cell.
-__device__ __forceinline__ void ra_open_cell(const RaArgs &a, uint32_t c)
-{
-  const uint32_t r = ra_take_record(a);
-  a.rec[c] = r;
-  atomicAdd(&a.words[kRaClaims], 1u);
-  if (r == kRaNoRec) refuse(a.status, a.status_flag, kStPoolFull);
+  base = (uint32_t)__shfl((int)base, leader, kWave);
+  if (claimed) {
+    const uint32_t h = base + (uint32_t)__popcll(cl & ((1ull << lane) - 1ull));
+    const uint32_t tail = a.words[kRaTail];
+    const uint32_t r = (int32_t)(tail - h) > 0 ? a.free_ring[h & a.rmask] : kRaNoRec;
+    a.rec[cell] = r;
+    if (r == kRaNoRec) refuse(a.status, a.status_flag, kStPoolFull);
+  }
 }
 
 // Fragments of one request tend to arrive together, so the lanes of a
@@ -1199,6 +1499,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
   const bool in_range = i < n;
   const uint32_t epoch = a.words[kRaEpoch];  // advanced by k_ra_scan, behind this kernel
   uint32_t cell = kRaNoCell, len = 0, fidx = 0, want = 0;
+  uint32_t opened = kRaNoCell;  // the cell this lane has claimed for a new request, if any
   unsigned long long token = 0;
   bool pending = false;
   if (in_range) {
@@ -1241,7 +1542,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
       bool claimed;
       c = ra_find_cell(a, t, &claimed);
       if (c != kRaNoCell) {
-        if (claimed) ra_open_cell(a, c);
+        if (claimed) opened = c;
         atomicAdd(&a.cnt[c], (uint32_t)__popcll(group));
         atomicAdd(&a.bytes[c], (unsigned long long)g_bytes);
         atomicMax(&a.last[c], i - lane + (63u - (uint32_t)__clzll((long long)group)));
@@ -1259,7 +1560,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
     bool claimed;
     cell = ra_find_cell(a, token, &claimed);
     if (cell != kRaNoCell) {
-      if (claimed) ra_open_cell(a, cell);
+      if (claimed) opened = cell;
       atomicAdd(&a.cnt[cell], 1u);
       atomicAdd(&a.bytes[cell], (unsigned long long)len);
       atomicMax(&a.last[cell], i);
@@ -1267,6 +1568,8 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
       a.seen[cell] = epoch;
     }
   }
+  // the cells this wavefront has claimed get their records (a lane claims one cell at most)
+  ra_open_cells(a, opened != kRaNoCell, opened, lane);
   if (in_range) {
     a.arr_cell[i] = cell;
     a.arr_len[i] = len;
@@ -1337,6 +1640,8 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
       n_req = n_frag = 0;
     }
     a.words[kRaOverflow] = overflow;
+    // claims beyond the pool ran the head past the tail
+    if ((int32_t)(a.words[kRaHead] - a.words[kRaTail]) > 0) a.words[kRaHead] = a.words[kRaTail];
     a.req_first[n_req] = n_frag;
     const uint32_t in_flight = a.words[kRaInFlight] + a.words[kRaClaims] - n_req;
     const uint32_t dropped = a.words[kRaDropped];
@@ -1374,9 +1679,52 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
     if (cell != kRaNoCell && !completes) a.last[cell] = 0;
   }
   unsigned long long todo = __ballot(completes);
+  // reap_rr for all of this wavefront's requests: one addition to the ring's tail
+  uint32_t tail0 = 0;
+  if (todo) {
+    if (lane == 0) tail0 = atomicAdd(&a.words[kRaTail], (uint32_t)__popcll(todo));
+    tail0 = (uint32_t)__shfl((int)tail0, 0, kWave);
+  }
+  // requests of a few fragments are handed over by the completing lane itself, all such lanes
+  // at once; the wavefront then walks the larger ones together
+  constexpr uint32_t kOwn = 8;
+  const uint32_t my_rank = (uint32_t)__popcll(todo & ((1ull << lane) - 1ull));
+  bool own = false;
+  if (completes) {
+    const uint32_t cnt = a.cnt[cell];
+    own = cnt <= kOwn;
+    if (own) {
+      const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v, rc = a.rec[cell];
+      unsigned long long *t = a.tab + (size_t)rc * SG_MAX_BI_SIZE;
+      unsigned long long e[kOwn];
+#pragma unroll
+      for (uint32_t j = 0; j < kOwn; j++) e[j] = j < cnt ? t[j] : 0ull;
+#pragma unroll
+      for (uint32_t j = 0; j < kOwn; j++) {
+        if (j < cnt) {
+          a.frag_slot[first + j] = (uint32_t)e[j];
+          a.frag_len[first + j] = (uint32_t)(e[j] >> 32);
+          t[j] = 0;
+        }
+      }
+      a.req_first[r] = first;
+      if (a.req_token) a.req_token[r] = a.keys[cell];
+      if (a.req_hdr_slot) a.req_hdr_slot[r] = (uint32_t)e[0];
+      a.free_ring[(tail0 + my_rank) & a.rmask] = rc;
+      a.cnt[cell] = 0;
+      a.bytes[cell] = 0;
+      a.last[cell] = 0;
+      a.want[cell] = 0;
+      a.rec[cell] = kRaNoRec;
+      __hip_atomic_store(&a.keys[cell], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  const unsigned long long all_done = todo;
+  todo &= ~__ballot(own);
   while (todo) {
     const int l = __ffsll((long long)todo) - 1;
     todo &= todo - 1;
+    const uint32_t nth = (uint32_t)__popcll(all_done & ((1ull << l) - 1ull));
     const uint32_t c = (uint32_t)__shfl((int)cell, l, kWave);
     const uint32_t r = (uint32_t)__shfl((int)(uint32_t)(v >> 32), l, kWave);
     const uint32_t first = (uint32_t)__shfl((int)(uint32_t)v, l, kWave);
@@ -1394,9 +1742,8 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
       }
     }
     if (lane == 0) {
-      // reap_rr: the record goes back to the free ring, the token leaves the table
-      const uint32_t tl = atomicAdd(&a.words[kRaTail], 1u);
-      a.free_ring[tl & a.rmask] = rc;
+      // the record goes back to the free ring, the token leaves the table
+      a.free_ring[(tail0 + nth) & a.rmask] = rc;
       a.cnt[c] = 0;
       a.bytes[c] = 0;
       a.last[c] = 0;
@@ -1736,6 +2083,34 @@ static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
   while ((1ull << l) < d) l++;
   *shift = 27 + l;
   *mul = (uint32_t)(((1ull << *shift) + d - 1) / d);
+}
+
+// Lanes a short frame of at most `bytes` payload bytes is given (two steps of L - 1
+// chunks without looping), or 0 where a whole wavefront per frame is the better deal.
+static uint32_t small_lanes(uint64_t bytes)
+{
+  if (bytes <= 2 * 15 * 16) return 16;
+  if (bytes <= 2 * 31 * 16) return 32;
+  return 0;
+}
+
+// Remainder fragments get wavefronts of their own kind when they are a good share of the
+// call's wavefronts -- and, where that takes a launch of its own (scatter), when the call is
+// large enough to hide one more launch.
+static bool small_last_pays(uint64_t per_req, uint32_t n_req, uint32_t flags, bool own_launch)
+{
+  if (per_req < 2) return false;
+  return (flags & SG_F_FORCE_SMALL) || (per_req <= 8 && (!own_launch || n_req >= 1024));
+}
+
+static void launch_scatter_small(hipStream_t st, const ScatterArgs &sa, uint32_t lanes, uint32_t n_frames, bool full_csum)
+{
+  const uint32_t per_wave = kWave / lanes;
+  const uint32_t grid = (n_frames + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
+  if (lanes == 16 && full_csum) k_scatter_small<16, true><<<grid, kBlock, 0, st>>>(sa);
+  else if (lanes == 16) k_scatter_small<16, false><<<grid, kBlock, 0, st>>>(sa);
+  else if (full_csum) k_scatter_small<32, true><<<grid, kBlock, 0, st>>>(sa);
+  else k_scatter_small<32, false><<<grid, kBlock, 0, st>>>(sa);
 }
 
 template <bool FUSED>
@@ -2080,6 +2455,17 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     ga.counts = a->counts;
     ga.per_req = (uint32_t)per;
     magic_div(per, &ga.div_mul, &ga.div_shift);
+    // short fragments go several to a wavefront: all of them where a full fragment is short, else
+    // the remainder fragment that ends every request
+    const uint64_t full_frag = a->fixed_req_size < a->mtu ? a->fixed_req_size : a->mtu;
+    const uint64_t last_frag = a->fixed_req_size - (per - 1) * a->mtu;
+    uint32_t small_all = 0, small_last = 0;
+    if (!(a->flags & SG_F_NO_SMALL)) {
+      small_all = small_lanes(full_frag);
+      if (!small_all && last_frag < a->mtu && small_last_pays(per, a->n_req, a->flags, false)) small_last = small_lanes(last_frag);
+    }
+    ga.per_launch = small_last ? (uint32_t)per - 1 : (uint32_t)per;
+    magic_div(ga.per_launch, &ga.lmul, &ga.lshift);
     ga.mtu = a->mtu;
     ga.slot_size = a->ring.slot_size;
     ga.hl = hl0;
@@ -2093,14 +2479,36 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     ga.app = app;
     ga.pieces = pieces_for(a->mtu);
     uint32_t grid, remap;
-    geometry((uint64_t)n_items * ga.pieces, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
+    uint64_t waves = (uint64_t)a->n_req * ga.per_launch * ga.pieces;
+    if (small_last) {
+      // turns of `period` wavefronts: the full fragments of 64 / small_last requests, then their remainders
+      const uint32_t per_turn = kWave / small_last;
+      ga.period = ga.per_launch * ga.pieces * per_turn + 1;
+      magic_div(ga.period, &ga.pmul, &ga.pshift);
+      waves = (uint64_t)((a->n_req + per_turn - 1) / per_turn) * ga.period;
+      if (waves >= (1u << 27)) return fail(c, SG_E_INVAL, "%llu wavefronts in one call: the limit is 2^27 - 1", (unsigned long long)waves);
+    }
+    geometry(waves, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
-              (app.n_tensors > 1 ? kOptMultiTensor : 0u) |
+              (app.n_tensors > 1 ? kOptMultiTensor : 0u) | (small_last ? kOptSmallLast : 0u) |
               ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    if (ga.pieces > 1) k_gather_rule<true><<<grid, kBlock, 0, st>>>(ga);
-    else k_gather_rule<false><<<grid, kBlock, 0, st>>>(ga);
+    if (small_all) {
+      const uint32_t per_wave = kWave / small_all;
+      const uint32_t sgrid = (n_items + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
+      if (small_all == 16) k_gather_small<16><<<sgrid, kBlock, 0, st>>>(ga);
+      else k_gather_small<32><<<sgrid, kBlock, 0, st>>>(ga);
+    } else if (small_last == 16) {
+      if (ga.pieces > 1) k_gather_rule<true, 16><<<grid, kBlock, 0, st>>>(ga);
+      else k_gather_rule<false, 16><<<grid, kBlock, 0, st>>>(ga);
+    } else if (small_last == 32) {
+      if (ga.pieces > 1) k_gather_rule<true, 32><<<grid, kBlock, 0, st>>>(ga);
+      else k_gather_rule<false, 32><<<grid, kBlock, 0, st>>>(ga);
+    } else {
+      if (ga.pieces > 1) k_gather_rule<true, 0><<<grid, kBlock, 0, st>>>(ga);
+      else k_gather_rule<false, 0><<<grid, kBlock, 0, st>>>(ga);
+    }
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
     launch_finish(sc, st, packed ? sc.cursor[0] : nullptr, a->fixed_req_size, app.cap, a->n_req, a->counts,
@@ -2236,6 +2644,9 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.rule.size = a->fixed_resp_size;
     sa.rule.mtu = a->mtu;
     sa.rule.per_req = (uint32_t)per;
+    sa.rule.per_launch = (uint32_t)per;
+    magic_div(per, &sa.rule.div_mul, &sa.rule.div_shift);
+    if (n_items >= (1u << 27)) return fail(c, SG_E_INVAL, "%u frames in one call: the limit is 2^27 - 1", n_items);
     sa.rule.n_req = a->n_req;
     sa.rule.n_slots = a->tx.n_slots;
     sa.rule.single_wrap = app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_resp_size <= app.cap;
@@ -2243,11 +2654,28 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.rule.offsets_out = packed ? a->offsets_out : nullptr;
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
-    geometry((uint64_t)n_items * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
-             !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+    // short frames go several to a wavefront: all of them where a full frame is short, else the
+    // remainder frame that ends every response
+    const bool full_csum = (a->flags & SG_F_UDP_CSUM_FULL) != 0;
+    const uint64_t full_frame = a->fixed_resp_size < a->mtu ? a->fixed_resp_size : a->mtu;
+    const uint64_t last_frame = a->fixed_resp_size - (per - 1) * a->mtu;
+    uint32_t small_all = 0, small_last = 0;
+    if (!(a->flags & SG_F_NO_SMALL)) {
+      small_all = small_lanes(full_frame);
+      if (!small_all && last_frame < a->mtu && small_last_pays(per, a->n_req, a->flags, true)) small_last = small_lanes(last_frame);
+    }
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    launch_scatter<true>(st, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
+    if (small_all) {
+      launch_scatter_small(st, sa, small_all, n_items, full_csum);
+    } else {
+      if (small_last) sa.rule.per_launch = (uint32_t)per - 1;
+      magic_div(sa.rule.per_launch, &sa.rule.lmul, &sa.rule.lshift);
+      geometry((uint64_t)a->n_req * sa.rule.per_launch * (full_csum ? 1u : sa.pieces), !(a->flags & SG_F_NO_XCD_REMAP),
+               &grid, &sa.remap);
+      launch_scatter<true>(st, sa, grid, full_csum);
+      if (small_last) launch_scatter_small(st, sa, small_last, a->n_req, full_csum);
+    }
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
     launch_finish(sc, st, packed ? sc.cursor[1] : nullptr, a->fixed_resp_size, app.cap, a->n_req, a->counts,
