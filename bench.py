@@ -94,7 +94,8 @@ class Pool:
     def step(self, ctx, i: int, flags: int) -> None:
         dw = self.items[i % len(self.items)]
         dw.gather(ctx, flags | self.extra_flags, rule=self.rule)
-        dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule)
+        # an echo answered in place (the mixed workload) takes the descriptors its gather just built
+        dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule, reuse=True)
 
 
 def timed(ctx, pool: Pool, steps: int, warmup: int):

@@ -68,6 +68,15 @@ extern "C" {
                                           destination bytes are then undefined). */
 #define SG_F_NO_FUSE (1u << 5)          /* scatter: run the descriptor pass even where the copy
                                           kernel could derive the descriptors (for experiments) */
+#define SG_F_REUSE_DESC (1u << 6)       /* scatter: the frames of this call are the fragments the latest
+                                          gather call with a descriptor pass on this context described --
+                                          same slots (tx_slot == its frag_slot), same lengths, same
+                                          requests in the same arena (an echo, answered in place or not):
+                                          its descriptors and arena offsets are used as they stand and no
+                                          descriptor pass runs.  Held against that pass's counts; a call
+                                          that does not match is refused with SG_E_DATA.  resp_size is
+                                          not read; the response cursor ends up where the request cursor
+                                          did */
 #define SG_F_ASYNC (1u << 16)          /* enqueue only; completion through sg_hip_sync() */
 #define SG_F_NO_XCD_REMAP (1u << 17)   /* launch-order = item order (for experiments) */
 #define SG_F_NO_SMALL (1u << 18)       /* one wavefront per frame even for short frames (for experiments) */

@@ -27,6 +27,7 @@ F_UDP_CSUM_FULL = 1 << 2
 F_REF_QUIRKS = 1 << 3
 F_RULE_FRAGS = 1 << 4
 F_NO_FUSE = 1 << 5
+F_REUSE_DESC = 1 << 6
 F_ASYNC = 1 << 16
 F_NO_XCD_REMAP = 1 << 17
 F_NO_SMALL = 1 << 18

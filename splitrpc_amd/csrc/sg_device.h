@@ -368,8 +368,11 @@ __device__ __forceinline__ uint32_t hdr_fetch(const uint8_t *__restrict__ in, ui
 
 // Returns the final value of header byte `lane` (garbage on lanes >= hl) from
 // the fetched byte.
+// With l4_partial the finished UDP checksum is somebody else's business (the
+// payload's sum is not known yet): the field is left zero and *l4_partial gets
+// the sum of everything but the payload, unfolded.
 __device__ __forceinline__ uint32_t hdr_finish(uint32_t b, uint32_t lane, const HdrFields &f,
-                                               uint32_t payload_sum)
+                                               uint32_t payload_sum, uint32_t *l4_partial = nullptr)
 {
   const uint32_t j = lane;
   const bool live = j < f.hl;
@@ -413,9 +416,14 @@ __device__ __forceinline__ uint32_t hdr_finish(uint32_t b, uint32_t lane, const 
     if (f.flags & (1u << 2)) {  // finished UDP checksum
       const uint32_t s_l4 = wave_sum(((j >= 34 && j < 40) || (j >= 42 && j < f.hl)) ? w : 0u);
       uint32_t s = s_addr + (proto << 8) + (((ulen & 0xffu) << 8) | (ulen >> 8)) + s_l4;
-      s = fold16(fold16(s) + fold16(payload_sum));
-      uint32_t c = (~s) & 0xffffu;
-      if (c == 0) c = 0xffffu;
+      uint32_t c = 0;
+      if (l4_partial) {
+        *l4_partial = s;
+      } else {
+        s = fold16(fold16(s) + fold16(payload_sum));
+        c = (~s) & 0xffffu;
+        if (c == 0) c = 0xffffu;
+      }
       if (j == 40) b = c & 0xffu;
       if (j == 41) b = c >> 8;
     }

@@ -100,6 +100,10 @@ struct PrepArgs {
   // [1] items.  n_req and n_items above are then upper bounds the launch was
   // sized with.  nullptr: the bounds are the counts.
   const uint32_t *counts;
+  // What this pass leaves for a later call that wants to reuse its descriptors
+  // (SG_F_REUSE_DESC): desc_tag = {gen, requests, items}.
+  uint32_t *desc_tag;
+  uint32_t gen;
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
@@ -223,6 +227,11 @@ __device__ __forceinline__ void prep_finish(const PrepArgs &a, uint32_t r, uint6
   if (a.mode == 0 && a.fixed_size && total != a.fixed_size) bad |= kStBadSize;
   if (bad) refuse(a.status, a.status_flag, bad);
   a.req_size[r] = total;
+  if (r == 0 && a.desc_tag) {
+    a.desc_tag[0] = a.gen;
+    a.desc_tag[1] = a.n_req;
+    a.desc_tag[2] = a.n_items;
+  }
   if (a.packed && a.fixed_offsets) {
     // bump ring with equal sizes: ret = base + off; off = (off + size) % capacity
     const uint64_t c0 = *a.cursor % a.cap;
@@ -1036,6 +1045,17 @@ struct ScatterArgs {
   const uint64_t *next_cursor;
   const uint32_t *hdr_src_req;  // one header source per request instead of hdr_src_slot per frame
   const uint32_t *counts;       // device-resident request count, or nullptr
+  // full UDP checksum of long frames in two phases: every sub-run's wavefront leaves the sum of
+  // its bytes in csum_part[frame * kPartStride + piece], wavefront 0 of a frame also the header's
+  // share at [.. + pieces] and a mark in csum_valid[frame]; k_udp_finish folds them into the field
+  uint32_t *csum_part;
+  uint32_t *csum_valid;
+  // SG_F_REUSE_DESC: the descriptors and offsets are those an earlier descriptor pass left (tagged
+  // reuse_gen); they are held against the tag and the TX ring, and offsets_out is written from them
+  const uint32_t *desc_tag;
+  uint32_t reuse_gen;
+  uint32_t tx_n_slots;
+  uint64_t *offsets_out;
   RuleArgs rule;
   AppDev app;
 };
@@ -1047,11 +1067,16 @@ struct ScatterArgs {
 // measured slower: 3 at a time +1 %, 5 at a time +8 %).  (Summing per piece and combining with one returning atomic
 // per wavefront was measured: the atomic's round trip at the end of every
 // wavefront's life cost more than the shorter tail gained.)
-template <bool FULL_CSUM, bool FUSED, bool LONG>
+constexpr uint32_t kPartStride = 8;  // words of csum_part per frame: up to 7 sub-runs and the header's share
+
+// DEFER (long frames with the full UDP checksum): the frame's sub-runs go to
+// several wavefronts all the same, each leaving the sum of its bytes behind,
+// and k_udp_finish writes the checksum field afterwards.
+template <bool FULL_CSUM, bool FUSED, bool LONG, bool DEFER = false>
 __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
-  constexpr bool SPLIT = LONG && !FULL_CSUM;  // several wavefronts per frame
-  constexpr bool WHOLE_LONG = LONG && FULL_CSUM;  // one wavefront walks all sub-runs of its frame
+  constexpr bool SPLIT = LONG && (!FULL_CSUM || DEFER);      // several wavefronts per frame
+  constexpr bool WHOLE_LONG = LONG && FULL_CSUM && !DEFER;   // one wavefront walks all sub-runs of its frame
   // every argument of the common path in one burst of scalar loads
   const u32x4 *desc = a.desc;
   const uint64_t *req_off = a.req_off;
@@ -1081,8 +1106,18 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   const uint32_t pieces = SPLIT ? n_pieces : 1u;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   // descriptor path: this kernel does not read the cursor and commits what the descriptor pass left
-  if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts)))
-    *a.cursor = sload(a.next_cursor);
+  if (!FUSED && a.reuse_gen && n_req) {
+    // the caller says these are the items the tagged descriptor pass described
+    if (sload(a.desc_tag) != a.reuse_gen || sload(a.desc_tag + 1) != n_req || sload(a.desc_tag + 2) != n_items) {
+      if (w == 0 && lane == 0) refuse(a.status, a.status_flag, kStBadTable);
+      return;
+    }
+  }
+  if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts))) {
+    const uint64_t nc = sload(a.next_cursor);
+    *a.cursor = nc;
+    if (a.reuse_gen && a.offsets_out) a.offsets_out[n_req] = nc;
+  }
   uint32_t item = SPLIT ? w / pieces : w;
   const uint32_t piece = SPLIT ? w - item * pieces : 0;
   if (FUSED && a.rule.per_launch != a.rule.per_req) {
@@ -1109,6 +1144,13 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     f0 = sload(first + r);
     nf = sload(first + r + 1) - f0;
     ro = a.app.n_tensors == 0 ? sload(req_off + r) : 0;
+    if (a.reuse_gen) {
+      if (d[0] >= a.tx_n_slots) {  // described for another ring
+        if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
+        return;
+      }
+      if (a.offsets_out && item == f0 && lane == 0 && piece == 0) a.offsets_out[r] = ro;
+    }
   } else {
     uint32_t slot_i, len, off, i;
     const uint32_t bad = rule_desc(a.rule, a.app, item, n_items, n_req, piece == 0 ? lane : 1u, &slot_i, &len,
@@ -1137,7 +1179,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     if (hdr_src_req) hs = sload(hdr_src_req + r);
     if (hs >= rx_n_slots) {
       // descriptor path: the descriptor pass has refused the batch already and nothing gets here
-      if (FUSED && lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
+      // (unless its descriptors are being reused: no pass has seen this call's header sources)
+      if ((FUSED || a.reuse_gen) && lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
       return;
     }
     hin = rx + (size_t)hs * rx_slot_size;
@@ -1146,10 +1189,15 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   if (SPLIT && piece != 0) {
     // a later piece of a long frame: payload only
     uint8_t *from;
+    uint32_t part = 0;
     if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
       uint32_t o, n;
       sub_run(slot + hl, d[1], piece, &o, &n);
-      if (n) copy_run<false>(from + o, slot + hl + o, n, lane);
+      if (n) part = copy_run<DEFER>(from + o, slot + hl + o, n, lane);
+    }
+    if (DEFER) {
+      part = wave_sum(part);
+      if (lane == 0) a.csum_part[(size_t)item * kPartStride + piece] = part;
     }
     return;
   }
@@ -1175,10 +1223,48 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   } else if (d[1]) {
     acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + hl, d[1], lane);
   }
-  if (FULL_CSUM) hb = hdr_finish(raw, lane, hf, wave_sum(acc));
+  if (FULL_CSUM && !DEFER) hb = hdr_finish(raw, lane, hf, wave_sum(acc));
+  if (DEFER) {
+    uint32_t l4 = 0;
+    hb = hdr_finish(raw, lane, hf, 0, &l4);
+    const uint32_t part = wave_sum(acc);
+    if (lane == 0) {
+      a.csum_part[(size_t)item * kPartStride] = part;
+      a.csum_part[(size_t)item * kPartStride + n_pieces] = l4;
+      a.csum_valid[item] = 1u;  // this frame was written: its checksum field is to be finished
+    }
+  }
   // the payload went past the header only, so a TX slot that is the header's own
   // source still held the request header when it was fetched above
   if (lane < hl) slot[lane] = (uint8_t)hb;
+}
+
+// Second phase of the full UDP checksum of long frames: one thread per frame
+// folds the sums its wavefronts left and writes the field (bytes 40, 41).
+// Frames that were not written (refused) carry no mark and are left alone;
+// marks are taken down for the next call.
+template <bool FUSED>
+__global__ __launch_bounds__(kBlock) void k_udp_finish(ScatterArgs a)
+{
+  const uint32_t item = blockIdx.x * kBlock + threadIdx.x;
+  uint32_t n_items = a.n_items;
+  if (a.counts) {
+    const uint32_t n_req = dev_count(a.counts, 0, a.n_req);
+    const uint32_t live = FUSED ? n_req * a.rule.per_req : (n_req ? a.first[n_req] : 0u);
+    n_items = live < n_items ? live : n_items;
+  }
+  if (item >= n_items) return;
+  if (!a.csum_valid[item]) return;
+  a.csum_valid[item] = 0;
+  const uint32_t *p = a.csum_part + (size_t)item * kPartStride;
+  uint32_t sum = 0;
+  for (uint32_t k = 0; k < a.pieces; k++) sum += p[k];  // each below 2^27
+  uint32_t s = fold16(fold16(p[a.pieces]) + fold16(sum));
+  uint32_t c = (~s) & 0xffffu;
+  if (c == 0) c = 0xffffu;
+  const uint32_t slot = FUSED ? a.rule.item_slot[item] : a.desc[item][0];
+  // slots start at even addresses; the sums ran over the words as they lie in memory
+  *reinterpret_cast<uint16_t *>(a.tx + (size_t)slot * a.tx_slot_size + 40) = (uint16_t)c;
 }
 
 // Scatter of SHORT frames, 64 / L frames per wavefront (L = 16 or 32 lanes per
@@ -1849,6 +1935,10 @@ struct Scratch {
   uint64_t *cursor[2] = {nullptr, nullptr};
   uint64_t *next_cursor[2] = {nullptr, nullptr};
   uint32_t *slot_idx[2] = {nullptr, nullptr};  // next slot of the application ring to fill / to serve
+  uint32_t *desc_tag = nullptr;    // {generation, requests, items} of the descriptors in `desc`
+  uint32_t *desc_gen = nullptr;    // host counter behind the generation (one per scratch)
+  uint32_t *csum_part = nullptr;   // kPartStride words per frame (two-phase UDP checksum of long frames)
+  uint32_t *csum_valid = nullptr;  // one mark per frame, zero between calls
   uint32_t *status = nullptr;
   volatile uint32_t *flag = nullptr;  // raised with every refusal (pinned host memory in a context)
 };
@@ -1865,6 +1955,8 @@ struct sg_hip_ctx {
   uint64_t *tile_tot = nullptr;  // one total per 4096 requests, for the tiled request scan
   // [0] request-arena cursor, [1] response-arena cursor, [2], [3] their staged successors
   uint64_t *cursors = nullptr;
+  uint32_t *csum_scratch = nullptr;  // csum_part and csum_valid
+  uint32_t desc_gen = 0;
   uint32_t *status = nullptr;
   Scratch sc;
   // pinned staging for the per-request entry points (device reads it in place)
@@ -2113,11 +2205,21 @@ static void launch_scatter_small(hipStream_t st, const ScatterArgs &sa, uint32_t
   else k_scatter_small<32, false><<<grid, kBlock, 0, st>>>(sa);
 }
 
+// Long frames with the full UDP checksum go to several wavefronts per frame when the
+// scratch has room for their sums (k_scatter<.., DEFER> + k_udp_finish).
+static bool csum_in_two_phases(const Scratch &sc, uint32_t pieces, bool full_csum)
+{
+  return full_csum && pieces > 1 && pieces + 1 <= kPartStride && sc.csum_part != nullptr;
+}
+
 template <bool FUSED>
-static void launch_scatter(hipStream_t st, const ScatterArgs &sa, uint32_t grid, bool full_csum)
+static void launch_scatter(hipStream_t st, const ScatterArgs &sa, uint32_t grid, bool full_csum, bool defer = false)
 {
   const bool lng = sa.pieces > 1;
-  if (full_csum && lng) k_scatter<true, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
+  if (defer) {
+    k_scatter<true, FUSED, true, true><<<grid, kBlock, 0, st>>>(sa);
+    k_udp_finish<FUSED><<<(sa.n_items + kBlock - 1) / kBlock, kBlock, 0, st>>>(sa);
+  } else if (full_csum && lng) k_scatter<true, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
   else if (full_csum) k_scatter<true, FUSED, false><<<grid, kBlock, 0, st>>>(sa);
   else if (lng) k_scatter<false, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
   else k_scatter<false, FUSED, false><<<grid, kBlock, 0, st>>>(sa);
@@ -2156,9 +2258,11 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->tile_tot, sizeof(uint64_t) * ((size_t)c->max_reqs / kScanTile + 2)));
-  HIP_TRY(nullptr, hipMalloc(&c->cursors, 5 * sizeof(uint64_t)));  // [4]: the two slot indices
+  HIP_TRY(nullptr, hipMalloc(&c->cursors, 7 * sizeof(uint64_t)));  // [4]: the two slot indices, [5], [6]: descriptor tag
   HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
-  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 5 * sizeof(uint64_t), c->stream));
+  HIP_TRY(nullptr, hipMalloc(&c->csum_scratch, sizeof(uint32_t) * (size_t)c->max_frames * (kPartStride + 1)));
+  HIP_TRY(nullptr, hipMemsetAsync(c->csum_scratch, 0, sizeof(uint32_t) * (size_t)c->max_frames * (kPartStride + 1), c->stream));
+  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 7 * sizeof(uint64_t), c->stream));
   HIP_TRY(nullptr, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
   c->h_runs_cap = 8192;
   HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
@@ -2180,6 +2284,10 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   sc.next_cursor[1] = c->cursors + 3;
   sc.slot_idx[0] = reinterpret_cast<uint32_t *>(c->cursors + 4);
   sc.slot_idx[1] = sc.slot_idx[0] + 1;
+  sc.desc_tag = reinterpret_cast<uint32_t *>(c->cursors + 5);
+  sc.desc_gen = &c->desc_gen;
+  sc.csum_part = c->csum_scratch;
+  sc.csum_valid = c->csum_scratch + (size_t)c->max_frames * kPartStride;
   sc.status = c->status;
   sc.flag = c->h_flag;
   return SG_OK;
@@ -2216,6 +2324,7 @@ void sg_hip_destroy(sg_hip_ctx *c)
   (void)hipFree(c->req_off);
   (void)hipFree(c->tile_tot);
   (void)hipFree(c->cursors);
+  (void)hipFree(c->csum_scratch);
   (void)hipFree(c->status);
   if (c->h_runs) (void)hipHostFree(c->h_runs);
   if (c->h_ptrs) (void)hipHostFree(c->h_ptrs);
@@ -2540,6 +2649,10 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
   p.next_cursor = sc.next_cursor[0];
   p.offsets_out = packed ? a->offsets_out : nullptr;
   p.counts = a->counts;
+  if (sc.desc_gen) {
+    p.desc_tag = sc.desc_tag;
+    p.gen = ++*sc.desc_gen ? *sc.desc_gen : ++*sc.desc_gen;  // never zero
+  }
   p.status = sc.status;
   p.status_flag = sc.flag;
   rc = launch_prep(c, sc, st, p);
@@ -2609,7 +2722,10 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
   if (a->slot_state && a->n_req > a->n_slot_states)
     return fail(c, SG_E_INVAL, "%u responses do not fit a ring of %u application slots", a->n_req, a->n_slot_states);
 
-  const bool fused = a->resp_size == nullptr && !(a->flags & SG_F_NO_FUSE);
+  const bool reuse = (a->flags & SG_F_REUSE_DESC) != 0;
+  if (reuse && (!packed || !sc.desc_gen || !*sc.desc_gen))
+    return fail(c, SG_E_INVAL, "SG_F_REUSE_DESC needs a packed arena and a descriptor pass of an earlier call on this context");
+  const bool fused = a->resp_size == nullptr && !(a->flags & (SG_F_NO_FUSE | SG_F_REUSE_DESC));
   if (fused) {
     if (a->fixed_resp_size == 0 || a->fixed_resp_size > 0xffffffffull)
       return fail(c, SG_E_INVAL, "fixed response size %llu out of range", (unsigned long long)a->fixed_resp_size);
@@ -2671,9 +2787,12 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     } else {
       if (small_last) sa.rule.per_launch = (uint32_t)per - 1;
       magic_div(sa.rule.per_launch, &sa.rule.lmul, &sa.rule.lshift);
-      geometry((uint64_t)a->n_req * sa.rule.per_launch * (full_csum ? 1u : sa.pieces), !(a->flags & SG_F_NO_XCD_REMAP),
-               &grid, &sa.remap);
-      launch_scatter<true>(st, sa, grid, full_csum);
+      const bool defer = csum_in_two_phases(sc, sa.pieces, full_csum);
+      sa.csum_part = sc.csum_part;
+      sa.csum_valid = sc.csum_valid;
+      geometry((uint64_t)a->n_req * sa.rule.per_launch * ((full_csum && !defer) ? 1u : sa.pieces),
+               !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+      launch_scatter<true>(st, sa, grid, full_csum, defer);
       if (small_last) launch_scatter_small(st, sa, small_last, a->n_req, full_csum);
     }
     rc = prof_end(c);
@@ -2712,10 +2831,16 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     p.rx_n_slots = a->rx.n_slots;
   }
   p.counts = a->counts;
+  if (sc.desc_gen && !reuse) {
+    p.desc_tag = sc.desc_tag;
+    p.gen = ++*sc.desc_gen ? *sc.desc_gen : ++*sc.desc_gen;
+  }
   p.status = sc.status;
   p.status_flag = sc.flag;
-  rc = launch_prep(c, sc, st, p);
-  if (rc != SG_OK) return rc;
+  if (!reuse) {
+    rc = launch_prep(c, sc, st, p);
+    if (rc != SG_OK) return rc;
+  }
 
   if (a->n_frames || packed) {
     ScatterArgs sa;
@@ -2744,14 +2869,26 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
       sa.cursor = sc.cursor[1];
       sa.next_cursor = sc.next_cursor[1];
     }
+    if (reuse) {
+      // the response cursor ends up where the reused descriptors end
+      sa.next_cursor = sc.next_cursor[0];
+      sa.desc_tag = sc.desc_tag;
+      sa.reuse_gen = *sc.desc_gen;
+      sa.tx_n_slots = a->tx.n_slots;
+      sa.offsets_out = a->offsets_out;
+    }
     sa.app = app;
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
-    geometry((uint64_t)(a->n_frames ? a->n_frames : 1u) * ((a->flags & SG_F_UDP_CSUM_FULL) ? 1u : sa.pieces),
+    const bool full_csum = (a->flags & SG_F_UDP_CSUM_FULL) != 0;
+    const bool defer = csum_in_two_phases(sc, sa.pieces, full_csum);
+    sa.csum_part = sc.csum_part;
+    sa.csum_valid = sc.csum_valid;
+    geometry((uint64_t)(a->n_frames ? a->n_frames : 1u) * ((full_csum && !defer) ? 1u : sa.pieces),
              !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
-    launch_scatter<false>(st, sa, grid, (a->flags & SG_F_UDP_CSUM_FULL) != 0);
+    launch_scatter<false>(st, sa, grid, full_csum, defer);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
   }

@@ -425,14 +425,20 @@ class DeviceWorkload:
             a._base_flags = capi.F_RULE_FRAGS if (rule and fx) else 0
             self._args[key] = a
         a.flags = flags | a._base_flags
+        self._described = not (a._base_flags & capi.F_RULE_FRAGS)  # a descriptor pass ran
         ctx.gather_batch_raw(a)
 
     def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True,
-                templates: Optional[torch.Tensor] = None, tokens: Optional[torch.Tensor] = None) -> None:
+                templates: Optional[torch.Tensor] = None, tokens: Optional[torch.Tensor] = None,
+                reuse: bool = False) -> None:
         """``templates`` (n_req x 64 uint8 on the device) takes the frame
-        headers from connection templates instead of request headers."""
+        headers from connection templates instead of request headers.
+        ``reuse``: an echo answered in place right after this workload's gather
+        reuses that call's descriptors where it ran a descriptor pass."""
         if not fuse:
             flags |= capi.F_NO_FUSE
+        if reuse and self.w.tx_in_place and getattr(self, "_described", False):
+            flags |= capi.F_REUSE_DESC
         key = ("s", fixed)
         a = self._args.get(key)
         if a is not None:

@@ -615,3 +615,46 @@ def test_tiled_request_scan_beyond_8192_requests():
         exp[idx] = pay
         assert np.array_equal(got, exp), first_diff(got, exp)
     big.close()
+
+
+# ---------------------------------------------------------------- descriptors reused by the echo
+
+def test_echo_scatter_reuses_the_descriptors_of_its_gather(ctx):
+    """SG_F_REUSE_DESC: the in-place echo of variable-size requests runs no
+    descriptor pass of its own; same bytes, same offsets, same cursor as with
+    one.  A call that does not match what was described is refused."""
+    w = synth.make_workload(4, 300)
+    for reuse in (False, True):
+        dw = DeviceWorkload(w, arena_slack=4321)
+        start = dw.req_app.cap - 7000
+        ctx.set_cursor(0, start)
+        ctx.set_cursor(1, start)
+        dw.gather(ctx, fixed=False)
+        exp, offs, cur = expected_gather(w, arena_cap=dw.req_app.cap, cursor=start)
+        assert np.array_equal(dw.req_arena.cpu().numpy(), exp)
+        dw.scatter(ctx, fixed=False, reuse=reuse)
+        assert getattr(dw, "_described")
+        exp_tx, eoffs, ecur = expected_scatter(w, exp, resp_cap=dw.req_app.cap, cursor=start)
+        got = dw.ring.cpu().numpy()
+        assert np.array_equal(got, exp_tx), f"reuse={reuse}: " + first_diff(got, exp_tx)
+        assert np.array_equal(dw.resp_offsets.cpu().numpy().view(np.uint64), eoffs)
+        assert ctx.get_cursor(1) == ecur == cur
+    # fewer frames than were described: refused, nothing written
+    dw = DeviceWorkload(w)
+    ctx.set_cursor(0, 0)
+    dw.gather(ctx, fixed=False)
+    before = dw.ring.clone()
+    a = ctx.scatter_args(dw.rx, dw.tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first, None, 0, dw.n_req - 1,
+                         int(w.resp_first[-2]), w.mtu, dw.resp_app, None, w.flags | capi.F_REUSE_DESC)
+    with pytest.raises(SgError) as e:
+        ctx.scatter_batch_raw(a)
+    assert e.value.code == capi.SG_E_DATA
+    assert torch.equal(dw.ring, before)
+    # nothing described yet on a fresh context: refused by the host
+    fresh = SgContext(0)
+    a = ctx.scatter_args(dw.rx, dw.tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first, None, 0, dw.n_req, dw.n_frames,
+                         w.mtu, dw.resp_app, None, w.flags | capi.F_REUSE_DESC)
+    with pytest.raises(SgError) as e:
+        fresh.scatter_batch_raw(a)
+    assert e.value.code == capi.SG_E_INVAL
+    fresh.close()
