@@ -29,10 +29,19 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one launch of the dominant kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this file scaled by a plain 512 MiB copy in the same runs (FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000): 340.2 MB read + 308.3 MB written.  Known for the default call only.
-MEASURED_TRAFFIC = {(2, 32, "k_gather"): 652.2e6}
+# HBM bytes the copy kernels of one call move, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this file (--calib-copy --steps 40 --warmup 5), each counter scaled by what it reads for a plain
+# 512 MiB device copy in the same run (FETCH_SIZE x 2.000 KiB, WRITE_SIZE x 1.000 KiB).  Keyed by
+# (workload, batches per launch, kernel family); the default call: 340.5 MB read + 312.2 MB written.
+# bert's scatter is both of its kernels (full frames + short remainder frames), jumbo's the copy
+# phase without the 1.9 MB of the checksum-finishing kernel.
+MEASURED_TRAFFIC = {
+    (2, 32, "k_gather"): 652.7e6, (2, 32, "k_scatter"): 4.8e6,
+    (1, 2048, "k_gather"): 449.8e6, (1, 2048, "k_scatter"): 23.3e6,
+    (3, 512, "k_gather"): 582.5e6, (3, 512, "k_scatter"): 935.1e6,
+    (4, 8, "k_gather"): 661.7e6, (4, 8, "k_scatter"): 677.1e6,
+    (5, 4, "k_gather"): 817.2e6, (5, 4, "k_scatter"): 549.7e6,
+}
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 
@@ -66,6 +75,8 @@ def parse():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 512 MiB device copy a few times (a kernel of known "
                          "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="gather and scatter calls on one context and stream (default: one each)")
     ap.add_argument("--general", action="store_true",
                     help="always run the descriptor pass (do not declare the fragmenting rule)")
     return ap.parse_args()
@@ -91,28 +102,46 @@ class Pool:
         self.scatter_bytes = w.scatter_bytes() * bpl
         self.n_req = w.n_req * bpl
 
-    def step(self, ctx, i: int, flags: int) -> None:
+    def step(self, ctx, i: int, flags: int, ctx_tx=None) -> None:
+        """One pass of the hot path.  With ctx_tx the scatter call goes to a
+        second context on a stream of its own, as the reference keeps one copy
+        context (and stream) per direction (src/p2p_rpc_sg_engine.h:185-196);
+        an echo answered in place reads what its gather wrote and stays on one."""
         dw = self.items[i % len(self.items)]
         dw.gather(ctx, flags | self.extra_flags, rule=self.rule)
-        # an echo answered in place (the mixed workload) takes the descriptors its gather just built
-        dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule, reuse=True)
+        if ctx_tx is not None and not self.w.tx_in_place:
+            dw.scatter(ctx_tx, flags | self.extra_flags, fuse=self.rule)
+        else:
+            # an echo answered in place (the mixed workload) takes the descriptors its gather just built
+            dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule, reuse=True)
 
 
-def timed(ctx, pool: Pool, steps: int, warmup: int):
+def timed(ctx, pool: Pool, steps: int, warmup: int, ctx_tx=None, reps: int = 5):
+    """Seconds per step: `warmup` untimed steps, then `reps` timed runs of
+    exactly `steps` steps each, bracketed by synchronization on both sides; the
+    median run is reported (one run of 20 steps of 0.1 ms is a 2 ms sample)."""
     import torch
     from splitrpc_amd import capi
+
+    def drain():
+        ctx.sync()
+        if ctx_tx is not None:
+            ctx_tx.sync()
+        torch.cuda.synchronize()
+
     # every rotated copy is touched at least once before the clock starts
     for i in range(max(warmup, len(pool.items))):
-        pool.step(ctx, i, capi.F_ASYNC)
-    ctx.sync()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        pool.step(ctx, warmup + i, capi.F_ASYNC)
-    ctx.sync()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    return dt / steps
+        pool.step(ctx, i, capi.F_ASYNC, ctx_tx)
+    drain()
+    runs = []
+    for rep in range(reps):
+        t0 = time.perf_counter()
+        for i in range(steps):
+            pool.step(ctx, warmup + i, capi.F_ASYNC, ctx_tx)
+        drain()
+        runs.append((time.perf_counter() - t0) / steps)
+    runs.sort()
+    return runs[len(runs) // 2]
 
 
 def kernel_times(ctx, pool: Pool, steps: int):
@@ -241,37 +270,67 @@ def per_request_calls(ctx, dw, calls: int = 300):
             "GBps": round((2 * size + 16 * int(skbs[0].num_items)) / dt / 1e9, 2)}
 
 
-def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, replays: int = 50) -> float:
-    """Seconds per step of the single-batch call when `steps` steps (an even
-    number of calls per arena) are recorded into one HIP graph on the context's
-    stream and the graph is replayed: the launch-bound loop without the
-    per-launch host cost."""
+def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, replays: int = 50,
+                    streams: int = 1):
+    """Seconds per step of the single-batch call when `steps` steps are recorded
+    into one HIP graph per stream and the graphs are replayed: the launch-bound
+    loop without the per-launch host cost.  With `streams` > 1 that many
+    contexts, each with a stream, a graph and rings of its own, replay side by
+    side (several batch-sized calls in flight at once); the figure is then wall
+    time over ALL steps of all streams."""
     import torch
     from splitrpc_amd import capi
     from splitrpc_amd.engine import SgContext
-    stream = torch.cuda.Stream()
-    ctx = SgContext(0, max_reqs=max(4096, w.n_req), max_frames=max(65536, w.n_frags, w.n_resp_frames),
-                    stream=stream.cuda_stream)
-    pool = Pool(w, 1, rotate_mb, extra, rule=rule)
-    for i in range(len(pool.items)):
-        pool.step(ctx, i, capi.F_ASYNC)
-    ctx.sync()
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g, stream=stream):
-        for i in range(steps):
+    lanes = []
+    for _ in range(streams):
+        stream = torch.cuda.Stream()
+        ctx = SgContext(0, max_reqs=max(4096, w.n_req), max_frames=max(65536, w.n_frags, w.n_resp_frames),
+                        stream=stream.cuda_stream)
+        pool = Pool(w, 1, max(64, rotate_mb // streams), extra, rule=rule)
+        for i in range(len(pool.items)):
             pool.step(ctx, i, capi.F_ASYNC)
+        ctx.sync()
+        lanes.append((stream, ctx, pool))
+    torch.cuda.synchronize()
+    graphs = []
+    for stream, ctx, pool in lanes:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(steps):
+                pool.step(ctx, i, capi.F_ASYNC)
+        graphs.append(g)
+
+    def replay_all():
+        for (stream, _, _), g in zip(lanes, graphs):
+            with torch.cuda.stream(stream):
+                g.replay()
+
     for _ in range(3):
-        g.replay()
+        replay_all()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(replays):
-        g.replay()
+        replay_all()
     torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / (replays * steps)
-    ctx.sync()
-    ctx.close()
+    dt = (time.perf_counter() - t0) / (replays * steps * streams)
+    for _, ctx, _ in lanes:
+        ctx.sync()
+        ctx.close()
     return dt
+
+
+def roofline_of(pool: Pool, kt, traffic_known: bool = True) -> dict:
+    """Both copy kernels of a workload against the HBM peak: algorithmic bytes
+    per call over the average duration of the call's copy kernels (HIP events
+    around each launch on the stream they run on)."""
+    out = {}
+    for name, nbytes in (("k_gather", pool.gather_bytes), ("k_scatter", pool.scatter_bytes)):
+        ms = kt[name][0]
+        gbps = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+        out[name] = {"avg_kernel_us": round(ms * 1e3, 3), "bytes_per_launch": nbytes, "GBps": round(gbps, 1),
+                     "frac": round(gbps / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((pool.w.cfg, pool.bpl, name)) if traffic_known else None}
+    return out
 
 
 def cpu_baseline(w, seconds: float):
@@ -318,9 +377,16 @@ def main() -> int:
     bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
     prof = synth.HDR_REF64 if a.ref64 else synth.HDR_BL58
     w = synth.make_workload(a.workload, profile=prof)
-    ctx = SgContext(0, max_reqs=max(4096, w.n_req * bpl), max_frames=max(65536, max(w.n_frags, w.n_resp_frames) * bpl))
+    rule = not a.general
+
+    def contexts(wl, b):
+        mr, mf = max(4096, wl.n_req * b), max(65536, max(wl.n_frags, wl.n_resp_frames) * b)
+        # gather and scatter each on a context (and stream) of their own, unless one stream is asked for
+        return SgContext(0, max_reqs=mr, max_frames=mf), (None if a.one_stream else SgContext(0, max_reqs=mr, max_frames=mf))
+
+    ctx, ctx_tx = contexts(w, bpl)
     _log(f"staging {w.name} x {bpl} batches per launch")
-    pool = Pool(w, bpl, a.rotate_mb, extra, rule=not a.general)
+    pool = Pool(w, bpl, a.rotate_mb, extra, rule=rule)
     _log(f"{len(pool.items)} ring copies staged")
 
     if a.calib_copy:
@@ -331,8 +397,8 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    sec = timed(ctx, pool, a.steps, a.warmup)
-    _log(f"timed: {sec * 1e6:.1f} us per step")
+    sec = timed(ctx, pool, a.steps, a.warmup, ctx_tx)
+    _log(f"timed: {sec * 1e6:.1f} us per step (median of 5 runs of {a.steps} steps)")
     kt = kernel_times(ctx, pool, min(a.steps, 100))
     total_bytes = pool.gather_bytes + pool.scatter_bytes
     value = total_bytes / sec / 1e9
@@ -341,6 +407,9 @@ def main() -> int:
     dom_ms = kt[dom][0]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     b2b = back_to_back(ctx, pool, dom, min(a.steps, 100))
+    # the counters were read with the default kernels and headers only
+    traffic_known = not (a.general or a.ref64 or a.no_small or a.no_remap)
+    headline_roofs = roofline_of(pool, kt, traffic_known)
 
     _log("kernel times and back-to-back done; reassembly")
     # request reassembly on the device for the same call's arrivals (synchronous: counts come back)
@@ -365,14 +434,46 @@ def main() -> int:
     reassembly = {"arrivals": n_arr, "requests": got[0], "ms_per_call": round(ra_sec * 1e3, 4),
                   "arrivals_per_sec": round(n_arr / ra_sec, 1),
                   "tables_match_pre_staged": bool(got[0] == pool.n_req and torch.equal(ra_fs, dw0.frag_slot))}
+    # the same arrivals in bursts of 64, as a NIC delivers them: incomplete requests stay on the device
+    n_b = min(n_arr, 64 * 200)
+    for b in range(0, n_b, 64):
+        ctx.reassemble(dw0.rx, dw0.arrivals[b:b + 64], min(64, n_b - b), ra_fs, ra_fl, ra_rf, **ra_kw)
+    ctx.reassemble_reset()
+    t0 = time.perf_counter()
+    for b in range(0, n_b, 64):
+        ctx.reassemble(dw0.rx, dw0.arrivals[b:b + 64], min(64, n_b - b), ra_fs, ra_fl, ra_rf, **ra_kw)
+    reassembly["us_per_burst_of_64"] = round((time.perf_counter() - t0) / max(1, (n_b + 63) // 64) * 1e6, 2)
+    ctx.reassemble_reset()
     del ra_fs, ra_fl, ra_rf
 
-    _log("reassembly done; single-batch call")
+    # how the dominant kernel and the whole step scale with the batches laid side by side in one call
+    by_bpl = {}
+    if not a.no_sweep:
+        _log("batches-per-launch sweep")
+        for b in (1, 2, 4, 8, 16, 32):
+            if b == bpl:
+                by_bpl[str(b)] = {"ms_per_step": round(sec * 1e3, 5), "GBps": round(value, 1),
+                                  "kernel": dom, "avg_kernel_us": round(dom_ms * 1e3, 3),
+                                  "frac": round(achieved / HBM_PEAK_GBS, 4)}
+                continue
+            pb = Pool(w, b, a.rotate_mb, extra, rule=rule)
+            sb = timed(ctx, pb, max(20, a.steps // 4), max(5, a.warmup // 4), ctx_tx, reps=3)
+            kb = kernel_times(ctx, pb, 50)
+            nb = pb.gather_bytes if dom == "k_gather" else pb.scatter_bytes
+            gb = nb / (kb[dom][0] * 1e-3) / 1e9 if kb[dom][0] > 0 else 0.0
+            by_bpl[str(b)] = {"ms_per_step": round(sb * 1e3, 5),
+                              "GBps": round((pb.gather_bytes + pb.scatter_bytes) / sb / 1e9, 1),
+                              "kernel": dom, "avg_kernel_us": round(kb[dom][0] * 1e3, 3),
+                              "frac": round(gb / HBM_PEAK_GBS, 4)}
+            del pb
+            torch.cuda.empty_cache()
+
+    _log("single-batch call")
     # the single-batch call of the same workload, for the record
     single = None
     if bpl != 1:
-        p1 = Pool(w, 1, a.rotate_mb, extra, rule=not a.general)
-        s1 = timed(ctx, p1, a.steps, a.warmup)
+        p1 = Pool(w, 1, a.rotate_mb, extra, rule=rule)
+        s1 = timed(ctx, p1, a.steps, a.warmup, ctx_tx)
         k1 = kernel_times(ctx, p1, min(a.steps, 100))
         b1 = p1.gather_bytes + p1.scatter_bytes
         single = {"ms_per_step": round(s1 * 1e3, 5), "GBps": round(b1 / s1 / 1e9, 2),
@@ -381,9 +482,13 @@ def main() -> int:
                   "k_gather_GBps": round(p1.gather_bytes / (k1["k_gather"][0] * 1e-3) / 1e9, 1)
                   if k1["k_gather"][0] > 0 else None}
         del p1
-        sg = graph_step_time(w, extra, not a.general, a.rotate_mb)
-        single["hip_graph_ms_per_step"] = round(sg * 1e3, 5)
-        single["hip_graph_requests_per_sec"] = round(w.n_req / sg, 1)
+        for n_streams in (1, 2, 4):
+            sg = graph_step_time(w, extra, rule, a.rotate_mb, streams=n_streams)
+            key = "hip_graph" if n_streams == 1 else f"hip_graph_{n_streams}_streams"
+            single[key + "_ms_per_step"] = round(sg * 1e3, 5)
+            single[key + "_GBps"] = round(b1 / sg / 1e9, 1)
+            single[key + "_requests_per_sec"] = round(w.n_req / sg, 1)
+            torch.cuda.empty_cache()
 
     _log("per-request calls")
     per_req = per_request_calls(ctx, pool.items[0]) if not w.in_tensor_sizes else None
@@ -396,22 +501,26 @@ def main() -> int:
             wc = synth.make_workload(cfg)
             b = DEFAULT_BPL[cfg]
             _log(f"sweep: {wc.name} x {b}")
-            c2 = SgContext(0, max_reqs=max(4096, wc.n_req * b),
-                           max_frames=max(65536, max(wc.n_frags, wc.n_resp_frames) * b))
-            pc = Pool(wc, b, a.rotate_mb, extra, rule=not a.general)
-            sc = timed(c2, pc, max(20, a.steps // 4), max(5, a.warmup // 4))
+            c2, c2_tx = contexts(wc, b)
+            pc = Pool(wc, b, a.rotate_mb, extra, rule=rule)
+            sc = timed(c2, pc, max(20, a.steps // 4), max(5, a.warmup // 4), c2_tx, reps=3)
+            kc = kernel_times(c2, pc, 50)
             rps[wc.name] = round(pc.n_req / sc, 1)
             sweep[wc.name] = {"batches_per_launch": b, "ms_per_step": round(sc * 1e3, 5),
-                              "GBps": round((pc.gather_bytes + pc.scatter_bytes) / sc / 1e9, 2)}
+                              "GBps": round((pc.gather_bytes + pc.scatter_bytes) / sc / 1e9, 2),
+                              "frac_of_hbm_peak": round((pc.gather_bytes + pc.scatter_bytes) / sc / 1e9 / HBM_PEAK_GBS, 4),
+                              "kernels": roofline_of(pc, kc, traffic_known)}
             del pc
             c2.close()
+            if c2_tx is not None:
+                c2_tx.close()
             torch.cuda.empty_cache()
 
     if not a.no_sweep and not a.ref64:
         # the headline workload again with the reference's own 64-byte header
         wr = synth.make_workload(a.workload, profile=synth.HDR_REF64)
-        pr = Pool(wr, bpl, a.rotate_mb, extra, rule=not a.general)
-        sr = timed(ctx, pr, max(20, a.steps // 4), max(5, a.warmup // 4))
+        pr = Pool(wr, bpl, a.rotate_mb, extra, rule=rule)
+        sr = timed(ctx, pr, max(20, a.steps // 4), max(5, a.warmup // 4), ctx_tx, reps=3)
         sweep[wr.name + "_ref64_headers"] = {"batches_per_launch": bpl, "ms_per_step": round(sr * 1e3, 5),
                                              "GBps": round((pr.gather_bytes + pr.scatter_bytes) / sr / 1e9, 2)}
         del pr
@@ -436,13 +545,15 @@ def main() -> int:
                    "requests_per_step": pool.n_req, "header_profile": "REF64" if a.ref64 else "BL58",
                    "descriptor_pass": "general (prefix scan)" if a.general else
                    "fused where the workload has one size (fragmenting rule declared and checked)",
-                   "flags": w.flags},
+                   "streams": "one" if (a.one_stream or w.tx_in_place) else
+                   "gather and scatter calls on a stream each (a copy context per direction)",
+                   "timing": f"median of 5 runs of {a.steps} steps", "flags": w.flags},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "requests_per_sec": rps,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None if (a.general or a.ref64) else MEASURED_TRAFFIC.get((a.workload, bpl, dom)),
+                     "traffic": MEASURED_TRAFFIC.get((a.workload, bpl, dom)) if traffic_known else None,
                      "traffic_unit": "HBM bytes per launch (rocprofv3 --pmc, see profiles/)",
                      "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3),
                      # the same call launched back to back, two events around the burst (all of the
@@ -450,15 +561,20 @@ def main() -> int:
                      "back_to_back_us_per_call": round(b2b * 1e6, 3),
                      "back_to_back_GBps": round(dom_bytes / b2b / 1e9, 1)},
         "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in kt.items()},
+        "kernels": headline_roofs,
+        "roofline_by_batches_per_launch": by_bpl,
         "single_batch_call": single,
         "per_request_call": per_req,
         "device_reassembly": reassembly,
         "other_workloads": sweep,
     }
     if not a.no_cpu:
+        _log("CPU baseline")
         out["cpu_baseline"] = cpu_baseline(w, a.cpu_seconds)
     print(json.dumps(out))
     ctx.close()
+    if ctx_tx is not None:
+        ctx_tx.close()
     return 0
 
 
