@@ -660,4 +660,153 @@ __device__ __forceinline__ void small_hdr_finish(SmallHdr s, uint8_t *out, uint3
   if (on1) w[h1] = (uint16_t)v1;
 }
 
+// ---- the header as 16-bit words, one per lane -------------------------------
+// For a kernel whose wavefront has ONE frame (k_scatter): lanes 0..31 hold the
+// header's 16-bit words (29 of them with the 58-byte header, 32 with the
+// 64-byte one).  Every field is a whole number of such words at an even
+// offset, and everything that goes into a field is wavefront-uniform, so a
+// field is written into its lane (v_writelane) and the few words a checksum
+// needs are read out of their lanes (v_readlane): a couple of dozen
+// instructions, where the byte-per-lane form above pays a compare and a select
+// for every byte position and a cross-lane reduction for every sum.  Same
+// fields, flags and results as hdr_finish.
+
+// Sum over the wavefront, wavefront-uniform: row reductions by DPP, the four
+// row totals added on the scalar side.
+__device__ __forceinline__ uint32_t wave_sum_uniform(uint32_t v)
+{
+  v = row_sum(v);
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 0) + (uint32_t)__builtin_amdgcn_readlane((int)v, 16) +
+         (uint32_t)__builtin_amdgcn_readlane((int)v, 32) + (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+}
+
+// Distance from header word h to the word it takes its value from when MACs,
+// addresses and ports change places (words 0-2 <-> 3-5, 13-14 <-> 15-16,
+// 17 <-> 18), three bits two's complement per word; words from 19 on stay.
+__host__ __device__ constexpr uint64_t hdrw_delta_table()
+{
+  uint64_t t = 0;
+  for (int h = 0; h < 19; h++) {
+    int d = 0;
+    if (h < 3) d = 3;
+    else if (h < 6) d = -3;
+    else if (h == 13 || h == 14) d = 2;
+    else if (h == 15 || h == 16) d = -2;
+    else if (h == 17) d = 1;
+    else if (h == 18) d = -1;
+    t |= (uint64_t)(d & 7) << (3 * h);
+  }
+  return t;
+}
+
+__device__ __forceinline__ uint32_t hdrw_src(uint32_t h)
+{
+  constexpr uint64_t kDelta = hdrw_delta_table();
+  const uint32_t k = h < 19u ? h : 19u;  // bits 57.. of the table are zero
+  const uint32_t code = (uint32_t)(kDelta >> (3u * k));
+  return h + (uint32_t)((int32_t)(code << 29) >> 29);
+}
+
+// The word lane `lane` starts from (zero on lanes past the header).
+__device__ __forceinline__ uint32_t hdrw_fetch(const uint8_t *__restrict__ in, uint32_t lane, uint32_t hl, bool swap)
+{
+  const uint16_t *w = reinterpret_cast<const uint16_t *>(in);  // rings and templates start at even addresses
+  uint32_t v = 0;
+  if (lane < (hl >> 1)) v = w[swap ? hdrw_src(lane) : lane];
+  return v;
+}
+
+// v_writelane_b32: clang has no builtin of this name for the LLVM intrinsic, so the intrinsic
+// is declared under its own name (the compiler then also places the wait states it needs)
+extern "C" __device__ int sg_llvm_amdgcn_writelane(int value, int lane, int old) __asm("llvm.amdgcn.writelane.i32");
+
+__device__ __forceinline__ uint32_t hdrw_put(uint32_t v, uint32_t word, uint32_t value)
+{
+  return (uint32_t)sg_llvm_amdgcn_writelane((int)value, (int)word, (int)v);
+}
+
+__device__ __forceinline__ uint32_t hdrw_get(uint32_t v, uint32_t word)
+{
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, (int)word);
+}
+
+// Lengths, routing words and the token; both checksum words cleared after a swap.
+__device__ __forceinline__ uint32_t hdrw_fields(uint32_t v, const HdrFields &f)
+{
+  const uint32_t L = (f.hl - 42u) + f.payload_len;
+  const uint32_t tot = (28u + L) & 0xffffu, ulen = (8u + L) & 0xffffu;
+  v = hdrw_put(v, 8, bswap16(tot));
+  v = hdrw_put(v, 19, bswap16(ulen));
+  if (!f.from_template) {  // swap_eth_hdr zeroes both sums
+    v = hdrw_put(v, 12, 0);
+    v = hdrw_put(v, 20, 0);
+  }
+  if (f.set_token) {
+#pragma unroll
+    for (uint32_t k = 0; k < 4; k++) v = hdrw_put(v, 21 + k, (uint32_t)(f.token >> (16u * k)) & 0xffffu);
+  }
+  if (f.ref64) {
+    v = hdrw_put(v, 25, 0);  // sock_perf_header &= 0xFFFFFFFF00000000
+    v = hdrw_put(v, 26, 0);
+    v = hdrw_put(v, 29, f.frag_idx & 0xffffu);
+  } else {
+    v = hdrw_put(v, 25, f.frag_idx & 0xffffu);
+    v = hdrw_put(v, 26, f.num_frags & 0xffffu);
+    v = hdrw_put(v, 27, f.payload_len & 0xffffu);
+    v = hdrw_put(v, 28, f.payload_len >> 16);
+  }
+  return v;
+}
+
+// This lane's share of the UDP checksum's sum over the header (UDP header
+// without the checksum word, and everything behind it): to be added to the
+// lane's payload sum before the wavefront-wide reduction.
+__device__ __forceinline__ uint32_t hdrw_l4_share(uint32_t v, uint32_t lane, uint32_t hl)
+{
+  return (lane >= 17u && lane < (hl >> 1) && lane != 20u) ? v : 0u;
+}
+
+// Checksum words.  l4_sum: wavefront-uniform sum of the payload's words plus
+// the lanes' hdrw_l4_share.  With l4_partial the finished UDP checksum is
+// somebody else's business: the word is left zero and *l4_partial gets the
+// pseudo-header's share of the sum, unfolded.
+__device__ __forceinline__ uint32_t hdrw_csums(uint32_t v, const HdrFields &f, uint32_t l4_sum,
+                                               uint32_t *l4_partial = nullptr)
+{
+  const uint32_t kAnyCsum = 0x7u;  // IPV4 | PSEUDO | FULL
+  if (f.flags & kAnyCsum) {
+    const uint32_t L = (f.hl - 42u) + f.payload_len;
+    const uint32_t tot = (28u + L) & 0xffffu, ulen = (8u + L) & 0xffffu;
+    const uint32_t w7 = hdrw_get(v, 7), w11 = hdrw_get(v, 11);
+    const uint32_t s_addr = hdrw_get(v, 13) + hdrw_get(v, 14) + hdrw_get(v, 15) + hdrw_get(v, 16);
+    const uint32_t b14 = w7 & 0xffu, proto = w11 >> 8;
+    if (f.flags & (1u << 1)) {  // raw pseudo sum, reference style
+      const uint32_t hdr_bytes = (f.flags & (1u << 3)) ? (b14 >> 4) * 4u : (b14 & 0xfu) * 4u;
+      const uint32_t l = (tot - hdr_bytes) & 0xffffu;
+      v = hdrw_put(v, 20, fold16(s_addr + (proto << 8) + bswap16(l)));
+    }
+    if (f.flags & (1u << 2)) {  // finished UDP checksum
+      const uint32_t s = s_addr + (proto << 8) + bswap16(ulen);
+      uint32_t c = 0;
+      if (l4_partial) {
+        *l4_partial = s;
+      } else {
+        c = (~fold16(fold16(s) + fold16(l4_sum))) & 0xffffu;
+        if (c == 0) c = 0xffffu;
+      }
+      v = hdrw_put(v, 20, c);
+    }
+    if (f.flags & (1u << 0)) {  // finished IPv4 header checksum: words 7..16 without word 12
+      const uint32_t s_ip = s_addr + w7 + hdrw_get(v, 8) + hdrw_get(v, 9) + hdrw_get(v, 10) + w11;
+      v = hdrw_put(v, 12, (~fold16(s_ip)) & 0xffffu);
+    }
+  }
+  return v;
+}
+
+__device__ __forceinline__ void hdrw_store(uint8_t *out, uint32_t lane, uint32_t hl, uint32_t v)
+{
+  if (lane < (hl >> 1)) reinterpret_cast<uint16_t *>(out)[lane] = (uint16_t)v;
+}
+
 }  // namespace sg

@@ -540,7 +540,7 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
                                               uint32_t *i, uint64_t *req_off)
 {
   uint32_t bad = 0;
-  *r = item / g.per_req;
+  *r = (uint32_t)(((uint64_t)item * g.div_mul) >> g.div_shift);  // item / per_req
   *i = item - *r * g.per_req;
   // the three table reads are independent: asked for together
   *slot = sload_here(g.item_slot + item);
@@ -1196,7 +1196,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
       if (n) part = copy_run<DEFER>(from + o, slot + hl + o, n, lane);
     }
     if (DEFER) {
-      part = wave_sum(part);
+      part = wave_sum_uniform(part);
       if (lane == 0) a.csum_part[(size_t)item * kPartStride + piece] = part;
     }
     return;
@@ -1205,7 +1205,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   // (the TX slot may be the very slot the header comes from);
   // header bytes and payload chunks are fetched together; the header arithmetic
   // then runs while the payload is still on its way
-  const uint32_t raw = hdr_fetch(hin, lane, hl, !from_template);
+  const uint32_t raw = hdrw_fetch(hin, lane, hl, !from_template);
   uint32_t hb = 0, acc = 0;
   uint8_t *from = nullptr;
   const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
@@ -1216,18 +1216,21 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     sub_run(slot + hl, d[1], 0, &o, &first_len);
   }
   if (plain && !WHOLE_LONG) run_begin(rs, from, slot + hl, first_len, lane);
-  if (!FULL_CSUM) hb = hdr_finish(raw, lane, hf, 0);
+  hb = hdrw_fields(raw, hf);
+  if (!FULL_CSUM) hb = hdrw_csums(hb, hf, 0);
   if (plain) {
     if (WHOLE_LONG) acc = copy_long_run<FULL_CSUM, 2>(from, slot + hl, d[1], lane);
     else acc = run_end<FULL_CSUM>(rs, lane);
   } else if (d[1]) {
     acc = move_run<false, FULL_CSUM>(a.app, ro, r, d[2], slot + hl, d[1], lane);
   }
-  if (FULL_CSUM && !DEFER) hb = hdr_finish(raw, lane, hf, wave_sum(acc));
+  // the header's own share of the UDP sum rides with the payload's
+  if (FULL_CSUM) acc += hdrw_l4_share(hb, lane, hl);
+  if (FULL_CSUM && !DEFER) hb = hdrw_csums(hb, hf, wave_sum_uniform(acc));
   if (DEFER) {
     uint32_t l4 = 0;
-    hb = hdr_finish(raw, lane, hf, 0, &l4);
-    const uint32_t part = wave_sum(acc);
+    hb = hdrw_csums(hb, hf, 0, &l4);
+    const uint32_t part = wave_sum_uniform(acc);
     if (lane == 0) {
       a.csum_part[(size_t)item * kPartStride] = part;
       a.csum_part[(size_t)item * kPartStride + n_pieces] = l4;
@@ -1236,7 +1239,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   }
   // the payload went past the header only, so a TX slot that is the header's own
   // source still held the request header when it was fetched above
-  if (lane < hl) slot[lane] = (uint8_t)hb;
+  hdrw_store(slot, lane, hl, hb);
 }
 
 // Second phase of the full UDP checksum of long frames: one thread per frame
