@@ -48,6 +48,17 @@ __device__ __forceinline__ u32x4 load16_aligned(const uint8_t *p)
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
 }
 
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+
+// Address of byte `off` of the running kernel's argument block.  A kernel with one by-value
+// argument finds that argument at byte 0: a table inside it can then be indexed by a value
+// known only at run time with one scalar load (indexing the by-value copy itself would have
+// the compiler spill the table to private memory).
+__device__ __forceinline__ const uint8_t *kernarg_at(size_t off)
+{
+  return reinterpret_cast<const uint8_t *>((uintptr_t)__builtin_amdgcn_kernarg_segment_ptr()) + off;
+}
+
 // Load through the scalar data cache: for wave-uniform addresses of data that
 // NO wavefront of the running kernel writes (tables and cursors produced by an
 // earlier kernel, ring headers in a kernel that only reads the ring).  The

@@ -736,6 +736,17 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   }
 }
 
+// Where the bytes of fragment i of every request go, several tensor-major buffers:
+// request r's share of the fragment starts at base + r * stride.
+struct FragPlan {
+  uint64_t base_a, base_b;      // tensor base + offset inside the request's share (b: the next tensor's base)
+  uint32_t stride_a, stride_b;  // bytes per request of the tensor(s)
+  uint32_t len_a;               // bytes that go to the first tensor
+  uint32_t kind;                // 0: one tensor, 1: two tensors, 2: more (general path)
+};
+constexpr uint32_t kPlanMax = 8;
+static_assert(sizeof(FragPlan) == 32, "a plan entry is one 8-dword scalar load");
+
 // Gather without a descriptor pass: all requests have `size` bytes cut by the
 // fragmenting rule, so a wavefront derives its descriptor from its item
 // number (item f belongs to request f / per_req, is its fragment f % per_req,
@@ -773,6 +784,13 @@ struct GatherRuleArgs {
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   AppDev app;  // consulted for several tensor-major buffers only
+  // Several tensor-major buffers: where fragment i of a request lands depends on i alone (all
+  // requests have one size), so the host walks the tensors once per fragment index and the
+  // wavefront reads one entry instead of walking them itself.  n_plan == 0: no plan (too many
+  // fragments per request, or tensors of 4 GiB and more per request).
+  uint32_t n_plan;
+  uint32_t plan_pad;
+  FragPlan plan[kPlanMax];
 };
 constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
 // slots start at 16-byte aligned addresses: the header's length field can be read as part of
@@ -850,6 +868,8 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   uint64_t ro = 0;
   bool plain = !(opts & kOptMultiTensor);
   uint8_t *to = nullptr;
+  uint8_t *to_a = nullptr, *to_b = nullptr;
+  uint32_t len_a = 0, plan_kind = 3;  // 3: no plan, the tensors are walked here
   if (cap) {
     // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
     if (c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
@@ -870,7 +890,17 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     to = dst + o;
   } else if (opts & kOptMultiTensor) {
     // tensor-major buffers: a fragment inside one tensor still takes the fast path
-    plain = plain_target(a.app, 0, r, off, len, &to);
+    if (a.n_plan) {
+      const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(GatherRuleArgs, plan))) + i);
+      plan_kind = fp[7];
+      plain = plan_kind == 0;
+      to = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
+      to_a = to;
+      len_a = fp[6];
+      to_b = reinterpret_cast<uint8_t *>(((uint64_t)fp[3] << 32 | fp[2]) + (uint64_t)r * fp[5]);
+    } else {
+      plain = plain_target(a.app, 0, r, off, len, &to);
+    }
   } else {
     to = dst + (uint64_t)r * size + off;
   }
@@ -898,10 +928,8 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   if (LONG && plain) sub_run(to, len, piece, &sub_off, &sub_len);
   if (plain && sub_len) run_begin(rs, pkt + hl + sub_off, to + sub_off, sub_len, lane);
   // a fragment that runs from one tensor into the next: two runs, both in flight at once
-  uint8_t *to_a = nullptr, *to_b = nullptr;
-  uint32_t len_a = 0;
   const bool two = !plain && (opts & kOptMultiTensor) && piece == 0 &&
-                   two_tensor_target(a.app, r, off, len, &to_a, &len_a, &to_b);
+                   (plan_kind == 3 ? two_tensor_target(a.app, r, off, len, &to_a, &len_a, &to_b) : plan_kind == 1);
   RunState rb;
   if (two) {
     run_begin(rs, pkt + hl, to_a, len_a, lane);
@@ -936,6 +964,11 @@ template <int L>
 __device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave)
 {
   constexpr uint32_t G = kWave / L;
+  // every argument of the common path in one burst of scalar loads
+  SG_PIN(a.per_req); SG_PIN(a.mtu); SG_PIN(a.hl); SG_PIN(a.counts); SG_PIN(a.n_req); SG_PIN(a.opts);
+  SG_PIN(a.size); SG_PIN(a.frag_slot); SG_PIN(a.first); SG_PIN(a.n_slots); SG_PIN(a.cap); SG_PIN(a.cursor);
+  SG_PIN(a.offsets_out); SG_PIN(a.ring); SG_PIN(a.slot_size); SG_PIN(a.frag_len); SG_PIN(a.dst);
+  SG_PIN(a.n_plan); SG_PIN(a.div_mul); SG_PIN(a.div_shift);
   const uint32_t lane = threadIdx.x & (kWave - 1), gl = lane & (L - 1);
   const uint32_t per_req = a.per_req, mtu = a.mtu, hl = a.hl;
   const uint32_t n_req = dev_count(a.counts, 0, a.n_req);
@@ -994,7 +1027,14 @@ __device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint3
       // the packed arena, walked through the AppDev view the host filled in for this kernel
       plain = plain_target(a.app, ro, r, off, len, &to);
     } else if (a.opts & kOptMultiTensor) {
-      plain = plain_target(a.app, 0, r, off, len, &to);
+      if (last_only && a.n_plan) {
+        // every group has the request's last fragment: one plan entry for the wavefront
+        const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(GatherRuleArgs, plan))) + (per_req - 1));
+        plain = fp[7] == 0;
+        to = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
+      } else {
+        plain = plain_target(a.app, 0, r, off, len, &to);
+      }
     } else {
       to = a.dst + (uint64_t)r * a.size + off;
       plain = true;
@@ -1058,6 +1098,11 @@ struct ScatterArgs {
   uint64_t *offsets_out;
   RuleArgs rule;
   AppDev app;
+  // fused, tensor-major buffers: where the bytes of frame i of a response come from (as
+  // GatherRuleArgs::plan); n_plan == 0: the tensors are walked by the wavefront
+  uint32_t n_plan;
+  uint32_t plan_pad;
+  FragPlan plan[kPlanMax];
 };
 
 // LONG: frames longer than kPieceChunks chunks are spread over a.pieces
@@ -1067,6 +1112,19 @@ struct ScatterArgs {
 // measured slower: 3 at a time +1 %, 5 at a time +8 %).  (Summing per piece and combining with one returning atomic
 // per wavefront was measured: the atomic's round trip at the end of every
 // wavefront's life cost more than the shorter tail gained.)
+// Where the payload of a frame comes from; false: not one contiguous piece.
+template <bool FUSED>
+__device__ __forceinline__ bool scatter_source(const ScatterArgs &a, uint64_t ro, uint32_t r, uint32_t i,
+                                               uint32_t off, uint32_t len, uint8_t **from)
+{
+  if (FUSED && a.n_plan) {
+    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(ScatterArgs, plan))) + i);
+    *from = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
+    return fp[7] == 0;
+  }
+  return plain_target(a.app, ro, r, off, len, from);
+}
+
 constexpr uint32_t kPartStride = 8;  // words of csum_part per frame: up to 7 sub-runs and the header's share
 
 // DEFER (long frames with the full UDP checksum): the frame's sub-runs go to
@@ -1190,7 +1248,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     // a later piece of a long frame: payload only
     uint8_t *from;
     uint32_t part = 0;
-    if (d[1] && plain_target(a.app, ro, r, d[2], d[1], &from)) {
+    if (d[1] && scatter_source<FUSED>(a, ro, r, item - f0, d[2], d[1], &from)) {
       uint32_t o, n;
       sub_run(slot + hl, d[1], piece, &o, &n);
       if (n) part = copy_run<DEFER>(from + o, slot + hl + o, n, lane);
@@ -1208,7 +1266,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   const uint32_t raw = hdrw_fetch(hin, lane, hl, !from_template);
   uint32_t hb = 0, acc = 0;
   uint8_t *from = nullptr;
-  const bool plain = d[1] != 0 && plain_target(a.app, ro, r, d[2], d[1], &from);
+  const bool plain = d[1] != 0 && scatter_source<FUSED>(a, ro, r, item - f0, d[2], d[1], &from);
   RunState rs;
   uint32_t first_len = d[1];
   if (SPLIT && plain) {
@@ -1282,6 +1340,15 @@ template <int L, bool FULL_CSUM>
 __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_t wave)
 {
   constexpr uint32_t G = kWave / L;
+  // every argument of the common path in one burst of scalar loads (left to their first uses they
+  // arrive one dependent round trip after the other, a good part of this wavefront's life)
+  SG_PIN(a.rule.per_req); SG_PIN(a.rule.mtu); SG_PIN(a.hl); SG_PIN(a.counts); SG_PIN(a.n_req);
+  SG_PIN(a.rule.per_launch); SG_PIN(a.rule.size); SG_PIN(a.hdr_templates); SG_PIN(a.rule.item_slot);
+  SG_PIN(a.rule.first); SG_PIN(a.hdr_src_req); SG_PIN(a.hdr_src_slot); SG_PIN(a.rule.n_slots);
+  SG_PIN(a.rx_n_slots); SG_PIN(a.app.n_tensors); SG_PIN(a.rule.cursor); SG_PIN(a.app.cap);
+  SG_PIN(a.rule.single_wrap); SG_PIN(a.rule.offsets_out); SG_PIN(a.rule.div_mul); SG_PIN(a.rule.div_shift);
+  SG_PIN(a.req_token); SG_PIN(a.rx); SG_PIN(a.rx_slot_size); SG_PIN(a.tx); SG_PIN(a.tx_slot_size);
+  SG_PIN(a.ref64); SG_PIN(a.flags); SG_PIN(a.n_plan); SG_PIN(a.app.arena); SG_PIN(a.app.mirrored);
   const uint32_t lane = threadIdx.x & (kWave - 1), gl = lane & (L - 1);
   const uint32_t per_req = a.rule.per_req, mtu = a.rule.mtu, hl = a.hl;
   const uint32_t n_req = dev_count(a.counts, 0, a.n_req);
@@ -1351,7 +1418,15 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
   // source still holds the request header then (the payload goes past the header only)
   const SmallHdr sh = small_hdr_fetch(hin, gl, hl, !from_template, live && gl < 16);
   uint8_t *from = nullptr;
-  const bool plain = live && len != 0 && plain_target(a.app, ro, r, off, len, &from);
+  bool plain;
+  if (last_only && a.n_plan) {
+    // every group has the response's last frame: one plan entry for the wavefront
+    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(ScatterArgs, plan))) + (per_req - 1));
+    from = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
+    plain = live && len != 0 && fp[7] == 0;
+  } else {
+    plain = live && len != 0 && plain_target(a.app, ro, r, off, len, &from);
+  }
   GroupRun<L> run;
   group_run_begin<L>(run, from, slot + hl, plain ? len : 0u, gl);
   uint32_t acc = group_run_end<L, FULL_CSUM>(run, gl);
@@ -2172,6 +2247,44 @@ int finish(sg_hip_ctx *c, uint32_t flags)
 }  // namespace
 
 // floor(n / d) == (n * M) >> (27 + l) for every n < 2^27, with l = ceil(log2 d), M = ceil(2^(27 + l) / d)
+// Walks the tensor-major buffers once per fragment index (all requests of the call have `size`
+// bytes cut at `mtu`): where fragment i lands, for every i.  Returns the number of entries, or 0
+// when there is no plan (more fragments per request than entries, a tensor of 4 GiB or more per
+// request).
+static uint32_t fill_plan(const AppDev &app, uint64_t size, uint32_t mtu, uint64_t per, FragPlan *plan)
+{
+  if (per > kPlanMax) return 0;
+  for (uint32_t t = 0; t < app.n_tensors; t++)
+    if (app.tensor_size[t] > 0xffffffffull) return 0;
+  for (uint32_t i = 0; i < per; i++) {
+    const uint64_t off = (uint64_t)i * mtu;
+    const uint64_t len = size - off < mtu ? size - off : mtu;
+    FragPlan &fp = plan[i];
+    memset(&fp, 0, sizeof fp);
+    fp.kind = 2;
+    uint64_t t0 = 0;
+    for (uint32_t t = 0; t < app.n_tensors; t++) {
+      const uint64_t t1 = t0 + app.tensor_size[t];
+      if (off < t1) {
+        fp.base_a = (uint64_t)(uintptr_t)app.tensor_base[t] + (off - t0);
+        fp.stride_a = (uint32_t)app.tensor_size[t];
+        if (off + len <= t1) {
+          fp.kind = 0;
+          fp.len_a = (uint32_t)len;
+        } else if (t + 1 < app.n_tensors && off + len <= t1 + app.tensor_size[t + 1]) {
+          fp.kind = 1;
+          fp.len_a = (uint32_t)(t1 - off);
+          fp.base_b = (uint64_t)(uintptr_t)app.tensor_base[t + 1];
+          fp.stride_b = (uint32_t)app.tensor_size[t + 1];
+        }
+        break;
+      }
+      t0 = t1;
+    }
+  }
+  return (uint32_t)per;
+}
+
 static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
 {
   uint32_t l = 0;
@@ -2590,6 +2703,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     ga.status_flag = sc.flag;
     ga.app = app;
     ga.pieces = pieces_for(a->mtu);
+    if (app.n_tensors > 1) ga.n_plan = fill_plan(app, a->fixed_req_size, a->mtu, per, ga.plan);
     uint32_t grid, remap;
     uint64_t waves = (uint64_t)a->n_req * ga.per_launch * ga.pieces;
     if (small_last) {
@@ -2771,6 +2885,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.rule.single_wrap = app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_resp_size <= app.cap;
     sa.rule.cursor = sc.cursor[1];
     sa.rule.offsets_out = packed ? a->offsets_out : nullptr;
+    if (app.n_tensors > 0) sa.n_plan = fill_plan(app, a->fixed_resp_size, a->mtu, per, sa.plan);
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
     // short frames go several to a wavefront: all of them where a full frame is short, else the
@@ -2795,6 +2910,9 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
       sa.csum_valid = sc.csum_valid;
       geometry((uint64_t)a->n_req * sa.rule.per_launch * ((full_csum && !defer) ? 1u : sa.pieces),
                !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+      // (the remainder frames' kernel on a second stream beside this one, forked and joined with
+      // events, was measured as well: both kinds of wavefront at once cost the full frames more
+      // than the overlap gains, 180 against 172 us on 131072 responses of 1400 + 1400 + 272 bytes)
       launch_scatter<true>(st, sa, grid, full_csum, defer);
       if (small_last) launch_scatter_small(st, sa, small_last, a->n_req, full_csum);
     }
