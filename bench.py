@@ -77,6 +77,8 @@ def parse():
                          "traffic, to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     ap.add_argument("--one-stream", action="store_true",
                     help="gather and scatter calls on one context and stream (default: one each)")
+    ap.add_argument("--no-single", action="store_true",
+                    help="skip the single-batch legs (eager, HIP graphs on 1, 2 and 4 streams)")
     ap.add_argument("--general", action="store_true",
                     help="always run the descriptor pass (do not declare the fragmenting rule)")
     return ap.parse_args()
@@ -471,7 +473,7 @@ def main() -> int:
     _log("single-batch call")
     # the single-batch call of the same workload, for the record
     single = None
-    if bpl != 1:
+    if bpl != 1 and not a.no_single:
         p1 = Pool(w, 1, a.rotate_mb, extra, rule=rule)
         s1 = timed(ctx, p1, a.steps, a.warmup, ctx_tx)
         k1 = kernel_times(ctx, p1, min(a.steps, 100))

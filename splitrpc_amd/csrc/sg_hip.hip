@@ -2199,6 +2199,8 @@ int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs
       k_req_scan<<<1, kScanBlock, 0, st>>>(p);
     } else {
       const uint32_t n_tiles = (p.n_req + kScanTile - 1) / kScanTile;
+      // (one launch in which every workgroup adds up the sizes before its tile by itself was
+      // measured at 32768 requests: 30.6 us for the descriptor pass against 26.9 us with these two)
       k_req_scan_local<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot);
       k_req_scan_add<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot, n_tiles);
     }

@@ -617,6 +617,32 @@ def test_tiled_request_scan_beyond_8192_requests():
     big.close()
 
 
+def test_tiled_request_scan_of_70000_small_requests():
+    """Seventeen tiles of request totals, many requests of a few dozen bytes:
+    same offsets as the sequential bump ring."""
+    rng = np.random.default_rng(77)
+    n = 70000
+    sizes = rng.integers(16, 200, size=n)
+    w = synth.make_custom(sizes, [16] * n, order="in_order", seed=5)
+    big = SgContext(0, max_reqs=n, max_frames=1 << 17)
+    dw = DeviceWorkload(w)
+    total = int(w.req_sizes.sum())
+    cursor, cap = 4242, total + 999
+    arena = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+    offs = torch.zeros(n + 1, dtype=torch.int64, device=DEV)
+    big.set_cursor(0, cursor)
+    big.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags,
+                     AppRef(arena=arena, cap=cap), offs)
+    want = (cursor + np.concatenate([[0], np.cumsum(w.req_sizes.astype(np.uint64))])) % cap
+    assert np.array_equal(offs.cpu().numpy().view(np.uint64), want.astype(np.uint64))
+    assert big.get_cursor(0) == int(want[-1])
+    exp = np.zeros(cap, np.uint8)
+    exp[(cursor + np.arange(w.req_payload.size, dtype=np.int64)) % cap] = w.req_payload
+    got = arena.cpu().numpy()
+    assert np.array_equal(got, exp), first_diff(got, exp)
+    big.close()
+
+
 # ---------------------------------------------------------------- descriptors reused by the echo
 
 def test_echo_scatter_reuses_the_descriptors_of_its_gather(ctx):
