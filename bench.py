@@ -32,15 +32,15 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes the copy kernels of one call move, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this file (--calib-copy --steps 40 --warmup 5), each counter scaled by what it reads for a plain
 # 512 MiB device copy in the same run (FETCH_SIZE x 2.000 KiB, WRITE_SIZE x 1.000 KiB).  Keyed by
-# (workload, batches per launch, kernel family); the default call: 340.5 MB read + 312.2 MB written.
+# (workload, batches per launch, kernel family); the default call: 340.5 MB read + 313.5 MB written.
 # bert's scatter is both of its kernels (full frames + short remainder frames), jumbo's the copy
 # phase without the 1.9 MB of the checksum-finishing kernel.
 MEASURED_TRAFFIC = {
-    (2, 32, "k_gather"): 652.7e6, (2, 32, "k_scatter"): 4.8e6,
-    (1, 2048, "k_gather"): 449.8e6, (1, 2048, "k_scatter"): 23.3e6,
-    (3, 512, "k_gather"): 582.5e6, (3, 512, "k_scatter"): 935.1e6,
-    (4, 8, "k_gather"): 661.7e6, (4, 8, "k_scatter"): 677.1e6,
-    (5, 4, "k_gather"): 817.2e6, (5, 4, "k_scatter"): 549.7e6,
+    (2, 32, "k_gather"): 654.1e6, (2, 32, "k_scatter"): 4.8e6,
+    (1, 2048, "k_gather"): 450.4e6, (1, 2048, "k_scatter"): 23.2e6,
+    (3, 512, "k_gather"): 583.4e6, (3, 512, "k_scatter"): 932.7e6,
+    (4, 8, "k_gather"): 661.8e6, (4, 8, "k_scatter"): 676.0e6,
+    (5, 4, "k_gather"): 817.9e6, (5, 4, "k_scatter"): 549.2e6,
 }
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
