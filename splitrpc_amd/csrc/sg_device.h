@@ -214,18 +214,24 @@ __device__ __forceinline__ void run_begin(RunState &r, const uint8_t *__restrict
 // words the run's bytes fall into, a byte's position in its word being the
 // parity of its DESTINATION ADDRESS (packet offsets and addresses have the
 // same parity: ring bases, slot sizes and header lengths are even).
-template <bool CSUM>
-__device__ __forceinline__ uint32_t run_end(RunState &r, uint32_t lane)
+//
+// BROKEN: the destination is two pieces -- aligned chunks from number `brk` on, and the tail
+// bytes, land `jump` bytes further (a fragment that runs from one tensor into the next, where
+// the second tensor's share starts on a 16-byte boundary and the first one's share ends on a
+// chunk boundary of the run): one run instead of two.
+template <bool CSUM, bool BROKEN = false>
+__device__ __forceinline__ uint32_t run_end(RunState &r, uint32_t lane, uint32_t brk = 0, int64_t jump = 0)
 {
   uint32_t acc = 0;
   const u32x4 o0 = realign(r.v0, r.p);
   const u32x4 o1 = realign(r.v1, r.p);
+  auto at = [&](uint32_t c) { return r.d + ((size_t)c << 4) + ((BROKEN && c >= brk) ? jump : (int64_t)0); };
   if (lane < 63 && lane < r.body) {
-    store16_aligned(r.d + ((size_t)lane << 4), o0);
+    store16_aligned(at(lane), o0);
     if (CSUM) acc += words_sum(o0);
   }
   if (lane < 63 && 63u + lane < r.body) {
-    store16_aligned(r.d + ((size_t)(63u + lane) << 4), o1);
+    store16_aligned(at(63u + lane), o1);
     if (CSUM) acc += words_sum(o1);
   }
   for (uint32_t base = 126; base < r.body; base += 126) {
@@ -236,17 +242,19 @@ __device__ __forceinline__ uint32_t run_end(RunState &r, uint32_t lane)
     const u32x4 q0 = realign(v0, r.p);
     const u32x4 q1 = realign(v1, r.p);
     if (lane < 63 && c0 < r.body) {
-      store16_aligned(r.d + ((size_t)c0 << 4), q0);
+      store16_aligned(at(c0), q0);
       if (CSUM) acc += words_sum(q0);
     }
     if (lane < 63 && c1 < r.body) {
-      store16_aligned(r.d + ((size_t)c1 << 4), q1);
+      store16_aligned(at(c1), q1);
       if (CSUM) acc += words_sum(q1);
     }
   }
   if (r.edge) {
-    r.dst[r.eoff] = (uint8_t)r.eb;
-    if (CSUM) acc += ((uintptr_t)(r.dst + r.eoff) & 1u) ? (r.eb << 8) : r.eb;
+    // head bytes sit on lanes 0..15, tail bytes (behind the last aligned chunk) on lanes 16..31
+    uint8_t *e = r.dst + r.eoff + ((BROKEN && lane >= 16) ? jump : (int64_t)0);
+    *e = (uint8_t)r.eb;
+    if (CSUM) acc += ((uintptr_t)e & 1u) ? (r.eb << 8) : r.eb;
   }
   return acc;
 }

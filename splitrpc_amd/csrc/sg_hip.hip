@@ -931,13 +931,22 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const bool two = !plain && (opts & kOptMultiTensor) && piece == 0 &&
                    (plan_kind == 3 ? two_tensor_target(a.app, r, off, len, &to_a, &len_a, &to_b) : plan_kind == 1);
   RunState rb;
-  if (two) {
+  // ... as ONE run with a break in its destination where the second tensor's share starts on a
+  // 16-byte boundary and the first one's ends on a chunk boundary of the run (tensors of whole
+  // chunks at aligned addresses)
+  const uint32_t head_a = (uint32_t)(-(uintptr_t)to_a) & 15u;
+  const bool one_run = two && ((uintptr_t)to_b & 15u) == 0 && len_a >= head_a && ((len_a - head_a) & 15u) == 0;
+  if (one_run) {
+    run_begin(rs, pkt + hl, to_a, len, lane);
+  } else if (two) {
     run_begin(rs, pkt + hl, to_a, len_a, lane);
     run_begin(rb, pkt + hl + len_a, to_b, len - len_a, lane);
   }
   asm volatile("" ::"v"(hc), "v"(hv));  // consumed only after the payload loads are under way
   if (plain) {
     if (sub_len) run_end<false>(rs, lane);
+  } else if (one_run) {
+    run_end<false, true>(rs, lane, (len_a - head_a) >> 4, (int64_t)(to_b - (to_a + len_a)));
   } else if (two) {
     run_end<false>(rs, lane);
     run_end<false>(rb, lane);
