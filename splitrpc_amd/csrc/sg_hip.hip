@@ -100,6 +100,9 @@ struct PrepArgs {
   // [1] items.  n_req and n_items above are then upper bounds the launch was
   // sized with.  nullptr: the bounds are the counts.
   const uint32_t *counts;
+  // k_prep_group: where every workgroup leaves the sum of its requests' totals (for the tiled
+  // scan of many requests, which then needs no launch of its own to total the tiles); or nullptr
+  uint64_t *part;
   // What this pass leaves for a later call that wants to reuse its descriptors
   // (SG_F_REUSE_DESC): desc_tag = {gen, requests, items}.
   uint32_t *desc_tag;
@@ -304,6 +307,58 @@ __global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
   if (lane == 0) prep_finish(a, r, carry, bad);
 }
 
+// Several requests per wavefront, L = 16 or 32 lanes each (requests of a handful of fragments:
+// with a wavefront per request most lanes idle and the launch is as many wavefronts' worth of
+// dependent round trips -- table, header, scan -- as there are requests).  The scan runs over the
+// L lanes of a group; a request of more than L fragments takes more steps, and the wavefront
+// keeps stepping while any of its groups has fragments left.
+template <int L>
+__global__ __launch_bounds__(kBlock) void k_prep_group(PrepArgs a)
+{
+  constexpr uint32_t G = kWave / L;
+  __shared__ uint64_t group_tot[kWavesPerBlock * G];
+  prep_effective(a);
+  const uint32_t lane = threadIdx.x & (kWave - 1), gl = lane & (L - 1);
+  const uint32_t wave = blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  const uint32_t r = wave * G + lane / L;
+  const bool live = r < a.n_req;
+  uint32_t f0 = 0, f1 = 0, bad = 0;
+  uint64_t size = 0;
+  if (live) bad = prep_range(a, r, &f0, &f1, &size);
+  uint64_t carry = 0;
+  for (uint32_t base = f0; __any(base < f1); base += L) {
+    const uint32_t f = base + gl;
+    uint32_t len = 0, slot = 0;
+    if (f < f1) prep_item(a, f, f - f0, size, &slot, &len, &bad);
+    // inclusive scan over the group's lanes
+    uint32_t inc = len;
+#pragma unroll
+    for (int d = 1; d < L; d <<= 1) {
+      const uint32_t up = __shfl_up(inc, d, L);
+      if ((int)gl >= d) inc += up;
+    }
+    if (f < f1) {
+      u32x4 d = {slot, len, (uint32_t)(carry + (inc - len)), r};
+      a.desc[f] = d;
+    }
+    carry += __shfl(inc, L - 1, L);
+  }
+#pragma unroll
+  for (int m = L / 2; m >= 1; m >>= 1) bad |= __shfl_xor(bad, m, L);
+  if (live && gl == 0) prep_finish(a, r, carry, bad);
+  if (a.part) {
+    // the workgroup's requests added up: kWavesPerBlock * G consecutive requests per entry
+    if (gl == 0) group_tot[threadIdx.x / L] = live ? carry : 0;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint64_t t = 0;
+#pragma unroll
+      for (uint32_t k = 0; k < kWavesPerBlock * G; k++) t += group_tot[k];
+      a.part[blockIdx.x] = t;
+    }
+  }
+}
+
 // Scan of the request totals through the bump ring:
 //   ret = base + off; off = (off + size) % capacity   (src/p2p_rpc_tring.h:27-33)
 // Up to kScanTile requests: one workgroup does it all (k_req_scan).  Beyond:
@@ -313,6 +368,8 @@ __global__ __launch_bounds__(kBlock) void k_prep_wave(PrepArgs a)
 constexpr int kScanBlock = 1024;
 constexpr int kScanPerThread = 4;
 constexpr uint32_t kScanTile = kScanBlock * kScanPerThread;
+// fewest requests behind one entry of the tile-total scratch (k_prep_group<32>: two per wavefront)
+constexpr uint32_t kPartMin = 2 * kWavesPerBlock;
 
 // Exclusive scan of one tile; returns this thread's prefix for its first
 // request and leaves its requests' sizes in sz[].
@@ -382,6 +439,32 @@ __global__ __launch_bounds__(kScanBlock) void k_req_scan_local(PrepArgs a, uint6
 
 // Every tile sums the totals of the tiles before it (a few values) for its base
 // and scans again from there; the last tile also publishes the advanced cursor.
+// The tiled scan behind k_prep_group, in one launch: the sizes before a tile are the sums the
+// descriptor kernel's workgroups left (`per_part` requests each; a tile's worth of them is a few
+// hundred values), so no launch is spent on totalling the tiles.
+__global__ __launch_bounds__(kScanBlock) void k_req_scan_parts(PrepArgs a, uint32_t per_part, uint32_t n_tiles)
+{
+  __shared__ uint64_t wave_tot[kScanBlock / kWave];
+  const bool is_last = blockIdx.x == n_tiles - 1;
+  const uint32_t parts_before = blockIdx.x * (kScanTile / per_part);  // a tile is a whole number of parts
+  uint64_t s = 0, before = 0;
+  for (uint32_t q = threadIdx.x; q < parts_before; q += kScanBlock) s += a.part[q];
+  (void)block_exclusive_scan<kScanBlock>(s, wave_tot, &before);
+  const uint64_t c0 = *a.cursor % a.cap;
+  const uint64_t tile_base = (c0 + before % a.cap) % a.cap;
+  const uint32_t q0 = blockIdx.x * kScanTile + threadIdx.x * kScanPerThread;
+  uint64_t sz[kScanPerThread], tot;
+  const uint64_t ex = scan_tile(a, q0, sz, wave_tot, &tot);
+  scan_emit(a, q0, sz, (tile_base + ex % a.cap) % a.cap);
+  if (is_last && threadIdx.x == 0) {
+    const uint64_t batch_bytes = before + tot;
+    const uint64_t end = (c0 + batch_bytes % a.cap) % a.cap;
+    *a.next_cursor = end;
+    if (a.offsets_out) a.offsets_out[a.n_req] = end;
+    scan_check_batch(a, batch_bytes);
+  }
+}
+
 __global__ __launch_bounds__(kScanBlock) void k_req_scan_add(PrepArgs a, const uint64_t *tile_tot, uint32_t n_tiles)
 {
   __shared__ uint64_t wave_tot[kScanBlock / kWave];
@@ -1993,7 +2076,7 @@ __global__ __launch_bounds__(kBlock) void k_zero_words(uint32_t *p, uint32_t n)
 namespace {
 constexpr size_t kStaticDesc = sizeof(u32x4) * (size_t)SG_STATIC_MAX_FRAMES;
 constexpr size_t kStaticReq = sizeof(uint64_t) * (size_t)SG_STATIC_MAX_REQS;
-constexpr size_t kStaticTile = sizeof(uint64_t) * (SG_STATIC_MAX_REQS / kScanTile + 2);
+constexpr size_t kStaticTile = sizeof(uint64_t) * (SG_STATIC_MAX_REQS / kPartMin + 2);
 constexpr size_t kStaticWords = 256;  // cursors, staged cursors, status, refusal flag
 constexpr size_t kStaticBytes = kStaticDesc + 2 * kStaticReq + kStaticTile + kStaticWords;
 }  // namespace
@@ -2191,12 +2274,21 @@ int prof_drain(sg_hip_ctx *c)
 
 // Descriptor build: kernel shape by the average request, then the bump-ring
 // scan of the request totals where offsets are not plain multiples.
-int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs &p)
+int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs &args)
 {
   int rc = prof_begin(c, 0);
   if (rc != SG_OK) return rc;
+  PrepArgs p = args;
   const uint32_t avg = p.n_items / p.n_req;
-  if (avg <= 32) {
+  const bool tiled = p.packed && !p.fixed_offsets && !(p.n_req <= 2 * kScanTile || p.counts);
+  // requests per entry of the workgroup sums k_prep_group leaves for the tiled scan
+  const uint32_t per_part = avg <= 8 ? 4 * kWavesPerBlock : avg <= 16 ? 2 * kWavesPerBlock : 0;
+  if (tiled && per_part) p.part = sc.tile_tot;
+  if (avg <= 8) {
+    k_prep_group<16><<<(p.n_req + 4 * kWavesPerBlock - 1) / (4 * kWavesPerBlock), kBlock, 0, st>>>(p);
+  } else if (avg <= 16) {
+    k_prep_group<32><<<(p.n_req + 2 * kWavesPerBlock - 1) / (2 * kWavesPerBlock), kBlock, 0, st>>>(p);
+  } else if (avg <= 32) {
     k_prep_wave<<<(p.n_req + kWavesPerBlock - 1) / kWavesPerBlock, kBlock, 0, st>>>(p);
   } else if (avg <= 256) {
     k_prep_block<256><<<p.n_req, 256, 0, st>>>(p);
@@ -2208,10 +2300,14 @@ int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs
       k_req_scan<<<1, kScanBlock, 0, st>>>(p);
     } else {
       const uint32_t n_tiles = (p.n_req + kScanTile - 1) / kScanTile;
-      // (one launch in which every workgroup adds up the sizes before its tile by itself was
-      // measured at 32768 requests: 30.6 us for the descriptor pass against 26.9 us with these two)
-      k_req_scan_local<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot);
-      k_req_scan_add<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot, n_tiles);
+      if (p.part) {
+        k_req_scan_parts<<<n_tiles, kScanBlock, 0, st>>>(p, per_part, n_tiles);
+      } else {
+        // (one launch in which every workgroup adds up the REQUEST sizes before its tile by itself
+        // was measured at 32768 requests: 30.6 us for the descriptor pass against 26.9 us with these)
+        k_req_scan_local<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot);
+        k_req_scan_add<<<n_tiles, kScanBlock, 0, st>>>(p, sc.tile_tot, n_tiles);
+      }
     }
   }
   return prof_end(c);
@@ -2384,7 +2480,7 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMalloc(&c->desc, sizeof(u32x4) * (size_t)c->max_frames));
   HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
-  HIP_TRY(nullptr, hipMalloc(&c->tile_tot, sizeof(uint64_t) * ((size_t)c->max_reqs / kScanTile + 2)));
+  HIP_TRY(nullptr, hipMalloc(&c->tile_tot, sizeof(uint64_t) * ((size_t)c->max_reqs / kPartMin + 2)));
   HIP_TRY(nullptr, hipMalloc(&c->cursors, 7 * sizeof(uint64_t)));  // [4]: the two slot indices, [5], [6]: descriptor tag
   HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
   HIP_TRY(nullptr, hipMalloc(&c->csum_scratch, sizeof(uint32_t) * (size_t)c->max_frames * (kPartStride + 1)));
