@@ -1407,15 +1407,23 @@ __global__ __launch_bounds__(kBlock) void k_udp_finish(ScatterArgs a)
     n_items = live < n_items ? live : n_items;
   }
   if (item >= n_items) return;
-  if (!a.csum_valid[item]) return;
+  // everything this thread reads, asked for at once: the mark, the frame's eight words, its slot
+  const u32x4 *p = reinterpret_cast<const u32x4 *>(a.csum_part + (size_t)item * kPartStride);
+  const uint32_t valid = a.csum_valid[item];
+  const u32x4 lo = p[0], hi = p[1];
+  const uint32_t slot = FUSED ? a.rule.item_slot[item] : a.desc[item][0];
+  if (!valid) return;
   a.csum_valid[item] = 0;
-  const uint32_t *p = a.csum_part + (size_t)item * kPartStride;
-  uint32_t sum = 0;
-  for (uint32_t k = 0; k < a.pieces; k++) sum += p[k];  // each below 2^27
-  uint32_t s = fold16(fold16(p[a.pieces]) + fold16(sum));
+  const uint32_t w[kPartStride] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  uint32_t sum = 0, hdr = 0;
+#pragma unroll
+  for (uint32_t k = 0; k < kPartStride; k++) {
+    if (k < a.pieces) sum += w[k];  // each below 2^27
+    if (k == a.pieces) hdr = w[k];
+  }
+  uint32_t s = fold16(fold16(hdr) + fold16(sum));
   uint32_t c = (~s) & 0xffffu;
   if (c == 0) c = 0xffffu;
-  const uint32_t slot = FUSED ? a.rule.item_slot[item] : a.desc[item][0];
   // slots start at even addresses; the sums ran over the words as they lie in memory
   *reinterpret_cast<uint16_t *>(a.tx + (size_t)slot * a.tx_slot_size + 40) = (uint16_t)c;
 }
@@ -1688,9 +1696,19 @@ __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long 
   uint32_t first_empty = kRaBucket;
 #pragma unroll 1
   for (uint32_t h = 0; h < kRaBucket; h += 16) {
+    // Ordinary 16-byte loads, two keys each.  While arrivals are being filed a key only ever goes
+    // from empty to a token, so all a load that is behind the times can show is an empty cell that
+    // has just been taken -- and the claim below goes through atomicCAS, which then returns the
+    // taker (this thread's own token included).  Device-scope loads of single keys, 32 per arrival,
+    // made this kernel several times slower on bursts of many small requests.
     unsigned long long k[16];
+    const ulonglong2 *kp = reinterpret_cast<const ulonglong2 *>(a.keys + b + h);
 #pragma unroll
-    for (int j = 0; j < 16; j++) k[j] = ra_key(a.keys + b + h + j);
+    for (int j = 0; j < 8; j++) {
+      const ulonglong2 v = kp[j];
+      k[2 * j] = v.x;
+      k[2 * j + 1] = v.y;
+    }
 #pragma unroll
     for (int j = 0; j < 16; j++) {
       if (k[j] == token) return b + h + j;
@@ -1792,6 +1810,9 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
                                  (uint32_t)__shfl((int)(uint32_t)token, first, kWave);
     const bool mine = pending && token == t;
     const unsigned long long group = __ballot(mine);
+    // a burst that interleaves many requests: groups of one or two lanes, each a chain of
+    // dependent round trips that the other lanes sit out -- every lane for itself then
+    if (round == 0 && 8 * __popcll(group) < __popcll(waiting)) break;
     const uint32_t g_bytes = wave_sum(mine ? len : 0u);
     uint32_t c = kRaNoCell;
     if ((int)lane == first) {
