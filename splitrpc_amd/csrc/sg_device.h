@@ -533,6 +533,25 @@ __device__ __forceinline__ void group_run_begin(GroupRun<L> &r, const uint8_t *s
   }
 }
 
+// A run begun against a stand-in destination of the right phase (its loads are then under way
+// before the real destination is known) gets its destination here ...
+template <int L>
+__device__ __forceinline__ void group_run_rebase(GroupRun<L> &r, uint8_t *dst)
+{
+  const ptrdiff_t head = r.d - r.dst;
+  r.dst = dst;
+  r.d = dst + head;
+}
+
+// ... or is called off: nothing is stored.
+template <int L>
+__device__ __forceinline__ void group_run_cancel(GroupRun<L> &r)
+{
+  r.body = 0;
+  r.has_head = false;
+  r.has_tail = false;
+}
+
 // Returns this lane's share of the little-endian 16-bit word sum with CSUM.
 // Every lane of the wavefront has to call this (the realignment shifts values
 // across lanes); a group without a run passes body = 0 and no edge bytes.

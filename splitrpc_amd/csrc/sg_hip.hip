@@ -1479,11 +1479,10 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
   const uint32_t first_r = live ? a.rule.first[r] : 0u;
   uint32_t hs = 0;
   if (live && !from_template) hs = a.hdr_src_req ? a.hdr_src_req[r] : a.hdr_src_slot[item];
-  if (tslot >= a.rule.n_slots) bad |= kStBadSlot;
-  if (i == 0 && first_r != item) bad |= kStBadTable;
-  if (hs >= a.rx_n_slots) bad |= kStBadSlot;
-  if (live && bad && gl == 0) refuse(a.status, a.status_flag, bad);
-  // offsets depend on the item, the size and the cursor only: they are out before a bad frame is dropped
+  // Where the payload comes from depends on the frame's number alone, and so does the phase of
+  // where it goes when slots lie whole chunks apart: its loads are asked for now, a round trip
+  // before the tables above say which slot the frame goes to (and whether it goes at all).
+  const bool early = (a.tx_slot_size & 15u) == 0;
   uint64_t ro = 0;
   if (a.app.n_tensors == 0) {
     uint64_t c0 = sload(a.rule.cursor);
@@ -1492,15 +1491,34 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
     if (a.rule.single_wrap) o = o >= a.app.cap ? o - a.app.cap : o;
     else o %= a.app.cap;
     ro = o;
-    if (live && gl == 0 && a.rule.offsets_out) {
-      if (i == 0) a.rule.offsets_out[r] = ro;
-      if (item == n_req * per_req - 1) {
-        const uint64_t end = ro + a.rule.size;  // size <= capacity
-        a.rule.offsets_out[n_req] = end >= a.app.cap ? end - a.app.cap : end;
-      }
+  }
+  uint8_t *from = nullptr;
+  bool plain;
+  if (last_only && a.n_plan) {
+    // every group has the response's last frame: one plan entry for the wavefront
+    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(ScatterArgs, plan))) + (per_req - 1));
+    from = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
+    plain = live && len != 0 && fp[7] == 0;
+  } else {
+    plain = live && len != 0 && plain_target(a.app, ro, r, off, len, &from);
+  }
+  GroupRun<L> run;
+  if (early)
+    group_run_begin<L>(run, from, reinterpret_cast<uint8_t *>(((uintptr_t)a.tx + hl) & 15u), plain ? len : 0u, gl);
+  if (tslot >= a.rule.n_slots) bad |= kStBadSlot;
+  if (i == 0 && first_r != item) bad |= kStBadTable;
+  if (hs >= a.rx_n_slots) bad |= kStBadSlot;
+  if (live && bad && gl == 0) refuse(a.status, a.status_flag, bad);
+  // offsets depend on the item, the size and the cursor only: they are out before a bad frame is dropped
+  if (a.app.n_tensors == 0 && live && gl == 0 && a.rule.offsets_out) {
+    if (i == 0) a.rule.offsets_out[r] = ro;
+    if (item == n_req * per_req - 1) {
+      const uint64_t end = ro + a.rule.size;  // size <= capacity
+      a.rule.offsets_out[n_req] = end >= a.app.cap ? end - a.app.cap : end;
     }
   }
   live = live && !bad;
+  plain = plain && live;
   uint8_t *slot = a.tx + (size_t)tslot * a.tx_slot_size;
   HdrFields hf{hl, a.ref64, a.flags, i, per_req, len, 0, 0, 0};
   const uint8_t *hin;
@@ -1517,18 +1535,12 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
   // header words and payload chunks are fetched together; a TX slot that is its own header
   // source still holds the request header then (the payload goes past the header only)
   const SmallHdr sh = small_hdr_fetch(hin, gl, hl, !from_template, live && gl < 16);
-  uint8_t *from = nullptr;
-  bool plain;
-  if (last_only && a.n_plan) {
-    // every group has the response's last frame: one plan entry for the wavefront
-    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(ScatterArgs, plan))) + (per_req - 1));
-    from = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
-    plain = live && len != 0 && fp[7] == 0;
+  if (early) {
+    group_run_rebase<L>(run, slot + hl);
+    if (!plain) group_run_cancel<L>(run);  // a frame the tables have just ruled out
   } else {
-    plain = live && len != 0 && plain_target(a.app, ro, r, off, len, &from);
+    group_run_begin<L>(run, from, slot + hl, plain ? len : 0u, gl);
   }
-  GroupRun<L> run;
-  group_run_begin<L>(run, from, slot + hl, plain ? len : 0u, gl);
   uint32_t acc = group_run_end<L, FULL_CSUM>(run, gl);
   if (live && len != 0 && !plain) {
     // across an arena end or a tensor boundary: byte by byte
