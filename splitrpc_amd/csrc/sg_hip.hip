@@ -3248,9 +3248,12 @@ int ra_state(sg_hip_ctx *c, RaArgs *r, bool *fresh)
                        kRaWords * 4 + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 256;
   *fresh = false;
   if (!c->ra_mem) {
+    // the small allocation first: a context never holds the state without its pinned counts
+    if (!c->h_counts) {
+      HIP_TRY(c, hipHostMalloc((void **)&c->h_counts, 4 * sizeof(uint32_t), hipHostMallocDefault));
+      memset(c->h_counts, 0, 4 * sizeof(uint32_t));
+    }
     HIP_TRY(c, hipMalloc(&c->ra_mem, bytes));
-    HIP_TRY(c, hipHostMalloc((void **)&c->h_counts, 4 * sizeof(uint32_t), hipHostMallocDefault));
-    memset(c->h_counts, 0, 4 * sizeof(uint32_t));
     c->ra_cells = cells;
     c->ra_records = records;
     *fresh = true;

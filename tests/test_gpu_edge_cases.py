@@ -397,6 +397,31 @@ def test_odd_arena_base_and_tensor_major_split(ctx):
             assert not bb[:shift].any() and not bb[shift + e.size:].any()  # nothing written outside
 
 
+@pytest.mark.parametrize("tensor_sizes", [(1024, 1024), (1008, 1040), (1000, 1056), (16, 2032), (700, 700, 648)])
+def test_fragment_between_two_tensors_with_the_rule_declared(ctx, tensor_sizes):
+    """Requests of one size cut by the rule into tensor-major buffers: the
+    fragment that runs from one tensor into the next moves as one run with a
+    break in its destination where both shares lie on chunk boundaries, as two
+    runs where they do not, byte by byte across three tensors -- at tensor
+    bases of several phases, so that all of these occur."""
+    size = int(sum(tensor_sizes))
+    n = 37
+    w = synth.make_custom([size] * n, [64] * n, order="shuffle_all", seed=11, in_tensor_sizes=tensor_sizes)
+    dw = DeviceWorkload(w)
+    exp, _, _ = expected_gather(w)
+    for shift in (0, 8, 3):
+        backing = [torch.full((n * s + 64,), 0xEE, dtype=torch.uint8, device=DEV) for s in tensor_sizes]
+        tensors = [b[shift:shift + n * s] for b, s in zip(backing, tensor_sizes)]
+        app = AppRef(tensors=tensors, sizes=list(tensor_sizes))
+        ctx.gather_batch(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, app,
+                         flags=capi.F_RULE_FRAGS, fixed_req_size=size, mtu=w.mtu)
+        for t, e, b in zip(tensors, exp, backing):
+            got = t.cpu().numpy()
+            assert np.array_equal(got, e), f"shift {shift}: " + first_diff(got, e)
+            bb = b.cpu().numpy()
+            assert (bb[:shift] == 0xEE).all() and (bb[shift + e.size:] == 0xEE).all()  # nothing written outside
+
+
 # ---------------------------------------------------------------- refused input
 
 def test_bad_slot_index_refuses_the_whole_batch(ctx):
