@@ -1637,11 +1637,14 @@ __global__ __launch_bounds__(kBlock) void k_swap_hdrs(const uint64_t *hdr_ptrs, 
 // progress by itself.
 
 constexpr uint32_t kRaBucket = 32;
+static_assert(kRaBucket == 32, "ra_find_cell takes a token's first cell from the top five bits of its hash");
 constexpr uint32_t kRaNoCell = 0xffffffffu;
 constexpr uint32_t kRaNoRec = 0xffffffffu;
 constexpr int kRaBlock = 1024;
 // device words of the reassembly state
-enum { kRaHead = 0, kRaTail, kRaEpoch, kRaInFlight, kRaClaims, kRaDropped, kRaOverflow, kRaEvicted, kRaWords = 16 };
+// kRaHeadSeen: where k_ra_scan last saw the head -- how far it has moved since is the number of
+// cells claimed in between
+enum { kRaHead = 0, kRaTail, kRaEpoch, kRaInFlight, kRaHeadSeen, kRaDropped, kRaOverflow, kRaEvicted, kRaWords = 16 };
 
 struct RaArgs {
   const uint8_t *ring;
@@ -1656,8 +1659,8 @@ struct RaArgs {
   uint32_t max_req, max_frag;  // room in the output tables
   // request table: cells
   unsigned long long *keys;
-  unsigned long long *bytes;
-  uint32_t *cnt, *want, *last, *rec, *seen;
+  unsigned long long *acc;  // fragments so far << 40 | payload bytes so far: one atomic addition per arrival
+  uint32_t *want, *last, *rec, *seen;
   // record pool
   unsigned long long *tab;  // records x SG_MAX_BI_SIZE entries: slot | length << 32
   uint32_t *free_ring;
@@ -1681,6 +1684,20 @@ __device__ __forceinline__ uint32_t ra_n(const RaArgs &a)
   return dev_count(a.n_dev, 0, a.n);
 }
 
+// A cell's fragment count and byte total in one word (a request has at most SG_MAX_BI_SIZE
+// fragments and far fewer than 2^40 bytes): device-scope atomics are what a burst of many small
+// requests pays for, one per arrival instead of two.
+constexpr int kRaCntShift = 40;
+__device__ __forceinline__ unsigned long long ra_pack(uint32_t n, unsigned long long bytes)
+{
+  return ((unsigned long long)n << kRaCntShift) + bytes;
+}
+__device__ __forceinline__ uint32_t ra_cnt(unsigned long long acc) { return (uint32_t)(acc >> kRaCntShift); }
+__device__ __forceinline__ unsigned long long ra_bytes(unsigned long long acc)
+{
+  return acc & ((1ull << kRaCntShift) - 1ull);
+}
+
 __device__ __forceinline__ uint32_t ra_hash(unsigned long long k)
 {
   k ^= k >> 33;
@@ -1695,24 +1712,29 @@ __device__ __forceinline__ unsigned long long ra_key(const unsigned long long *p
 }
 
 // Find or claim the cell of `token`.  The whole bucket is read first: the
-// request may sit behind cells that have emptied since it came in.  Only then
-// is an empty cell claimed, walking up from the lowest one seen empty and
-// trying every empty cell on the way; cells below that one were taken when
-// they were read and stay taken while arrivals are being filed, so two threads
-// that bring the same new token end up in the same cell whatever else is
-// claimed around them.
+// request may sit anywhere in it (cells empty as requests complete).  Only then
+// is an empty cell claimed.  Every token walks the bucket in an order of its
+// own -- cyclically from a cell its hash picks -- starting at the first cell of
+// that order it has seen empty and trying every empty cell on the way; cells
+// before that one in the order were taken when they were read and stay taken
+// while arrivals are being filed, so two threads that bring the same new token
+// end up in the same cell whatever else is claimed around them.  (With one
+// order for all tokens -- lowest cell first -- the new requests of a burst that
+// share a bucket queued up on its lowest empty cells, one failed
+// compare-and-swap round trip after the other.)
 __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long long token, bool *claimed)
 {
-  const uint32_t b = (ra_hash(token) & a.bmask) * kRaBucket;
+  const uint32_t hash = ra_hash(token);
+  const uint32_t b = (hash & a.bmask) * kRaBucket;
+  const uint32_t start = hash >> 27;  // kRaBucket == 32: the top five bits, the bucket takes the low ones
   *claimed = false;
-  uint32_t first_empty = kRaBucket;
+  uint32_t first_rank = kRaBucket;  // place in this token's order of the first cell seen empty
 #pragma unroll 1
   for (uint32_t h = 0; h < kRaBucket; h += 16) {
     // Ordinary 16-byte loads, two keys each.  While arrivals are being filed a key only ever goes
     // from empty to a token, so all a load that is behind the times can show is an empty cell that
     // has just been taken -- and the claim below goes through atomicCAS, which then returns the
-    // taker (this thread's own token included).  Device-scope loads of single keys, 32 per arrival,
-    // made this kernel several times slower on bursts of many small requests.
+    // taker (this thread's own token included).
     unsigned long long k[16];
     const ulonglong2 *kp = reinterpret_cast<const ulonglong2 *>(a.keys + b + h);
 #pragma unroll
@@ -1724,12 +1746,14 @@ __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long 
 #pragma unroll
     for (int j = 0; j < 16; j++) {
       if (k[j] == token) return b + h + j;
-      if (k[j] == 0ull && first_empty == kRaBucket) first_empty = h + j;
+      const uint32_t rank = (h + j - start) & (kRaBucket - 1);
+      if (k[j] == 0ull && rank < first_rank) first_rank = rank;
     }
   }
 #pragma unroll 1
-  for (uint32_t j = first_empty; j < kRaBucket; j++) {
-    unsigned long long k = j == first_empty ? 0ull : ra_key(a.keys + b + j);
+  for (uint32_t rank = first_rank; rank < kRaBucket; rank++) {
+    const uint32_t j = (start + rank) & (kRaBucket - 1);
+    unsigned long long k = rank == first_rank ? 0ull : ra_key(a.keys + b + j);
     if (k == 0ull) {
       k = atomicCAS(&a.keys[b + j], 0ull, token);
       if (k == 0ull) {
@@ -1742,25 +1766,39 @@ __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long 
   return kRaNoCell;  // bucket full
 }
 
-// Records for the cells the lanes of this wavefront have just claimed: one
-// addition to the ring's head for the whole wavefront (an addition per claim, let
-// alone a compare-and-swap loop, would queue every new request of a burst on
-// one word).  The tail does not move during the kernel that takes records
-// (returns happen in k_ra_emit), so a position at or beyond the tail read here
-// means the pool is exhausted: the cell then gets no record, the call is
-// refused, and k_ra_scan puts the head back to the tail.
-__device__ __forceinline__ void ra_open_cells(const RaArgs &a, bool claimed, uint32_t cell, uint32_t lane)
+// Positions on a ring word for a whole workgroup with ONE addition: every wavefront says how many it
+// needs and gets its first.  (A returning addition per wavefront on a word that thousands of wavefronts
+// on eight XCDs add to takes some 70 ns, one after the other: 0.29 ms of a 0.35-ms k_ra_insert on a
+// burst of 131072 new requests.)  Every thread of the workgroup has to call this.
+constexpr int kRaTakeBlock = 1024;
+__device__ __forceinline__ uint32_t ra_block_take(uint32_t *word, uint32_t n_wave, uint32_t *lds)
+{
+  constexpr uint32_t kWaves = kRaTakeBlock / kWave;
+  const uint32_t wv = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wv] = n_wave;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t tot = 0;
+    for (uint32_t w = 0; w < kWaves; w++) {
+      const uint32_t t = lds[w];
+      lds[w] = tot;
+      tot += t;
+    }
+    lds[kWaves] = tot ? atomicAdd(word, tot) : 0u;
+  }
+  __syncthreads();
+  return lds[kWaves] + lds[wv];
+}
+
+// Records for the cells the threads of this workgroup have just claimed: one addition to the
+// ring's head for all of them.  The tail does not move during the kernel that takes records
+// (returns happen in k_ra_emit), so a position at or beyond the tail read here means the pool is
+// exhausted: the cell then gets no record, the call is refused, and k_ra_scan puts the head back
+// to the tail.
+__device__ __forceinline__ void ra_open_cells(const RaArgs &a, bool claimed, uint32_t cell, uint32_t lane, uint32_t *lds)
 {
   const unsigned long long cl = __ballot(claimed);
-  if (!cl) return;
-  const uint32_t n = (uint32_t)__popcll(cl);
-  const int leader = __ffsll((long long)cl) - 1;
-  uint32_t base = 0;
-  if ((int)lane == leader) {
-    base = atomicAdd(&a.words[kRaHead], n);
-    atomicAdd(&a.words[kRaClaims], n);
-  }
-  base = (uint32_t)__shfl((int)base, leader, kWave);
+  const uint32_t base = ra_block_take(&a.words[kRaHead], (uint32_t)__popcll(cl), lds);
   if (claimed) {
     const uint32_t h = base + (uint32_t)__popcll(cl & ((1ull << lane) - 1ull));
     const uint32_t tail = a.words[kRaTail];
@@ -1777,10 +1815,11 @@ __device__ __forceinline__ void ra_open_cells(const RaArgs &a, bool claimed, uin
 // (bursts that interleave many requests).
 constexpr int kRaRounds = 4;
 
-__global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
+__global__ __launch_bounds__(kRaTakeBlock) void k_ra_insert(RaArgs a)
 {
+  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
   const uint32_t n = ra_n(a);
-  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t i = blockIdx.x * kRaTakeBlock + threadIdx.x;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const bool in_range = i < n;
   const uint32_t epoch = a.words[kRaEpoch];  // advanced by k_ra_scan, behind this kernel
@@ -1832,8 +1871,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
       c = ra_find_cell(a, t, &claimed);
       if (c != kRaNoCell) {
         if (claimed) opened = c;
-        atomicAdd(&a.cnt[c], (uint32_t)__popcll(group));
-        atomicAdd(&a.bytes[c], (unsigned long long)g_bytes);
+        atomicAdd(&a.acc[c], ra_pack((uint32_t)__popcll(group), g_bytes));
         atomicMax(&a.last[c], i - lane + (63u - (uint32_t)__clzll((long long)group)));
         if (!a.ref64) a.want[c] = want;  // every fragment of a request says the same
         a.seen[c] = epoch;
@@ -1850,15 +1888,14 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
     cell = ra_find_cell(a, token, &claimed);
     if (cell != kRaNoCell) {
       if (claimed) opened = cell;
-      atomicAdd(&a.cnt[cell], 1u);
-      atomicAdd(&a.bytes[cell], (unsigned long long)len);
+      atomicAdd(&a.acc[cell], ra_pack(1u, len));
       atomicMax(&a.last[cell], i);
       if (!a.ref64) a.want[cell] = want;
       a.seen[cell] = epoch;
     }
   }
   // the cells this wavefront has claimed get their records (a lane claims one cell at most)
-  ra_open_cells(a, opened != kRaNoCell, opened, lane);
+  ra_open_cells(a, opened != kRaNoCell, opened, lane, take);
   if (in_range) {
     a.arr_cell[i] = cell;
     a.arr_len[i] = len;
@@ -1872,7 +1909,7 @@ __global__ __launch_bounds__(256) void k_ra_insert(RaArgs a)
 
 __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell)
 {
-  return a.ref64 ? a.bytes[cell] == a.req_size : a.cnt[cell] == a.want[cell];
+  return a.ref64 ? ra_bytes(a.acc[cell]) == a.req_size : ra_cnt(a.acc[cell]) == a.want[cell];
 }
 
 __global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
@@ -1892,7 +1929,7 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
       } else {
         refuse(a.status, a.status_flag, kStBadTable);  // beyond what a request's tables hold (src/p2p_bufs.h:10)
       }
-      const uint32_t cnt = a.cnt[cell];
+      const uint32_t cnt = ra_cnt(a.acc[cell]);
       if (a.last[cell] == i && ra_complete(a, cell)) {
         if (cnt <= SG_MAX_BI_SIZE) pack = (1ull << 32) | cnt;
         else refuse(a.status, a.status_flag, kStBadTable);
@@ -1929,13 +1966,17 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
       n_req = n_frag = 0;
     }
     a.words[kRaOverflow] = overflow;
+    // cells claimed since the last call: as far as the head has moved
+    uint32_t head = a.words[kRaHead];
+    const uint32_t claims = head - a.words[kRaHeadSeen];
     // claims beyond the pool ran the head past the tail
-    if ((int32_t)(a.words[kRaHead] - a.words[kRaTail]) > 0) a.words[kRaHead] = a.words[kRaTail];
+    if ((int32_t)(head - a.words[kRaTail]) > 0) head = a.words[kRaTail];
+    a.words[kRaHead] = head;
+    a.words[kRaHeadSeen] = head;
     a.req_first[n_req] = n_frag;
-    const uint32_t in_flight = a.words[kRaInFlight] + a.words[kRaClaims] - n_req;
+    const uint32_t in_flight = a.words[kRaInFlight] + claims - n_req;
     const uint32_t dropped = a.words[kRaDropped];
     a.words[kRaInFlight] = in_flight;
-    a.words[kRaClaims] = 0;
     a.words[kRaDropped] = 0;
     a.words[kRaEpoch] += 1;
     const uint32_t c[4] = {n_req, n_frag, dropped, in_flight};
@@ -1950,10 +1991,11 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
 // into the output tables in sequence order, the record is emptied and returned
 // to the free ring, the cell is emptied.  The request's rank and first fragment
 // index hang on that arrival (arr_pack there plus its workgroup's scanned total).
-__global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
+__global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
 {
+  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
   const uint32_t n = ra_n(a);
-  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t i = blockIdx.x * kRaTakeBlock + threadIdx.x;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const bool overflow = a.words[kRaOverflow] != 0;
   uint32_t cell = kRaNoCell;
@@ -1968,19 +2010,15 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
     if (cell != kRaNoCell && !completes) a.last[cell] = 0;
   }
   unsigned long long todo = __ballot(completes);
-  // reap_rr for all of this wavefront's requests: one addition to the ring's tail
-  uint32_t tail0 = 0;
-  if (todo) {
-    if (lane == 0) tail0 = atomicAdd(&a.words[kRaTail], (uint32_t)__popcll(todo));
-    tail0 = (uint32_t)__shfl((int)tail0, 0, kWave);
-  }
+  // reap_rr for all of this workgroup's requests: one addition to the ring's tail
+  const uint32_t tail0 = ra_block_take(&a.words[kRaTail], (uint32_t)__popcll(todo), take);
   // requests of a few fragments are handed over by the completing lane itself, all such lanes
   // at once; the wavefront then walks the larger ones together
   constexpr uint32_t kOwn = 8;
   const uint32_t my_rank = (uint32_t)__popcll(todo & ((1ull << lane) - 1ull));
   bool own = false;
   if (completes) {
-    const uint32_t cnt = a.cnt[cell];
+    const uint32_t cnt = ra_cnt(a.acc[cell]);
     own = cnt <= kOwn;
     if (own) {
       const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v, rc = a.rec[cell];
@@ -2000,8 +2038,7 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
       if (a.req_token) a.req_token[r] = a.keys[cell];
       if (a.req_hdr_slot) a.req_hdr_slot[r] = (uint32_t)e[0];
       a.free_ring[(tail0 + my_rank) & a.rmask] = rc;
-      a.cnt[cell] = 0;
-      a.bytes[cell] = 0;
+      a.acc[cell] = 0;
       a.last[cell] = 0;
       a.want[cell] = 0;
       a.rec[cell] = kRaNoRec;
@@ -2017,7 +2054,7 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
     const uint32_t c = (uint32_t)__shfl((int)cell, l, kWave);
     const uint32_t r = (uint32_t)__shfl((int)(uint32_t)(v >> 32), l, kWave);
     const uint32_t first = (uint32_t)__shfl((int)(uint32_t)v, l, kWave);
-    const uint32_t rc = a.rec[c], cnt = a.cnt[c];
+    const uint32_t rc = a.rec[c], cnt = ra_cnt(a.acc[c]);
     unsigned long long *t = a.tab + (size_t)rc * SG_MAX_BI_SIZE;
     for (uint32_t j = lane; j < cnt; j += kWave) {
       const unsigned long long e = t[j];
@@ -2033,8 +2070,7 @@ __global__ __launch_bounds__(256) void k_ra_emit(RaArgs a)
     if (lane == 0) {
       // the record goes back to the free ring, the token leaves the table
       a.free_ring[(tail0 + nth) & a.rmask] = rc;
-      a.cnt[c] = 0;
-      a.bytes[c] = 0;
+      a.acc[c] = 0;
       a.last[c] = 0;
       a.want[c] = 0;
       a.rec[c] = kRaNoRec;
@@ -2049,8 +2085,8 @@ __global__ __launch_bounds__(256) void k_ra_reset(RaArgs a, uint32_t cells, uint
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i < cells) {
     a.keys[i] = 0;
-    a.bytes[i] = 0;
-    a.cnt[i] = a.want[i] = a.last[i] = a.seen[i] = 0;
+    a.acc[i] = 0;
+    a.want[i] = a.last[i] = a.seen[i] = 0;
     a.rec[i] = kRaNoRec;
   }
   if (i < records) a.free_ring[i] = (uint32_t)i;
@@ -2079,8 +2115,7 @@ __global__ __launch_bounds__(256) void k_ra_evict(RaArgs a, uint32_t cells, uint
       const uint32_t tl = atomicAdd(&a.words[kRaTail], 1u);
       a.free_ring[tl & a.rmask] = rc;
     }
-    a.cnt[c] = 0;
-    a.bytes[c] = 0;
+    a.acc[c] = 0;
     a.last[c] = 0;
     a.want[c] = 0;
     a.rec[c] = kRaNoRec;
@@ -3244,7 +3279,7 @@ int ra_state(sg_hip_ctx *c, RaArgs *r, bool *fresh)
   const uint32_t cells = pow2_at_least(4ull * c->max_reqs < 2 * kRaBucket ? 2 * kRaBucket : 4ull * c->max_reqs);
   const uint32_t records = pow2_at_least(c->max_reqs);
   const size_t n_blk = (n_max + kRaBlock - 1) / kRaBlock + 1;
-  const size_t bytes = (size_t)cells * (8 + 8 + 5 * 4) + (size_t)records * SG_MAX_BI_SIZE * 8 + (size_t)records * 4 +
+  const size_t bytes = (size_t)cells * (8 + 8 + 4 * 4) + (size_t)records * SG_MAX_BI_SIZE * 8 + (size_t)records * 4 +
                        kRaWords * 4 + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 256;
   *fresh = false;
   if (!c->ra_mem) {
@@ -3261,11 +3296,10 @@ int ra_state(sg_hip_ctx *c, RaArgs *r, bool *fresh)
   memset(r, 0, sizeof *r);
   uint8_t *m = static_cast<uint8_t *>(c->ra_mem);
   r->keys = reinterpret_cast<unsigned long long *>(m); m += (size_t)cells * 8;
-  r->bytes = reinterpret_cast<unsigned long long *>(m); m += (size_t)cells * 8;
+  r->acc = reinterpret_cast<unsigned long long *>(m); m += (size_t)cells * 8;
   r->tab = reinterpret_cast<unsigned long long *>(m); m += (size_t)records * SG_MAX_BI_SIZE * 8;
   r->arr_pack = reinterpret_cast<unsigned long long *>(m); m += (size_t)n_max * 8;
   r->blk = reinterpret_cast<unsigned long long *>(m); m += n_blk * 8;
-  r->cnt = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
   r->want = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
   r->last = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
   r->rec = reinterpret_cast<uint32_t *>(m); m += (size_t)cells * 4;
@@ -3360,15 +3394,15 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *coun
   r.req_hdr_slot = a->req_hdr_slot;
   r.counts_out = a->counts_out;
 
-  const uint32_t g256 = (a->n_arrivals + 255) / 256;
+  const uint32_t g_take = (a->n_arrivals + kRaTakeBlock - 1) / kRaTakeBlock;
   rc = prof_begin(c, 5);
   if (rc != SG_OK) return rc;
   if (a->n_arrivals) {
-    k_ra_insert<<<g256, 256, 0, c->stream>>>(r);
+    k_ra_insert<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
     k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
   }
   k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);  // an empty burst still leaves its counts
-  if (a->n_arrivals) k_ra_emit<<<g256, 256, 0, c->stream>>>(r);
+  if (a->n_arrivals) k_ra_emit<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
   rc = prof_end(c);
   if (rc != SG_OK) return rc;
   rc = finish(c, a->flags);

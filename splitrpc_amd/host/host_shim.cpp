@@ -330,6 +330,8 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
         rem -= cur;
         r->rr_append_mbuf((uintptr_t)slot, (uintptr_t)slot, (uintptr_t)(slot + hl), cur);
       }
+      // device-to-device copies do not make the host wait: the engine's stream does not know of them
+      (void)hipStreamSynchronize(nullptr);
       engine.swap_hdrs(r, profile, resp_size, mtu, flags & ~SG_F_UDP_CSUM_FULL);
       if (engine.last_rc != SG_OK) return -12;
       engine.scatter(r, slots[k]->h_stub);
