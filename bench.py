@@ -375,6 +375,10 @@ def main() -> int:
         print("bench.py needs a GPU (cuda:0)", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+    # no collector pauses inside timed loops (a full collection over this process's objects takes
+    # tens of milliseconds, and a loop of a few hundred microsecond-sized calls can trigger one)
+    import gc
+    gc.disable()
     extra = (capi.F_NO_XCD_REMAP if a.no_remap else 0) | (capi.F_NO_SMALL if a.no_small else 0)
     bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
     prof = synth.HDR_REF64 if a.ref64 else synth.HDR_BL58
@@ -445,6 +449,22 @@ def main() -> int:
     for b in range(0, n_b, 64):
         ctx.reassemble(dw0.rx, dw0.arrivals[b:b + 64], min(64, n_b - b), ra_fs, ra_fl, ra_rf, **ra_kw)
     reassembly["us_per_burst_of_64"] = round((time.perf_counter() - t0) / max(1, (n_b + 63) // 64) * 1e6, 2)
+    ctx.reassemble_reset()
+    # the same bursts queued without waiting for each one's counts (they stay on the device, where the
+    # gather reads them): what a burst costs the stream
+    queued = [ctx.reassemble_args(dw0.rx, dw0.arrivals[b:b + 64], min(64, n_b - b), ra_fs, ra_fl, ra_rf,
+                                  flags=capi.F_ASYNC, **ra_kw) for b in range(0, n_b, 64)]
+    for qa in queued[:8]:
+        ctx.reassemble_raw(qa)
+    ctx.sync()
+    ctx.reassemble_reset()
+    t0 = time.perf_counter()
+    for k, qa in enumerate(queued):
+        ctx.reassemble_raw(qa)
+        if k % 100 == 99:
+            ctx.sync()  # a caller takes the counts in now and then
+    ctx.sync()
+    reassembly["us_per_burst_of_64_queued"] = round((time.perf_counter() - t0) / max(1, len(queued)) * 1e6, 2)
     ctx.reassemble_reset()
     del ra_fs, ra_fl, ra_rf
 

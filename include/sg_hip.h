@@ -225,7 +225,7 @@ typedef struct sg_scatter_args {
    * frame i of request r gets a copy of template r with token req_token[r]
    * (the template's own when req_token is NULL), seq_num / frag_idx i,
    * lengths and sums.  Nothing is swapped and hdr_src_slot is not read. */
-  const uint8_t *hdr_templates; /* device, n_req * 64 bytes, or NULL: swap request headers */
+  const uint8_t *hdr_templates; /* device, n_req * 64 bytes at an even address, or NULL: swap request headers */
   const uint64_t *req_token;    /* device, n_req, or NULL */
   /* One header source per request instead of one per frame: every frame of
    * response r answers the header in RX slot hdr_src_req[r] (what

@@ -1815,11 +1815,26 @@ __device__ __forceinline__ void ra_open_cells(const RaArgs &a, bool claimed, uin
 // (bursts that interleave many requests).
 constexpr int kRaRounds = 4;
 
-__global__ __launch_bounds__(kRaTakeBlock) void k_ra_insert(RaArgs a)
+// The four steps of a call as functions of the arrival's index: launched as four kernels, or --
+// a burst that fits one workgroup, which is what a NIC delivers -- one behind the other in ONE
+// kernel (FUSED), with workgroup barriers where the kernel boundaries were.  What a step reads of
+// what other threads left through device-scope atomics in an earlier step of the same kernel
+// (counts and bytes, last positions, keys, ring words) it then reads with device-scope loads: an
+// ordinary load could still find the line as a cache held it before the atomic went to memory.
+template <bool FUSED>
+__device__ __forceinline__ unsigned long long ra_acc(const RaArgs &a, uint32_t cell)
 {
-  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
+  return FUSED ? __hip_atomic_load(a.acc + cell, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : a.acc[cell];
+}
+template <bool FUSED>
+__device__ __forceinline__ uint32_t ra_word(const uint32_t *p)
+{
+  return FUSED ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
+}
+
+__device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint32_t *take)
+{
   const uint32_t n = ra_n(a);
-  const uint32_t i = blockIdx.x * kRaTakeBlock + threadIdx.x;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const bool in_range = i < n;
   const uint32_t epoch = a.words[kRaEpoch];  // advanced by k_ra_scan, behind this kernel
@@ -1907,16 +1922,22 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_insert(RaArgs a)
   if (lane == 0 && lost) atomicAdd(&a.words[kRaDropped], (uint32_t)__popcll(lost));
 }
 
-__device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell)
+__global__ __launch_bounds__(kRaTakeBlock) void k_ra_insert(RaArgs a)
 {
-  return a.ref64 ? ra_bytes(a.acc[cell]) == a.req_size : ra_cnt(a.acc[cell]) == a.want[cell];
+  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
+  ra_insert_step(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take);
 }
 
-__global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
+__device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell, unsigned long long acc)
 {
-  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  return a.ref64 ? ra_bytes(acc) == a.req_size : ra_cnt(acc) == a.want[cell];
+}
+
+// Returns the workgroup's packed (requests, fragments) total.
+template <bool FUSED>
+__device__ __forceinline__ uint64_t ra_flag_step(const RaArgs &a, uint32_t i, uint64_t *wave_tot)
+{
   const uint32_t n = ra_n(a);
-  const uint32_t i = blockIdx.x * kRaBlock + threadIdx.x;
   unsigned long long pack = 0;
   if (i < n) {
     const uint32_t cell = a.arr_cell[i];
@@ -1929,8 +1950,9 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
       } else {
         refuse(a.status, a.status_flag, kStBadTable);  // beyond what a request's tables hold (src/p2p_bufs.h:10)
       }
-      const uint32_t cnt = ra_cnt(a.acc[cell]);
-      if (a.last[cell] == i && ra_complete(a, cell)) {
+      const unsigned long long acc = ra_acc<FUSED>(a, cell);
+      const uint32_t cnt = ra_cnt(acc);
+      if (ra_word<FUSED>(a.last + cell) == i && ra_complete(a, cell, acc)) {
         if (cnt <= SG_MAX_BI_SIZE) pack = (1ull << 32) | cnt;
         else refuse(a.status, a.status_flag, kStBadTable);
       }
@@ -1939,7 +1961,49 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
   uint64_t tot;
   const uint64_t ex = block_exclusive_scan<kRaBlock>(pack, wave_tot, &tot);
   if (i < n) a.arr_pack[i] = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
+  return tot;
+}
+
+__global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
+{
+  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  const uint64_t tot = ra_flag_step<false>(a, blockIdx.x * kRaBlock + threadIdx.x, wave_tot);
   if (threadIdx.x == 0) a.blk[blockIdx.x] = tot;
+}
+
+// One thread closes the call: counts, the free ring's head, the epoch.  `run` is the packed
+// (requests, fragments) total of the call.  Returns whether the output tables overflowed.
+template <bool FUSED>
+__device__ __forceinline__ uint32_t ra_scan_finish(const RaArgs &a, uint64_t run)
+{
+  uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
+  uint32_t overflow = 0;
+  if (n_req > a.max_req || n_frag > a.max_frag) {
+    // the output tables cannot take what completed: nothing is emitted, the requests stay parked
+    refuse(a.status, a.status_flag, kStBadTable);
+    overflow = 1;
+    n_req = n_frag = 0;
+  }
+  a.words[kRaOverflow] = overflow;
+  // cells claimed since the last call: as far as the head has moved
+  uint32_t head = ra_word<FUSED>(a.words + kRaHead);
+  const uint32_t claims = head - a.words[kRaHeadSeen];
+  // claims beyond the pool ran the head past the tail
+  if ((int32_t)(head - a.words[kRaTail]) > 0) head = a.words[kRaTail];
+  a.words[kRaHead] = head;
+  a.words[kRaHeadSeen] = head;
+  a.req_first[n_req] = n_frag;
+  const uint32_t in_flight = a.words[kRaInFlight] + claims - n_req;
+  const uint32_t dropped = ra_word<FUSED>(a.words + kRaDropped);
+  a.words[kRaInFlight] = in_flight;
+  a.words[kRaDropped] = 0;
+  a.words[kRaEpoch] += 1;
+  const uint32_t c[4] = {n_req, n_frag, dropped, in_flight};
+  for (int k = 0; k < 4; k++) {
+    if (a.counts_out) a.counts_out[k] = c[k];
+    a.counts_host[k] = c[k];  // straight into pinned host memory: nothing to copy back
+  }
+  return overflow;
 }
 
 __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
@@ -1956,48 +2020,18 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
     if (b < n_blocks) a.blk[b] = run + ex;
     run += tot;
   }
-  if (threadIdx.x == 0) {
-    uint32_t n_req = (uint32_t)(run >> 32), n_frag = (uint32_t)run;
-    uint32_t overflow = 0;
-    if (n_req > a.max_req || n_frag > a.max_frag) {
-      // the output tables cannot take what completed: nothing is emitted, the requests stay parked
-      refuse(a.status, a.status_flag, kStBadTable);
-      overflow = 1;
-      n_req = n_frag = 0;
-    }
-    a.words[kRaOverflow] = overflow;
-    // cells claimed since the last call: as far as the head has moved
-    uint32_t head = a.words[kRaHead];
-    const uint32_t claims = head - a.words[kRaHeadSeen];
-    // claims beyond the pool ran the head past the tail
-    if ((int32_t)(head - a.words[kRaTail]) > 0) head = a.words[kRaTail];
-    a.words[kRaHead] = head;
-    a.words[kRaHeadSeen] = head;
-    a.req_first[n_req] = n_frag;
-    const uint32_t in_flight = a.words[kRaInFlight] + claims - n_req;
-    const uint32_t dropped = a.words[kRaDropped];
-    a.words[kRaInFlight] = in_flight;
-    a.words[kRaDropped] = 0;
-    a.words[kRaEpoch] += 1;
-    const uint32_t c[4] = {n_req, n_frag, dropped, in_flight};
-    for (int k = 0; k < 4; k++) {
-      if (a.counts_out) a.counts_out[k] = c[k];
-      a.counts_host[k] = c[k];  // straight into pinned host memory: nothing to copy back
-    }
-  }
+  if (threadIdx.x == 0) (void)ra_scan_finish<false>(a, run);
 }
 
 // The wavefront of a completing arrival hands the request over: its record goes
 // into the output tables in sequence order, the record is emptied and returned
 // to the free ring, the cell is emptied.  The request's rank and first fragment
 // index hang on that arrival (arr_pack there plus its workgroup's scanned total).
-__global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
+template <bool FUSED>
+__device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32_t *take, bool overflow)
 {
-  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
   const uint32_t n = ra_n(a);
-  const uint32_t i = blockIdx.x * kRaTakeBlock + threadIdx.x;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  const bool overflow = a.words[kRaOverflow] != 0;
   uint32_t cell = kRaNoCell;
   unsigned long long v = 0;
   bool completes = false;
@@ -2005,7 +2039,7 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
     cell = a.arr_cell[i];
     const unsigned long long p = a.arr_pack[i];
     completes = cell != kRaNoCell && (p >> 63) && !overflow;
-    if (completes) v = (p & ~(1ull << 63)) + a.blk[i / kRaBlock];
+    if (completes) v = (p & ~(1ull << 63)) + (FUSED ? 0ull : a.blk[i / kRaBlock]);  // one workgroup: nothing before it
     // the position of a request's last arrival counts per call
     if (cell != kRaNoCell && !completes) a.last[cell] = 0;
   }
@@ -2018,7 +2052,7 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
   const uint32_t my_rank = (uint32_t)__popcll(todo & ((1ull << lane) - 1ull));
   bool own = false;
   if (completes) {
-    const uint32_t cnt = ra_cnt(a.acc[cell]);
+    const uint32_t cnt = ra_cnt(ra_acc<FUSED>(a, cell));
     own = cnt <= kOwn;
     if (own) {
       const uint32_t r = (uint32_t)(v >> 32), first = (uint32_t)v, rc = a.rec[cell];
@@ -2035,7 +2069,7 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
         }
       }
       a.req_first[r] = first;
-      if (a.req_token) a.req_token[r] = a.keys[cell];
+      if (a.req_token) a.req_token[r] = ra_key(a.keys + cell);
       if (a.req_hdr_slot) a.req_hdr_slot[r] = (uint32_t)e[0];
       a.free_ring[(tail0 + my_rank) & a.rmask] = rc;
       a.acc[cell] = 0;
@@ -2054,7 +2088,7 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
     const uint32_t c = (uint32_t)__shfl((int)cell, l, kWave);
     const uint32_t r = (uint32_t)__shfl((int)(uint32_t)(v >> 32), l, kWave);
     const uint32_t first = (uint32_t)__shfl((int)(uint32_t)v, l, kWave);
-    const uint32_t rc = a.rec[c], cnt = ra_cnt(a.acc[c]);
+    const uint32_t rc = a.rec[c], cnt = ra_cnt(ra_acc<FUSED>(a, c));
     unsigned long long *t = a.tab + (size_t)rc * SG_MAX_BI_SIZE;
     for (uint32_t j = lane; j < cnt; j += kWave) {
       const unsigned long long e = t[j];
@@ -2063,7 +2097,7 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
       t[j] = 0;  // a fresh request finds an empty record
       if (j == 0) {
         a.req_first[r] = first;
-        if (a.req_token) a.req_token[r] = a.keys[c];
+        if (a.req_token) a.req_token[r] = ra_key(a.keys + c);
         if (a.req_hdr_slot) a.req_hdr_slot[r] = (uint32_t)e;  // the slot whose header the responses answer
       }
     }
@@ -2077,6 +2111,28 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
       __hip_atomic_store(&a.keys[c], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
+}
+
+__global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
+{
+  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
+  ra_emit_step<false>(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take, a.words[kRaOverflow] != 0);
+}
+
+// A burst of at most kRaTakeBlock arrivals: the four steps by one workgroup in one launch.
+static_assert(kRaTakeBlock == kRaBlock, "one workgroup size for all steps of a burst");
+__global__ __launch_bounds__(kRaTakeBlock) void k_ra_burst(RaArgs a)
+{
+  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
+  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  __shared__ uint32_t overflow;
+  const uint32_t i = threadIdx.x;
+  ra_insert_step(a, i, take);
+  __syncthreads();
+  const uint64_t tot = ra_flag_step<true>(a, i, wave_tot);
+  if (threadIdx.x == 0) overflow = ra_scan_finish<true>(a, tot);
+  __syncthreads();
+  ra_emit_step<true>(a, i, take, overflow != 0);
 }
 
 // Empties the table: every cell, every record, all records back in the ring.
@@ -3001,6 +3057,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
   if (a->n_frames > sc.max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u", a->n_frames, sc.max_frames);
   if (!a->resp_first || (a->n_frames && (!a->tx_slot || (!a->hdr_src_slot && !a->hdr_src_req && !a->hdr_templates))))
     return fail(c, SG_E_INVAL, "null frame tables");
+  if ((uintptr_t)a->hdr_templates & 1u) return fail(c, SG_E_INVAL, "hdr_templates must start at an even address");
   const uint32_t hl = hdr_len_of(a->tx.hdr_profile);
   if (a->mtu == 0 || (uint64_t)a->mtu + hl > a->tx.slot_size)
     return fail(c, SG_E_INVAL, "mtu %u + %u header bytes does not fit a %u-byte slot", a->mtu, hl, a->tx.slot_size);
@@ -3397,12 +3454,15 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *coun
   const uint32_t g_take = (a->n_arrivals + kRaTakeBlock - 1) / kRaTakeBlock;
   rc = prof_begin(c, 5);
   if (rc != SG_OK) return rc;
-  if (a->n_arrivals) {
+  if (a->n_arrivals <= (uint32_t)kRaTakeBlock) {
+    // a NIC burst (an empty one still leaves its counts): one workgroup, one launch
+    k_ra_burst<<<1, kRaTakeBlock, 0, c->stream>>>(r);
+  } else {
     k_ra_insert<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
     k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
+    k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);
+    k_ra_emit<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
   }
-  k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);  // an empty burst still leaves its counts
-  if (a->n_arrivals) k_ra_emit<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
   rc = prof_end(c);
   if (rc != SG_OK) return rc;
   rc = finish(c, a->flags);
