@@ -81,6 +81,26 @@ def test_resnet_sized_requests_arrive_in_bursts_of_64(order_kind):
     ctx.close()
 
 
+@pytest.mark.parametrize("burst", [1000, 1024, 1025, 2500])
+def test_bursts_around_the_size_one_workgroup_takes(burst):
+    """A burst of up to 1024 arrivals is sorted by one workgroup in one launch,
+    a larger one by four kernels: the same stream in bursts on either side of
+    that size (requests carried across calls both ways) gives what the oracle
+    makes of the whole stream."""
+    w = synth.make_workload(4, 700)
+    order = np.random.default_rng(burst).permutation(w.arrivals)
+    ctx = SgContext(0, max_reqs=1024, max_frames=8192)
+    ctx.reassemble_reset()
+    tabs = Tables(1024, 8192)
+    fs, fl, first, tok, hdr, peak = _feed_in_bursts(ctx, w, order, burst, tabs)
+    efs, efl, erf, etok = oracle.reassemble(w, arrivals=order)
+    assert np.array_equal(tok, etok) and np.array_equal(first, erf)
+    assert np.array_equal(fs, efs) and np.array_equal(fl, efl)
+    assert np.array_equal(hdr, efs[erf[:-1]])
+    assert peak > 10
+    ctx.close()
+
+
 def test_bursts_with_the_reference_header_and_nic_lengths():
     """REF64: a request is complete when its bytes add up to the server-wide
     size; the running total is carried from call to call."""
