@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes the copy kernels of one call move, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this file (--calib-copy --steps 40 --warmup 5), each counter scaled by what it reads for a plain
 # 512 MiB device copy in the same run (FETCH_SIZE x 2.000 KiB, WRITE_SIZE x 1.000 KiB).  Keyed by
-# (workload, batches per launch, kernel family); the default call: 340.5 MB read + 313.5 MB written.
+# (workload, batches per launch, kernel family); the default call: 340.5 MB read + 313.1 MB written.
 # bert's scatter is both of its kernels (full frames + short remainder frames), jumbo's the copy
 # phase without the 1.9 MB of the checksum-finishing kernel.
 MEASURED_TRAFFIC = {
