@@ -67,7 +67,6 @@ class P2pRpcAppRrMemPool {
   hipMemGenericAllocationHandle_t req_h{}, resp_h{};
   bool mirrored_ = false;
   volatile uint32_t *states = nullptr;
-  int n_states;
 
   static size_t lcm(size_t a, size_t b) { return a / std::gcd(a, b) * b; }
 
@@ -99,7 +98,7 @@ class P2pRpcAppRrMemPool {
 
  public:
   P2pRpcAppRrMemPool(int pool_size, int _device_id, size_t req_size, size_t resp_size, bool want_mirror = true)
-      : device_id(_device_id), n_states(pool_size)
+      : device_id(_device_id)
   {
     SG_HIP_OK(hipSetDevice(device_id));
     size_t gran = 1 << 21;
