@@ -44,8 +44,12 @@ def _feed_in_bursts(ctx, w, order, burst, tabs, len_nic=None, req_size=0):
     ln = to_dev(len_nic, DEV) if len_nic is not None else None
     fs, fl, first, tok, hdr = [], [], [0], [], []
     peak = 0
-    for b in range(0, len(order), burst):
-        n = min(burst, len(order) - b)
+    b = -1
+    nxt = 0
+    while nxt < len(order):
+        # `burst`: one size for all calls, or a function that says how many arrivals the next call brings
+        b, n = nxt, min(burst() if callable(burst) else burst, len(order) - nxt)
+        nxt += n
         n_req, n_frag, in_flight = ctx.reassemble(rx, arr[b:b + n], n, tabs.fs, tabs.fl, tabs.rf, tabs.tok,
                                                   ln, req_size, req_hdr_slot=tabs.hdr, counts_out=tabs.counts)
         assert tabs.counts.cpu().tolist() == [n_req, n_frag, ctx.last_dropped, in_flight]
@@ -98,6 +102,42 @@ def test_bursts_around_the_size_one_workgroup_takes(burst):
     assert np.array_equal(fs, efs) and np.array_equal(fl, efl)
     assert np.array_equal(hdr, efs[erf[:-1]])
     assert peak > 10
+    ctx.close()
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_streams_in_bursts_of_random_sizes(seed):
+    """Seeded random streams -- request sizes, MTU, header profile, arrival order -- cut into calls of
+    random sizes on both sides of what one workgroup takes, so that the one-launch and the four-kernel
+    form alternate over the same table with requests carried from one to the other."""
+    rng = np.random.default_rng(7000 + seed)
+    profile = int(rng.integers(0, 2))
+    mtu = int(rng.choice([64, 256, 1400]))
+    n_req = int(rng.integers(1, 400))
+    if profile == synth.HDR_REF64:
+        sizes = [int(rng.integers(1, 12 * mtu))] * n_req   # ready when the bytes add up to the one size
+    else:
+        sizes = [int(x) for x in rng.integers(1, 12 * mtu, n_req)]
+    w = synth.make_custom(sizes, [1] * n_req, mtu=mtu, slot_size=2 * ((synth.hdr_len(profile) + mtu + 1) // 2),
+                          order=str(rng.choice(["in_order", "perm_within_request", "interleave_keep_order", "shuffle_all"])),
+                          seed=seed, profile=profile)
+    order = w.arrivals if rng.integers(0, 2) else rng.permutation(w.arrivals)
+    menu = [1, 7, 64, 500, 1024, 1025, 3000]
+    print(f"case random bursts seed={seed} profile={profile} mtu={mtu} n_req={n_req} arrivals={len(order)}", flush=True)
+    ctx = SgContext(0, max_reqs=512, max_frames=8192)
+    ctx.reassemble_reset()
+    tabs = Tables(512, 8192)
+    ln = None
+    if profile == synth.HDR_REF64:
+        ln = np.zeros(w.n_slots, np.uint32)
+        ln[w.frag_slot] = w.frag_len
+    fs, fl, first, tok, hdr, _ = _feed_in_bursts(ctx, w, order, lambda: int(rng.choice(menu)), tabs, len_nic=ln,
+                                                 req_size=sizes[0] if profile == synth.HDR_REF64 else 0)
+    efs, efl, erf, etok = oracle.reassemble(w, arrivals=order, frag_len_nic=ln,
+                                            req_size=sizes[0] if profile == synth.HDR_REF64 else 0)
+    assert np.array_equal(tok, etok) and np.array_equal(first, erf)
+    assert np.array_equal(fs, efs) and np.array_equal(fl, efl)
+    assert np.array_equal(hdr, efs[erf[:-1]])
     ctx.close()
 
 
