@@ -18,25 +18,29 @@ DEV = "cuda"
 ORDERS = ["in_order", "perm_within_request", "interleave_keep_order", "shuffle_all"]
 
 
-def random_case(seed: int):
-    rng = np.random.default_rng(1000 + seed)
+def random_case(seed: int, many: bool = False):
+    """``many``: hundreds to thousands of requests of a few frames each -- launches large enough for
+    the XCD-aware order, the tiled scan of request totals and the several-requests-per-wavefront
+    descriptor kernels -- instead of a dozen requests of any size."""
+    rng = np.random.default_rng((50000 if many else 1000) + seed)
     profile = int(rng.integers(0, 2))
     hl = synth.hdr_len(profile)
-    mtu = int(rng.choice([64, 256, 1400, 1408, 2000, 4242, 8800]))
-    slot_size = 2 * ((hl + mtu + int(rng.integers(0, 300)) + 1) // 2)
-    n_req = int(rng.integers(1, 14))
+    mtu = int(rng.choice([64, 256, 1400, 2000] if many else [64, 256, 1400, 1408, 2000, 4242, 8800]))
+    slot_size = 2 * ((hl + mtu + int(rng.integers(0, 100 if many else 300)) + 1) // 2)
+    n_req = int(rng.integers(500, 6000)) if many else int(rng.integers(1, 14))
     uniform = bool(rng.integers(0, 2))
     in_place = bool(rng.integers(0, 4) == 0)
     if uniform:
-        size = int(rng.integers(1, 6 * mtu + 2))
+        size = int(rng.integers(1, (4 if many else 6) * mtu + 2))
         sizes = [size] * n_req
-        rs = size if in_place else int(rng.integers(1, 5 * mtu + 2))
+        rs = size if in_place else int(rng.integers(1, (3 if many else 5) * mtu + 2))
         resp = [rs] * n_req
     else:
-        sizes = [int(x) for x in rng.integers(0, 5 * mtu + 2, n_req)]
+        top = [mtu // 4 + 2, 2 * mtu + 2, 6 * mtu + 2][int(rng.integers(0, 3))] if many else 5 * mtu + 2
+        sizes = [int(x) for x in rng.integers(0, top, n_req)]
         if rng.integers(0, 3) == 0:
             sizes[int(rng.integers(0, n_req))] = 0
-        resp = list(sizes) if in_place else [int(x) for x in rng.integers(0, 4 * mtu + 2, n_req)]
+        resp = list(sizes) if in_place else [int(x) for x in rng.integers(0, top if many else 4 * mtu + 2, n_req)]
         # a request without fragments has no header a response could be built from
         resp = [0 if s == 0 else r for s, r in zip(sizes, resp)]
     in_t, out_t = (), ()
@@ -60,11 +64,12 @@ def random_case(seed: int):
     return w, uniform, shift, rng
 
 
-@pytest.mark.parametrize("seed", range(300))
-def test_random_workload(ctx, seed):
-    w, uniform, shift, rng = random_case(seed)
+@pytest.mark.parametrize("seed,many", [(s, False) for s in range(300)] + [(s, True) for s in range(16)],
+                         ids=[str(s) for s in range(300)] + [f"many-{s}" for s in range(16)])
+def test_random_workload(ctx, seed, many):
+    w, uniform, shift, rng = random_case(seed, many)
     ref64 = w.profile == synth.HDR_REF64
-    print(f"case random seed={seed} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} mtu={w.mtu} "
+    print(f"case random seed={seed} many={many} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} mtu={w.mtu} "
           f"slot={w.slot_size} profile={w.profile} flags={w.flags} in_place={w.tx_in_place} "
           f"tensors={w.in_tensor_sizes}/{w.out_tensor_sizes} shift={shift}", flush=True)
     dw = DeviceWorkload(w, ring_shift=shift)
