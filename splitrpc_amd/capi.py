@@ -33,6 +33,7 @@ F_NO_XCD_REMAP = 1 << 17
 F_NO_SMALL = 1 << 18
 F_FORCE_SMALL = 1 << 19
 
+ABI_VERSION = 2  # SG_HIP_ABI_VERSION of include/sg_hip.h these mirrors were written against
 MAX_BI_SIZE = 1024
 MAX_TENSORS = 4
 
@@ -128,6 +129,9 @@ def load() -> C.CDLL:
     lib.sg_hip_last_error.argtypes = [P]
     lib.sg_hip_last_error.restype = C.c_char_p
     lib.sg_hip_abi_version.restype = C.c_int
+    if lib.sg_hip_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} speaks ABI version {lib.sg_hip_abi_version()}, this module {ABI_VERSION}: "
+                           "rebuild with `python -m splitrpc_amd.build`")
     lib.sg_hip_stream.argtypes = [P]
     lib.sg_hip_stream.restype = P
     lib.sg_hip_sync.argtypes = [P]
