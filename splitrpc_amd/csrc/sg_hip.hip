@@ -325,7 +325,6 @@ int finish(sg_hip_ctx *c, uint32_t flags)
 
 }  // namespace
 
-// floor(n / d) == (n * M) >> (27 + l) for every n < 2^27, with l = ceil(log2 d), M = ceil(2^(27 + l) / d)
 // Walks the tensor-major buffers once per fragment index (all requests of the call have `size`
 // bytes cut at `mtu`): where fragment i lands, for every i.  Returns the number of entries, or 0
 // when there is no plan (more fragments per request than entries, a tensor of 4 GiB or more per
@@ -364,6 +363,7 @@ static uint32_t fill_plan(const AppDev &app, uint64_t size, uint32_t mtu, uint64
   return (uint32_t)per;
 }
 
+// floor(n / d) == (n * M) >> (27 + l) for every n < 2^27, with l = ceil(log2 d), M = ceil(2^(27 + l) / d)
 static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
 {
   uint32_t l = 0;
