@@ -82,6 +82,13 @@ extern "C" {
 #define SG_F_NO_SMALL (1u << 18)       /* one wavefront per frame even for short frames (for experiments) */
 #define SG_F_FORCE_SMALL (1u << 19)    /* short remainder frames always go several to a wavefront, also where
                                           the call is too small for the extra launch to pay (for tests) */
+#define SG_F_SELF_ADVANCE (1u << 20)   /* a call whose copy kernel derives its offsets from the bump-ring
+                                          cursor has that kernel advance the cursor too, whatever the
+                                          call's size, instead of a one-workgroup kernel behind it: one
+                                          graph node fewer per call.  The library picks this by itself for
+                                          calls of few wavefronts; a call that publishes slot states
+                                          always has the kernel behind it. */
+#define SG_F_TAIL_KERNEL (1u << 21)    /* the opposite: always the kernel behind the call (for experiments) */
 
 /* States of an application slot (APP_RR_STATUS, src/p2p_rpc_app_ctx.h:22). */
 #define SG_SLOT_FREE 0u

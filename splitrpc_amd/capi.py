@@ -32,6 +32,8 @@ F_ASYNC = 1 << 16
 F_NO_XCD_REMAP = 1 << 17
 F_NO_SMALL = 1 << 18
 F_FORCE_SMALL = 1 << 19
+F_SELF_ADVANCE = 1 << 20
+F_TAIL_KERNEL = 1 << 21
 
 ABI_VERSION = 2  # SG_HIP_ABI_VERSION of include/sg_hip.h these mirrors were written against
 MAX_BI_SIZE = 1024

@@ -80,6 +80,113 @@ __device__ __forceinline__ T sload_here(const T *p)
   return *(cptr)(uintptr_t)p;
 }
 
+// ---------------------------------------------------------------------------
+// The bump-ring cursor of an arena
+// ---------------------------------------------------------------------------
+// A kernel that derives its offsets from the cursor cannot overwrite the word
+// its other wavefronts are still reading.  Two ways round that:
+//  * a one-workgroup kernel behind the copy kernel advances the cursor
+//    (k_finish) -- 2 to 4 us of stream time per call, which is nothing to a call
+//    of hundreds of thousands of wavefronts and a quarter of a call of one batch;
+//  * the copy kernel advances the cursor itself ("self-advancing"): a context
+//    keeps, beside the plain cursor word, TWO cells in one 64-byte line, the
+//    live one being the one written last (its two-bit version is one ahead of
+//    the other's).  Every wavefront takes the live cell, and exactly one thread
+//    of the launch writes the successor into the OTHER cell, stamped with what
+//    tells this launch from every other: the address of the queue it was
+//    dispatched on and its dispatch id there.  A wavefront of the same launch
+//    that already finds that stamp on the newer cell knows the cell for its own
+//    launch's work and takes the other one; the next kernel finds a foreign
+//    stamp and takes the new cell.  Nothing waits, nothing counts wavefronts.
+//    The queue word becomes visible before the stamp (a fence between the two
+//    stores; readers take a cell in one scalar load), so a cell that shows the
+//    new version also shows the whole new stamp.  Finding the live cell costs a
+//    wavefront some twenty scalar instructions, which the scalar-bound kernels
+//    of large calls feel (5 % on 400 000 response frames): the host picks this
+//    form for calls of few wavefronts and the trailing kernel for the others.
+// The plain word and the live cell hold the same value whenever no kernel that
+// writes them is running: whoever advances the cursor writes both (the plain
+// word is read by no wavefront of a self-advancing kernel, the cells by none of
+// any other kernel).  Layout, in 64-bit words: cell 0 {value, queue, stamp,
+// PLAIN WORD}, cell 1 {value, queue, stamp, unused}.  Callers of the
+// allocation-free entry point bring a bare 64-bit word instead (`cells` false).
+constexpr uint32_t kCurValue = 0, kCurQueue = 1, kCurStamp = 2, kCurPlain = 3, kCurCell = 4;
+constexpr uint32_t kCurWords = 2 * kCurCell;
+static_assert(kCurValue == 0 && kCurQueue == 1 && kCurStamp == 2 && kCurCell == 4, "cursor_take unpacks a cell by hand");
+
+__device__ __forceinline__ uint32_t cursor_newer(uint64_t stamp0, uint64_t stamp1)
+{
+  return ((((uint32_t)stamp1 & 3u) - ((uint32_t)stamp0 & 3u)) & 3u) == 1u ? 1u : 0u;
+}
+
+// For kernels beside which nothing else reads or writes the cursor (k_finish, the copy kernel
+// behind a descriptor pass): `p` is a context's cursor (cells) or a bare word.
+__device__ __forceinline__ uint64_t cursor_get(const uint64_t *p, bool cells)
+{
+  return p[cells ? kCurPlain : 0u];
+}
+__device__ __forceinline__ void cursor_put(uint64_t *p, bool cells, uint64_t v)
+{
+  if (cells) {
+    p[cursor_newer(p[kCurStamp], p[kCurCell + kCurStamp]) * kCurCell + kCurValue] = v;
+    p[kCurPlain] = v;
+  } else {
+    p[0] = v;
+  }
+}
+
+// What tells this launch from every other: the queue it was dispatched on and the index of its
+// dispatch packet there, both handed to every wavefront in scalar registers.  (The dispatch id
+// has no builtin of its own: the declaration names the compiler's intrinsic.)
+extern "C" __device__ unsigned long long sg_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
+__device__ __forceinline__ uint64_t launch_queue()
+{
+  return (uint64_t)(uintptr_t)__builtin_amdgcn_queue_ptr();
+}
+__device__ __forceinline__ uint64_t launch_stamp()
+{
+  return (uint64_t)sg_dispatch_id() << 2;  // the low two bits of a stamp are the cell's version
+}
+
+// The live value as a wavefront of a self-advancing kernel sees it (wave-uniform, through the
+// scalar cache).  *live: the cell it came from, *stamp: that cell's stamp.
+__device__ __forceinline__ uint64_t cursor_take(const uint64_t *p, uint32_t *live, uint64_t *stamp)
+{
+  // a cell is one 8-dword scalar load
+  const u32x8 c0 = sload_here(reinterpret_cast<const u32x8 *>(p)), c1 = sload_here(reinterpret_cast<const u32x8 *>(p + kCurCell));
+  const uint64_t v0 = (uint64_t)c0[1] << 32 | c0[0], q0 = (uint64_t)c0[3] << 32 | c0[2], s0 = (uint64_t)c0[5] << 32 | c0[4];
+  const uint64_t v1 = (uint64_t)c1[1] << 32 | c1[0], q1 = (uint64_t)c1[3] << 32 | c1[2], s1 = (uint64_t)c1[5] << 32 | c1[4];
+  // this launch's own write, once visible, is the newer cell: one comparison decides
+  const uint32_t n = cursor_newer(s0, s1);
+  const bool own = (n ? q1 : q0) == launch_queue() && ((n ? s1 : s0) & ~3ull) == launch_stamp();
+  const uint32_t l = own ? n ^ 1u : n;
+  *live = l;
+  *stamp = l ? s1 : s0;
+  return l ? v1 : v0;
+}
+
+// The successor, by ONE thread of the launch.  (Vector stores: nothing is ever
+// written through the scalar cache.)
+__device__ __forceinline__ void cursor_advance(uint64_t *p, uint32_t live, uint64_t live_stamp, uint64_t value)
+{
+  uint64_t *cell = p + (live ^ 1u) * kCurCell;
+  p[kCurPlain] = value;  // no wavefront of a self-advancing kernel reads the plain word
+  cell[kCurValue] = value;
+  cell[kCurQueue] = launch_queue();
+  __threadfence();
+  __hip_atomic_store(cell + kCurStamp, launch_stamp() | ((live_stamp + 1u) & 3ull), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// (c + n * size) % cap for c < cap.
+__device__ __forceinline__ uint64_t cursor_bump(uint64_t c, uint64_t n, uint64_t size, uint64_t cap)
+{
+  uint64_t t = n * size;
+  if (t >= cap) t %= cap;  // a gather batch fits its arena; responses may lap theirs
+  const uint64_t e = c + t;
+  return e >= cap ? e - cap : e;
+}
+
 // Sum of the eight 16-bit little-endian words of a 16-byte chunk.
 __device__ __forceinline__ uint32_t words_sum(u32x4 v)
 {

@@ -50,6 +50,9 @@ constexpr size_t kStaticDesc = sizeof(u32x4) * (size_t)SG_STATIC_MAX_FRAMES;
 constexpr size_t kStaticReq = sizeof(uint64_t) * (size_t)SG_STATIC_MAX_REQS;
 constexpr size_t kStaticTile = sizeof(uint64_t) * (SG_STATIC_MAX_REQS / kPartMin + 2);
 constexpr size_t kStaticWords = 256;  // cursors, staged cursors, status, refusal flag
+// 64-bit words a context keeps beside its scratch: two cursors of kCurWords each, their staged
+// successors, the two slot indices (one word), the descriptor tag (two words)
+constexpr size_t kCtxWords = 2 * kCurWords + 8;
 constexpr size_t kStaticBytes = kStaticDesc + 2 * kStaticReq + kStaticTile + kStaticWords;
 }  // namespace
 static __device__ __align__(256) uint8_t scratch[kStaticBytes];
@@ -76,6 +79,9 @@ struct Scratch {
   // descriptor pass stages for the copy kernel to commit
   uint64_t *cursor[2] = {nullptr, nullptr};
   uint64_t *next_cursor[2] = {nullptr, nullptr};
+  // the cursors are pairs of cells (a context: the single-kernel calls advance them themselves) or
+  // plain words (the allocation-free entry point, whose caller may bring the word)
+  bool cursor_cells = false;
   uint32_t *slot_idx[2] = {nullptr, nullptr};  // next slot of the application ring to fill / to serve
   uint32_t *desc_tag = nullptr;    // {generation, requests, items} of the descriptors in `desc`
   uint32_t *desc_gen = nullptr;    // host counter behind the generation (one per scratch)
@@ -95,7 +101,8 @@ struct sg_hip_ctx {
   uint64_t *req_size = nullptr;
   uint64_t *req_off = nullptr;
   uint64_t *tile_tot = nullptr;  // one total per 4096 requests, for the tiled request scan
-  // [0] request-arena cursor, [1] response-arena cursor, [2], [3] their staged successors
+  // kCurWords words each: request-arena cursor, response-arena cursor; then their staged
+  // successors, the two slot indices, the descriptor tag
   uint64_t *cursors = nullptr;
   uint32_t *csum_scratch = nullptr;  // csum_part and csum_valid
   uint32_t desc_gen = 0;
@@ -244,6 +251,23 @@ int prof_drain(sg_hip_ctx *c)
   return SG_OK;
 }
 
+// The word a kernel reads the cursor from when nothing advances it beside that kernel.
+const uint64_t *plain_cursor(const Scratch &sc, int which)
+{
+  return sc.cursor_cells ? sc.cursor[which] + kCurPlain : sc.cursor[which];
+}
+
+// A context's single-kernel call advances its cursor itself when it is small: finding the live
+// cell costs every wavefront some twenty scalar instructions (5 % of a scatter of 400 000 frames),
+// the one-workgroup kernel behind the call 2 to 4 us of stream time whatever the call's size.  A
+// call that publishes slot states has that kernel behind it anyway.
+constexpr uint64_t kSelfAdvanceMaxWaves = 12288;
+bool self_advancing(const Scratch &sc, bool packed, const void *slot_state, uint64_t waves, uint32_t flags)
+{
+  if (flags & SG_F_TAIL_KERNEL) return false;
+  return packed && sc.cursor_cells && !slot_state && (waves <= kSelfAdvanceMaxWaves || (flags & SG_F_SELF_ADVANCE));
+}
+
 // Descriptor build: kernel shape by the average request, then the bump-ring
 // scan of the request totals where offsets are not plain multiples.
 int launch_prep(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const PrepArgs &args)
@@ -294,6 +318,7 @@ void launch_finish(const Scratch &sc, hipStream_t st, uint64_t *cursor, uint64_t
   FinishArgs f;
   memset(&f, 0, sizeof f);
   f.cursor = cursor;
+  f.cursor_cells = sc.cursor_cells ? 1u : 0u;
   f.size = size;
   f.cap = cap;
   f.n_req = n_req;
@@ -390,14 +415,22 @@ static bool small_last_pays(uint64_t per_req, uint32_t n_req, uint32_t flags, bo
   return (flags & SG_F_FORCE_SMALL) || (per_req <= 8 && (!own_launch || n_req >= 1024));
 }
 
-static void launch_scatter_small(hipStream_t st, const ScatterArgs &sa, uint32_t lanes, uint32_t n_frames, bool full_csum)
+// adv: the kernel takes the cursor from the context's cells and advances it (self-advancing call)
+template <bool ADV>
+static void launch_scatter_small_as(hipStream_t st, const ScatterArgs &sa, uint32_t lanes, uint32_t n_frames, bool full_csum)
 {
   const uint32_t per_wave = kWave / lanes;
   const uint32_t grid = (n_frames + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
-  if (lanes == 16 && full_csum) k_scatter_small<16, true><<<grid, kBlock, 0, st>>>(sa);
-  else if (lanes == 16) k_scatter_small<16, false><<<grid, kBlock, 0, st>>>(sa);
-  else if (full_csum) k_scatter_small<32, true><<<grid, kBlock, 0, st>>>(sa);
-  else k_scatter_small<32, false><<<grid, kBlock, 0, st>>>(sa);
+  if (lanes == 16 && full_csum) k_scatter_small<16, true, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else if (lanes == 16) k_scatter_small<16, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else if (full_csum) k_scatter_small<32, true, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else k_scatter_small<32, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+}
+static void launch_scatter_small(hipStream_t st, const ScatterArgs &sa, uint32_t lanes, uint32_t n_frames, bool full_csum,
+                                 bool adv)
+{
+  if (adv) launch_scatter_small_as<true>(st, sa, lanes, n_frames, full_csum);
+  else launch_scatter_small_as<false>(st, sa, lanes, n_frames, full_csum);
 }
 
 // Long frames with the full UDP checksum go to several wavefronts per frame when the
@@ -407,17 +440,40 @@ static bool csum_in_two_phases(const Scratch &sc, uint32_t pieces, bool full_csu
   return full_csum && pieces > 1 && pieces + 1 <= kPartStride && sc.csum_part != nullptr;
 }
 
-template <bool FUSED>
+template <bool FUSED, bool ADV = false>
 static void launch_scatter(hipStream_t st, const ScatterArgs &sa, uint32_t grid, bool full_csum, bool defer = false)
 {
   const bool lng = sa.pieces > 1;
   if (defer) {
-    k_scatter<true, FUSED, true, true><<<grid, kBlock, 0, st>>>(sa);
+    k_scatter<true, FUSED, true, true, ADV><<<grid, kBlock, 0, st>>>(sa);
     k_udp_finish<FUSED><<<(sa.n_items + kBlock - 1) / kBlock, kBlock, 0, st>>>(sa);
-  } else if (full_csum && lng) k_scatter<true, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
-  else if (full_csum) k_scatter<true, FUSED, false><<<grid, kBlock, 0, st>>>(sa);
-  else if (lng) k_scatter<false, FUSED, true><<<grid, kBlock, 0, st>>>(sa);
-  else k_scatter<false, FUSED, false><<<grid, kBlock, 0, st>>>(sa);
+  } else if (full_csum && lng) k_scatter<true, FUSED, true, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else if (full_csum) k_scatter<true, FUSED, false, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else if (lng) k_scatter<false, FUSED, true, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else k_scatter<false, FUSED, false, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+}
+
+// The declared-rule gather in its shapes: all fragments short / a short last fragment per request
+// dealt in turns with the others / long fragments on several wavefronts.
+template <bool ADV>
+static void launch_gather_rule(hipStream_t st, const GatherRuleArgs &ga, uint32_t grid, uint32_t small_all,
+                               uint32_t small_last, uint32_t n_items)
+{
+  if (small_all) {
+    const uint32_t per_wave = kWave / small_all;
+    const uint32_t sgrid = (n_items + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
+    if (small_all == 16) k_gather_small<16, ADV><<<sgrid, kBlock, 0, st>>>(ga);
+    else k_gather_small<32, ADV><<<sgrid, kBlock, 0, st>>>(ga);
+  } else if (small_last == 16) {
+    if (ga.pieces > 1) k_gather_rule<true, 16, ADV><<<grid, kBlock, 0, st>>>(ga);
+    else k_gather_rule<false, 16, ADV><<<grid, kBlock, 0, st>>>(ga);
+  } else if (small_last == 32) {
+    if (ga.pieces > 1) k_gather_rule<true, 32, ADV><<<grid, kBlock, 0, st>>>(ga);
+    else k_gather_rule<false, 32, ADV><<<grid, kBlock, 0, st>>>(ga);
+  } else {
+    if (ga.pieces > 1) k_gather_rule<true, 0, ADV><<<grid, kBlock, 0, st>>>(ga);
+    else k_gather_rule<false, 0, ADV><<<grid, kBlock, 0, st>>>(ga);
+  }
 }
 
 extern "C" {
@@ -453,11 +509,16 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   HIP_TRY(nullptr, hipMalloc(&c->req_size, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->req_off, sizeof(uint64_t) * (size_t)c->max_reqs));
   HIP_TRY(nullptr, hipMalloc(&c->tile_tot, sizeof(uint64_t) * ((size_t)c->max_reqs / kPartMin + 2)));
-  HIP_TRY(nullptr, hipMalloc(&c->cursors, 7 * sizeof(uint64_t)));  // [4]: the two slot indices, [5], [6]: descriptor tag
+  HIP_TRY(nullptr, hipMalloc(&c->cursors, kCtxWords * sizeof(uint64_t)));
   HIP_TRY(nullptr, hipMalloc(&c->status, sizeof(uint32_t)));
   HIP_TRY(nullptr, hipMalloc(&c->csum_scratch, sizeof(uint32_t) * (size_t)c->max_frames * (kPartStride + 1)));
   HIP_TRY(nullptr, hipMemsetAsync(c->csum_scratch, 0, sizeof(uint32_t) * (size_t)c->max_frames * (kPartStride + 1), c->stream));
-  HIP_TRY(nullptr, hipMemsetAsync(c->cursors, 0, 7 * sizeof(uint64_t), c->stream));
+  {
+    // both cursors at 0: cell 0 of the pair is the live one (version 1 against the other cell's 0)
+    uint64_t init[kCtxWords] = {0};
+    init[kCurStamp] = init[kCurWords + kCurStamp] = 1;
+    HIP_TRY(nullptr, hipMemcpy(c->cursors, init, sizeof init, hipMemcpyHostToDevice));
+  }
   HIP_TRY(nullptr, hipMemsetAsync(c->status, 0, sizeof(uint32_t), c->stream));
   c->h_runs_cap = 8192;
   HIP_TRY(nullptr, hipHostMalloc(&c->h_runs, sizeof(Run) * c->h_runs_cap, hipHostMallocDefault));
@@ -474,12 +535,13 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   sc.req_off = c->req_off;
   sc.tile_tot = c->tile_tot;
   sc.cursor[0] = c->cursors + 0;
-  sc.cursor[1] = c->cursors + 1;
-  sc.next_cursor[0] = c->cursors + 2;
-  sc.next_cursor[1] = c->cursors + 3;
-  sc.slot_idx[0] = reinterpret_cast<uint32_t *>(c->cursors + 4);
+  sc.cursor[1] = c->cursors + kCurWords;
+  sc.cursor_cells = true;
+  sc.next_cursor[0] = c->cursors + 2 * kCurWords;
+  sc.next_cursor[1] = c->cursors + 2 * kCurWords + 1;
+  sc.slot_idx[0] = reinterpret_cast<uint32_t *>(c->cursors + 2 * kCurWords + 2);
   sc.slot_idx[1] = sc.slot_idx[0] + 1;
-  sc.desc_tag = reinterpret_cast<uint32_t *>(c->cursors + 5);
+  sc.desc_tag = reinterpret_cast<uint32_t *>(c->cursors + 2 * kCurWords + 3);
   sc.desc_gen = &c->desc_gen;
   sc.csum_part = c->csum_scratch;
   sc.csum_valid = c->csum_scratch + (size_t)c->max_frames * kPartStride;
@@ -562,7 +624,10 @@ int sg_hip_set_cursor(sg_hip_ctx *c, int which, uint64_t value)
   if (!c || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
-  HIP_TRY(c, hipMemcpy(c->cursors + which, &value, sizeof value, hipMemcpyHostToDevice));
+  uint64_t cells[kCurWords] = {0};  // the value in cell 0, one version ahead of cell 1, and in the plain word
+  cells[kCurValue] = cells[kCurPlain] = value;
+  cells[kCurStamp] = 1;
+  HIP_TRY(c, hipMemcpy(c->sc.cursor[which], cells, sizeof cells, hipMemcpyHostToDevice));
   return SG_OK;
 }
 
@@ -571,7 +636,8 @@ int sg_hip_get_cursor(sg_hip_ctx *c, int which, uint64_t *value)
   if (!c || !value || which < 0 || which > 1) return fail(c, SG_E_INVAL, "cursor index %d", which);
   DeviceGuard g(c->device);
   HIP_TRY(c, hipStreamSynchronize(c->stream));
-  HIP_TRY(c, hipMemcpy(value, c->cursors + which, sizeof *value, hipMemcpyDeviceToHost));
+  // between kernels the plain word and the live cell agree
+  HIP_TRY(c, hipMemcpy(value, c->sc.cursor[which] + kCurPlain, sizeof *value, hipMemcpyDeviceToHost));
   return SG_OK;
 }
 
@@ -794,30 +860,19 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
       if (waves >= (1u << 27)) return fail(c, SG_E_INVAL, "%llu wavefronts in one call: the limit is 2^27 - 1", (unsigned long long)waves);
     }
     geometry(waves, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &remap);
+    const bool self_advance = self_advancing(sc, packed, a->slot_state, waves, a->flags);
+    ga.cursor = const_cast<uint64_t *>(plain_cursor(sc, 0));
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
               (app.n_tensors > 1 ? kOptMultiTensor : 0u) | (small_last ? kOptSmallLast : 0u) |
               ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
-    if (small_all) {
-      const uint32_t per_wave = kWave / small_all;
-      const uint32_t sgrid = (n_items + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
-      if (small_all == 16) k_gather_small<16><<<sgrid, kBlock, 0, st>>>(ga);
-      else k_gather_small<32><<<sgrid, kBlock, 0, st>>>(ga);
-    } else if (small_last == 16) {
-      if (ga.pieces > 1) k_gather_rule<true, 16><<<grid, kBlock, 0, st>>>(ga);
-      else k_gather_rule<false, 16><<<grid, kBlock, 0, st>>>(ga);
-    } else if (small_last == 32) {
-      if (ga.pieces > 1) k_gather_rule<true, 32><<<grid, kBlock, 0, st>>>(ga);
-      else k_gather_rule<false, 32><<<grid, kBlock, 0, st>>>(ga);
-    } else {
-      if (ga.pieces > 1) k_gather_rule<true, 0><<<grid, kBlock, 0, st>>>(ga);
-      else k_gather_rule<false, 0><<<grid, kBlock, 0, st>>>(ga);
-    }
+    if (self_advance) launch_gather_rule<true>(st, ga, grid, small_all, small_last, n_items);
+    else launch_gather_rule<false>(st, ga, grid, small_all, small_last, n_items);
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
-    launch_finish(sc, st, packed ? sc.cursor[0] : nullptr, a->fixed_req_size, app.cap, a->n_req, a->counts,
-                  a->slot_state, a->n_slot_states, 0, false);
+    launch_finish(sc, st, packed && !self_advance ? sc.cursor[0] : nullptr, a->fixed_req_size, app.cap, a->n_req,
+                  a->counts, a->slot_state, a->n_slot_states, 0, false);
     return finish(c, a->flags);
   }
 
@@ -841,7 +896,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
   p.req_off = sc.req_off;
   p.fixed_size = a->fixed_req_size;
   p.fixed_offsets = p.packed && a->fixed_req_size != 0;
-  p.cursor = sc.cursor[0];
+  p.cursor = plain_cursor(sc, 0);
   p.next_cursor = sc.next_cursor[0];
   p.offsets_out = packed ? a->offsets_out : nullptr;
   p.counts = a->counts;
@@ -869,6 +924,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     if (packed) {
       ga.cursor = sc.cursor[0];
       ga.next_cursor = sc.next_cursor[0];
+      ga.cursor_cells = sc.cursor_cells ? 1u : 0u;
     }
     ga.counts = a->counts;
     ga.app = app;
@@ -963,7 +1019,6 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     sa.rule.n_req = a->n_req;
     sa.rule.n_slots = a->tx.n_slots;
     sa.rule.single_wrap = app.n_tensors == 0 && (uint64_t)a->n_req * a->fixed_resp_size <= app.cap;
-    sa.rule.cursor = sc.cursor[1];
     sa.rule.offsets_out = packed ? a->offsets_out : nullptr;
     if (app.n_tensors > 0) sa.n_plan = fill_plan(app, a->fixed_resp_size, a->mtu, per, sa.plan);
     sa.pieces = pieces_for(a->mtu);
@@ -978,10 +1033,14 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
       small_all = small_lanes(full_frame);
       if (!small_all && last_frame < a->mtu && small_last_pays(per, a->n_req, a->flags, true)) small_last = small_lanes(last_frame);
     }
+    // the call's last kernel that reads the cursor advances it where the call is self-advancing;
+    // a kernel before that one has no writer beside it and reads the plain word
+    const bool self_advance = self_advancing(sc, packed, a->slot_state, (uint64_t)n_items * sa.pieces, a->flags);
+    sa.rule.cursor = const_cast<uint64_t *>(plain_cursor(sc, 1));
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
     if (small_all) {
-      launch_scatter_small(st, sa, small_all, n_items, full_csum);
+      launch_scatter_small(st, sa, small_all, n_items, full_csum, self_advance);
     } else {
       if (small_last) sa.rule.per_launch = (uint32_t)per - 1;
       magic_div(sa.rule.per_launch, &sa.rule.lmul, &sa.rule.lshift);
@@ -993,13 +1052,19 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
       // (the remainder frames' kernel on a second stream beside this one, forked and joined with
       // events, was measured as well: both kinds of wavefront at once cost the full frames more
       // than the overlap gains, 180 against 172 us on 131072 responses of 1400 + 1400 + 272 bytes)
-      launch_scatter<true>(st, sa, grid, full_csum, defer);
-      if (small_last) launch_scatter_small(st, sa, small_last, a->n_req, full_csum);
+      if (small_last) {
+        launch_scatter<true>(st, sa, grid, full_csum, defer);
+        launch_scatter_small(st, sa, small_last, a->n_req, full_csum, self_advance);
+      } else if (self_advance) {
+        launch_scatter<true, true>(st, sa, grid, full_csum, defer);
+      } else {
+        launch_scatter<true>(st, sa, grid, full_csum, defer);
+      }
     }
     rc = prof_end(c);
     if (rc != SG_OK) return rc;
-    launch_finish(sc, st, packed ? sc.cursor[1] : nullptr, a->fixed_resp_size, app.cap, a->n_req, a->counts,
-                  a->slot_state, a->n_slot_states, 1, false);
+    launch_finish(sc, st, packed && !self_advance ? sc.cursor[1] : nullptr, a->fixed_resp_size, app.cap, a->n_req,
+                  a->counts, a->slot_state, a->n_slot_states, 1, false);
     return finish(c, a->flags);
   }
 
@@ -1023,7 +1088,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
   p.req_size = sc.req_size;
   p.req_off = sc.req_off;
   p.fixed_offsets = p.packed && a->resp_size == nullptr;
-  p.cursor = sc.cursor[1];
+  p.cursor = plain_cursor(sc, 1);
   p.next_cursor = sc.next_cursor[1];
   p.offsets_out = packed ? a->offsets_out : nullptr;
   if (!a->hdr_templates) {
@@ -1069,6 +1134,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     if (packed) {
       sa.cursor = sc.cursor[1];
       sa.next_cursor = sc.next_cursor[1];
+      sa.cursor_cells = sc.cursor_cells ? 1u : 0u;
     }
     if (reuse) {
       // the response cursor ends up where the reused descriptors end

@@ -32,19 +32,19 @@ __device__ __forceinline__ uint32_t item_of_wave(bool remap)
   return __builtin_amdgcn_readfirstlane(g * kWavesPerBlock + threadIdx.x / kWave);
 }
 
-// Advancing the cursor.  A copy kernel that derives its offsets from the
-// bump-ring cursor cannot advance that cursor itself: its own wavefronts may
-// still read it, and a second word to write into would need a device word
-// saying which of the two is live -- with the same problem.  (Letting the
-// wavefronts count themselves in or out with atomics so that the last one may
-// write was built and measured: one returning atomic per workgroup costs the
-// 32-batch gather 4 to 11 % -- the wavefront that waits for its ticket holds its
-// registers that much longer.)  So the advance is the business of a one-workgroup
-// kernel launched right behind the copy kernel, which also publishes slot
-// states where the caller keeps them.  A recorded graph may therefore hold any
-// number of calls.
+// Behind a call: a one-workgroup kernel that publishes application slot states
+// where the caller keeps a slot ring (they may only change once the copy kernel
+// is through), and advances the cursor for the calls whose copy kernel does not
+// do that itself: a call that publishes slot states, and every call of the
+// allocation-free entry point (its cursor is a plain word).  (Letting the
+// wavefronts of the copy kernel count themselves out with atomics so that the
+// last one may do this work was built and measured: one returning atomic per
+// workgroup costs the 32-batch gather 4 to 11 % -- the wavefront that waits for
+// its ticket holds its registers that much longer.)
 struct FinishArgs {
   uint64_t *cursor;       // advanced by n_req * size modulo cap; nullptr: nothing to advance
+  uint32_t cursor_cells;  // the cursor is a context's pair of cells, not a plain word
+  uint32_t pad;
   uint64_t size;
   uint64_t cap;
   uint32_t n_req;         // requests of the call, or their upper bound with `counts`
@@ -74,8 +74,8 @@ __global__ __launch_bounds__(kBlock) void k_finish(FinishArgs a)
   if (a.all_or_nothing && refused) return;
   if (a.cursor && threadIdx.x == 0) {
     // bump ring with equal sizes: off = (off + size) % capacity, n_req times
-    const uint64_t c = *a.cursor;
-    *a.cursor = (c % a.cap + ((uint64_t)n * a.size) % a.cap) % a.cap;
+    const uint64_t c = cursor_get(a.cursor, a.cursor_cells != 0);
+    cursor_put(a.cursor, a.cursor_cells != 0, (c % a.cap + ((uint64_t)n * a.size) % a.cap) % a.cap);
   }
   if (a.state) {
     const uint32_t i0 = *a.slot_idx % a.n_states;
@@ -112,7 +112,10 @@ struct RuleArgs {
   uint32_t per_launch;
   uint32_t div_mul, div_shift;  // item / per_req == (item * div_mul) >> div_shift for item < 2^27
   uint32_t lmul, lshift;        // the same for per_launch
-  const uint64_t *cursor;  // read only here; k_finish advances it behind this kernel
+  // The plain cursor word.  In the self-advancing kernels (ADV) it is a context's, the live value
+  // is in the cells that word belongs to, and the launch writes the successor (it is the call's
+  // last kernel that reads the cursor; no k_finish follows).
+  uint64_t *cursor;
   uint64_t *offsets_out;
 };
 
@@ -130,15 +133,19 @@ struct GatherArgs {
   uint64_t *cursor;             // packed: wavefront 0 commits *next_cursor unless the batch was refused
   const uint64_t *next_cursor;
   const uint32_t *counts;       // device-resident counts ([0] requests, [1] items), or nullptr
+  uint32_t cursor_cells;        // the cursor is a context's pair of cells, not a plain word
+  uint32_t cursor_pad;
   AppDev app;
 };
 
 // Descriptor of item `item` from the rule; publishes the request offset and, on
 // the batch's last item, the advanced cursor.  Returns status bits.
+// `writer`: this thread is the one of the launch that advances a self-advancing cursor (ADV).
+template <bool ADV>
 __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &app, uint32_t item,
                                               uint32_t n_items, uint32_t n_req, uint32_t lane, uint32_t *slot,
                                               uint32_t *len, uint32_t *off, uint32_t *r,
-                                              uint32_t *i, uint64_t *req_off)
+                                              uint32_t *i, uint64_t *req_off, bool writer)
 {
   uint32_t bad = 0;
   *r = (uint32_t)(((uint64_t)item * g.div_mul) >> g.div_shift);  // item / per_req
@@ -147,6 +154,9 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
   *slot = sload_here(g.item_slot + item);
   const uint32_t first_r = sload_here(g.first + *r);
   uint64_t c0 = app.n_tensors == 0 ? sload_here(g.cursor) : 0;
+  uint64_t cur_stamp = 0;
+  uint32_t cur_live = 0;
+  if (ADV && app.n_tensors == 0) c0 = cursor_take(g.cursor - kCurPlain, &cur_live, &cur_stamp);
   *off = *i * g.mtu;
   const uint64_t rem = g.size - *off;
   *len = (uint32_t)(rem <= g.mtu ? rem : g.mtu);
@@ -155,6 +165,8 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
   *req_off = 0;
   if (app.n_tensors == 0) {
     if (c0 >= app.cap) c0 %= app.cap;  // only after a set_cursor beyond the capacity
+    // the successor depends on the cursor, the size and the count only: it is out before a bad item is dropped
+    if (ADV && writer) cursor_advance(g.cursor - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, g.size, app.cap));
     uint64_t o = c0 + (uint64_t)*r * g.size;
     if (g.single_wrap) o = o >= app.cap ? o - app.cap : o;  // n_req * size <= capacity
     else o %= app.cap;
@@ -316,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   // this kernel does not read the cursor: the value the descriptor pass left is committed here
   // (a batch of no requests at all has left none)
   if (w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts)))
-    *a.cursor = sload(a.next_cursor);
+    cursor_put(a.cursor, a.cursor_cells != 0, sload(a.next_cursor));
   if (item >= n_items) return;
   const u32x4 d = sload_here(desc + item);  // asked for together with the status word
   if (sload_here(status)) return;           // the descriptor pass refused the batch: move nothing
@@ -354,12 +366,12 @@ static_assert(sizeof(FragPlan) == 32, "a plan entry is one 8-dword scalar load")
 // carries min(remaining, mtu) bytes and starts i * mtu bytes into the request;
 // request r starts at cursor + r * size in the bump ring) and holds the
 // fragment's real length against the rule.
-struct GatherRuleArgs {
+struct alignas(64) GatherRuleArgs {
   // hot: what a wavefront needs before its first payload load
   const uint8_t *ring;
   const uint32_t *frag_slot;
   uint8_t *dst;               // arena (packed) or the tensor (one tensor-major buffer)
-  const uint64_t *cursor;     // packed only; read only here, k_finish advances it behind this kernel
+  uint64_t *cursor;           // packed only: the plain cursor word (ADV kernels: of a context, whose cells hold the live value)
   uint64_t size;
   uint64_t cap;               // packed: arena capacity; 0: tensor-major
   uint32_t n_items;
@@ -391,7 +403,7 @@ struct GatherRuleArgs {
   // fragments per request, or tensors of 4 GiB and more per request).
   uint32_t n_plan;
   uint32_t plan_pad;
-  FragPlan plan[kPlanMax];
+  alignas(64) FragPlan plan[kPlanMax];  // an entry is one 8-dword scalar load: inside one cache line
 };
 constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
 // slots start at 16-byte aligned addresses: the header's length field can be read as part of
@@ -399,20 +411,21 @@ constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
 constexpr uint32_t kOptHdrChunk = 16u;
 constexpr uint32_t kOptSmallLast = 32u;  // the last fragment of every request is left to k_gather_small
 
-template <int L>
-__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave);
+template <int L, bool ADV>
+__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave, bool may_advance);
 
 // SMALL: lanes per remainder fragment (16 or 32) when the last fragment of every
 // request is short -- the wavefronts behind those of the full fragments then move
 // 64 / SMALL remainder fragments each, in the same launch (a launch of their own
 // would be all latency: tens of megabytes at most); 0: no such wavefronts.
-template <bool LONG, int SMALL>
+// ADV: the kernel takes the cursor from a context's cells and advances it itself (no k_finish follows).
+template <bool LONG, int SMALL, bool ADV>
 __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
 {
   const uint8_t *ring = a.ring;
   const uint32_t *frag_slot = a.frag_slot;
   uint8_t *dst = a.dst;
-  const uint64_t *cursor_in = a.cursor;
+  uint64_t *cursor_in = a.cursor;
   const uint64_t size = a.size, cap = a.cap;
   const uint32_t per_req = a.per_req, mtu = a.mtu, slot_size = a.slot_size;
   const uint32_t hl = a.hl, n_slots = a.n_slots, pieces = a.pieces, opts = a.opts;
@@ -429,6 +442,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   }
 
   uint32_t w = item_of_wave((opts & kOptRemap) != 0);
+  const bool first_wave = w == 0;
   const uint32_t pl = a.per_launch;
   if (SMALL) {
     // Wavefronts of the two kinds are dealt in turns: after the period - 1 wavefronts of the full
@@ -438,7 +452,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     const uint32_t blk = (uint32_t)(((uint64_t)w * a.pmul) >> a.pshift);
     const uint32_t j = w - blk * a.period;
     if (j == a.period - 1) {
-      gather_small_wave<(SMALL ? SMALL : 16)>(a, blk);
+      gather_small_wave<(SMALL ? SMALL : 16), ADV>(a, blk, false);  // wavefront 0 of the full fragments advances the cursor
       return;
     }
     w = blk * (a.period - 1) + j;
@@ -461,6 +475,9 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t slot = sload(frag_slot + item);
   uint64_t c0 = cap ? sload(cursor_in) : 0;
+  uint64_t cur_stamp = 0;
+  uint32_t cur_live = 0;
+  if (ADV && cap) c0 = cursor_take(cursor_in - kCurPlain, &cur_live, &cur_stamp);
   const uint32_t off = i * mtu;
   const uint32_t rem = (uint32_t)size - off;  // sizes are below 4 GiB (checked by the host)
   const uint32_t len = rem <= mtu ? rem : mtu;
@@ -474,6 +491,10 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   if (cap) {
     // bump ring with equal sizes: request r starts at (cursor + r * size) % capacity
     if (c0 >= cap) c0 %= cap;  // only after a set_cursor beyond the capacity
+    // the successor depends on the cursor, the size and the count only: it is out before a
+    // fragment with a bad slot index is dropped
+    if (ADV && first_wave && lane == 0)
+      cursor_advance(cursor_in - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, size, cap));
     ro = c0 + (uint64_t)r * size;
     ro = ro >= cap ? ro - cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
     if (lane == 0 && piece == 0 && a.offsets_out) {
@@ -570,8 +591,8 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
 // bytes -- every fragment of the call (per_launch == per_req) or the last
 // fragment of every request (the remainder; the full fragments then go through
 // k_gather_rule).  Addressing is per lane.
-template <int L>
-__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave)
+template <int L, bool ADV>
+__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave, bool may_advance)
 {
   constexpr uint32_t G = kWave / L;
   // every argument of the common path in one burst of scalar loads
@@ -611,7 +632,12 @@ __device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint3
   uint64_t ro = 0;
   if (a.cap) {
     uint64_t c0 = sload(a.cursor);
+    uint64_t cur_stamp = 0;
+    uint32_t cur_live = 0;
+    if (ADV) c0 = cursor_take(a.cursor - kCurPlain, &cur_live, &cur_stamp);
     if (c0 >= a.cap) c0 %= a.cap;  // only after a set_cursor beyond the capacity
+    if (ADV && may_advance && wave == 0 && lane == 0)
+      cursor_advance(a.cursor - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, a.size, a.cap));
     ro = c0 + (uint64_t)r * a.size;
     ro = ro >= a.cap ? ro - a.cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
     if (live && gl == 0 && a.offsets_out) {
@@ -664,13 +690,13 @@ __device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint3
 }
 
 // Every fragment of the call is short.
-template <int L>
+template <int L, bool ADV>
 __global__ __launch_bounds__(kBlock) void k_gather_small(GatherRuleArgs a)
 {
-  gather_small_wave<L>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
+  gather_small_wave<L, ADV>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave, true);
 }
 
-struct ScatterArgs {
+struct alignas(64) ScatterArgs {
   const u32x4 *desc;
   const uint64_t *req_off;
   const uint32_t *first;         // resp_first CSR (for frag_idx / num_frags)
@@ -693,6 +719,8 @@ struct ScatterArgs {
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
   uint64_t *cursor;             // descriptor path, packed: wavefront 0 commits *next_cursor
   const uint64_t *next_cursor;
+  uint32_t cursor_cells;        // the cursor is a context's pair of cells, not a plain word
+  uint32_t cursor_pad;
   const uint32_t *hdr_src_req;  // one header source per request instead of hdr_src_slot per frame
   const uint32_t *counts;       // device-resident request count, or nullptr
   // full UDP checksum of long frames in two phases: every sub-run's wavefront leaves the sum of
@@ -712,7 +740,7 @@ struct ScatterArgs {
   // GatherRuleArgs::plan); n_plan == 0: the tensors are walked by the wavefront
   uint32_t n_plan;
   uint32_t plan_pad;
-  FragPlan plan[kPlanMax];
+  alignas(64) FragPlan plan[kPlanMax];  // an entry is one 8-dword scalar load: inside one cache line
 };
 
 // Where the payload of a frame comes from; false: not one contiguous piece.
@@ -728,6 +756,7 @@ __device__ __forceinline__ bool scatter_source(const ScatterArgs &a, uint64_t ro
   return plain_target(a.app, ro, r, off, len, from);
 }
 
+static_assert(offsetof(ScatterArgs, plan) % 64 == 0 && offsetof(GatherRuleArgs, plan) % 64 == 0, "plan entries inside cache lines");
 constexpr uint32_t kPartStride = 8;  // words of csum_part per frame: up to 7 sub-runs and the header's share
 
 // LONG: frames longer than kPieceChunks chunks are spread over a.pieces
@@ -743,7 +772,8 @@ constexpr uint32_t kPartStride = 8;  // words of csum_part per frame: up to 7 su
 // DEFER (long frames with the full UDP checksum): the frame's sub-runs go to
 // several wavefronts all the same, each leaving the sum of its bytes behind,
 // and k_udp_finish writes the checksum field afterwards.
-template <bool FULL_CSUM, bool FUSED, bool LONG, bool DEFER = false>
+// ADV (fused only): the kernel takes the cursor from a context's cells and advances it itself.
+template <bool FULL_CSUM, bool FUSED, bool LONG, bool DEFER = false, bool ADV = false>
 __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
 {
   constexpr bool SPLIT = LONG && (!FULL_CSUM || DEFER);      // several wavefronts per frame
@@ -786,7 +816,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   }
   if (!FUSED && w == 0 && lane == 0 && a.cursor && !sload(status) && (!counts || sload(counts))) {
     const uint64_t nc = sload(a.next_cursor);
-    *a.cursor = nc;
+    cursor_put(a.cursor, a.cursor_cells != 0, nc);
     if (a.reuse_gen && a.offsets_out) a.offsets_out[n_req] = nc;
   }
   uint32_t item = SPLIT ? w / pieces : w;
@@ -824,8 +854,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     }
   } else {
     uint32_t slot_i, len, off, i;
-    const uint32_t bad = rule_desc(a.rule, a.app, item, n_items, n_req, piece == 0 ? lane : 1u, &slot_i, &len,
-                                   &off, &r, &i, &ro);
+    const uint32_t bad = rule_desc<ADV>(a.rule, a.app, item, n_items, n_req, piece == 0 ? lane : 1u, &slot_i, &len,
+                                   &off, &r, &i, &ro, w == 0 && lane == 0);
     if (bad) {
       if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, bad);
       return;
@@ -957,7 +987,7 @@ __global__ __launch_bounds__(kBlock) void k_udp_finish(ScatterArgs a)
 // == rule.per_req) or the last frame of every response (the remainder; the full
 // frames then go through k_scatter).  Addressing is per lane, the header is two
 // 16-bit words per lane, sums are row reductions.
-template <int L, bool FULL_CSUM>
+template <int L, bool FULL_CSUM, bool ADV>
 __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_t wave)
 {
   constexpr uint32_t G = kWave / L;
@@ -1007,7 +1037,12 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
   uint64_t ro = 0;
   if (a.app.n_tensors == 0) {
     uint64_t c0 = sload(a.rule.cursor);
+    uint64_t cur_stamp = 0;
+    uint32_t cur_live = 0;
+    if (ADV) c0 = cursor_take(a.rule.cursor - kCurPlain, &cur_live, &cur_stamp);
     if (c0 >= a.app.cap) c0 %= a.app.cap;  // only after a set_cursor beyond the capacity
+    if (ADV && wave == 0 && lane == 0)
+      cursor_advance(a.rule.cursor - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, a.rule.size, a.app.cap));
     uint64_t o = c0 + (uint64_t)r * a.rule.size;
     if (a.rule.single_wrap) o = o >= a.app.cap ? o - a.app.cap : o;
     else o %= a.app.cap;
@@ -1076,10 +1111,10 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
 }
 
 // Every frame of the call is short.
-template <int L, bool FULL_CSUM>
+template <int L, bool FULL_CSUM, bool ADV>
 __global__ __launch_bounds__(kBlock) void k_scatter_small(ScatterArgs a)
 {
-  scatter_small_wave<L, FULL_CSUM>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
+  scatter_small_wave<L, FULL_CSUM, ADV>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
 }
 
 // ---------------------------------------------------------------------------
