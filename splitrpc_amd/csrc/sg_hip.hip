@@ -258,10 +258,13 @@ const uint64_t *plain_cursor(const Scratch &sc, int which)
 }
 
 // A context's single-kernel call advances its cursor itself when it is small: finding the live
-// cell costs every wavefront some twenty scalar instructions (5 % of a scatter of 400 000 frames),
-// the one-workgroup kernel behind the call 2 to 4 us of stream time whatever the call's size.  A
-// call that publishes slot states has that kernel behind it anyway.
-constexpr uint64_t kSelfAdvanceMaxWaves = 12288;
+// cell costs every wavefront some twenty scalar instructions, the one-workgroup kernel behind the
+// call 2 to 4 us of stream time whatever the call's size.  Measured per step (gather and scatter
+// call on a stream each): 16 requests of 602112 bytes 13.0 -> 8.9 us, eight such batches in one
+// call 31.6 -> 30.7 us, 32 batches 105.9 -> 105.3 us; 8192 requests of 3136 bytes 18.1 -> 16.0 us,
+// 65536 of them 89.8 -> 90.4 us; 256 requests of 1.5 MB in 8800-byte fragments 233.5 -> 235.6 us.
+// A call that publishes slot states has the kernel behind it anyway.
+constexpr uint64_t kSelfAdvanceMaxWaves = 65536;
 bool self_advancing(const Scratch &sc, bool packed, const void *slot_state, uint64_t waves, uint32_t flags)
 {
   if (flags & SG_F_TAIL_KERNEL) return false;
