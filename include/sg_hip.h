@@ -339,10 +339,16 @@ int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_te
  * with request offsets taken from the bump ring.  Synchronous unless
  * SG_F_ASYNC is set; an SG_F_ASYNC call does nothing on the stream but launch
  * kernels (no allocation, no copy, no memset).  The bump-ring cursor of an
- * arena is one device word that only kernels advance (a one-workgroup kernel
- * behind the copy kernel, or the copy kernel itself where a descriptor pass has
- * read the cursor before it), so calls recorded into a HIP graph -- any number
- * of them -- continue the ring on every replay.
+ * arena lives on the device and only kernels advance it: the copy kernel where a
+ * descriptor pass has read the cursor before it; where the copy kernel reads the
+ * cursor itself (SG_F_RULE_FRAGS; scatter of one response size), that same
+ * kernel for calls of up to 65536 wavefronts (it tells its own write from the
+ * previous call's by the queue and dispatch id of its launch) and a
+ * one-workgroup kernel behind it for larger calls and for calls that publish
+ * slot states (SG_F_SELF_ADVANCE / SG_F_TAIL_KERNEL pick either).  Calls
+ * recorded into a HIP graph -- any number of them, replayed from any stream --
+ * therefore continue the ring on every replay.  Calls on one context must
+ * not overlap in time (one stream, or streams ordered by events).
  *
  * The cursor after a refusal.  A call the host refuses (SG_E_INVAL) launches
  * nothing and leaves the cursor alone.  With a descriptor pass (no
