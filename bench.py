@@ -81,6 +81,9 @@ def parse():
                     help="skip the single-batch legs (eager, HIP graphs on 1, 2 and 4 streams)")
     ap.add_argument("--general", action="store_true",
                     help="always run the descriptor pass (do not declare the fragmenting rule)")
+    ap.add_argument("--tx-in-order", action="store_true",
+                    help="response frames take their TX slots in ring order (the generator's default "
+                         "is a random permutation of the TX ring, the hardest order for the scatter)")
     return ap.parse_args()
 
 
@@ -383,6 +386,9 @@ def main() -> int:
     bpl = a.batches_per_launch or DEFAULT_BPL[a.workload]
     prof = synth.HDR_REF64 if a.ref64 else synth.HDR_BL58
     w = synth.make_workload(a.workload, profile=prof)
+    if a.tx_in_order and not w.tx_in_place:
+        import numpy as np
+        w.tx_slot = np.sort(w.tx_slot)
     rule = not a.general
 
     def contexts(wl, b):
@@ -533,6 +539,16 @@ def main() -> int:
                               "frac_of_hbm_peak": round((pc.gather_bytes + pc.scatter_bytes) / sc / 1e9 / HBM_PEAK_GBS, 4),
                               "kernels": roofline_of(pc, kc, traffic_known)}
             del pc
+            if cfg == 5 and not a.tx_in_order:
+                # the same responses into TX slots taken in ring order (the default is a random
+                # permutation of the TX ring, which costs the scatter a tenth)
+                import numpy as np
+                wc.tx_slot = np.sort(wc.tx_slot)
+                po = Pool(wc, b, a.rotate_mb, extra, rule=rule)
+                timed(c2, po, 20, 5, c2_tx, reps=1)
+                ko = kernel_times(c2, po, 50)
+                sweep[wc.name]["tx_slots_in_ring_order"] = roofline_of(po, ko, False)["k_scatter"]
+                del po
             c2.close()
             if c2_tx is not None:
                 c2_tx.close()
@@ -569,7 +585,8 @@ def main() -> int:
                    "fused where the workload has one size (fragmenting rule declared and checked)",
                    "streams": "one" if (a.one_stream or w.tx_in_place) else
                    "gather and scatter calls on a stream each (a copy context per direction)",
-                   "timing": f"median of 5 runs of {a.steps} steps", "flags": w.flags},
+                   "timing": f"median of 5 runs of {a.steps} steps", "flags": w.flags,
+                   "tx_slots": "ring order" if a.tx_in_order else "random permutation of the TX ring"},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "requests_per_sec": rps,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1),
