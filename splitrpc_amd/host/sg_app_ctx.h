@@ -39,8 +39,9 @@ class MetaAppCtx {
   // the doorbell is set once what was queued before is done (:45-47)
   inline void AppCompleteNotify(uint32_t value = 2)
   {
-    notify_value = value;
-    (void)hipLaunchHostFunc(work_stream, &MetaAppCtx::ring_door_bell, this);
+    // the value travels with the queued call (a later notification must not change what this one writes)
+    Ring *r = new Ring{door_bell, value};
+    if (hipLaunchHostFunc(work_stream, &MetaAppCtx::ring_door_bell, r) != hipSuccess) delete r;
   }
   inline void NotifyAppRunStart()
   {
@@ -75,11 +76,15 @@ class MetaAppCtx {
   hipGraphExec_t instance = nullptr;
 
  private:
-  uint32_t notify_value = 2;
-  static void ring_door_bell(void *self)
+  struct Ring {
+    uint32_t *bell;
+    uint32_t value;
+  };
+  static void ring_door_bell(void *ring)
   {
-    MetaAppCtx *c = static_cast<MetaAppCtx *>(self);
-    *(volatile uint32_t *)c->door_bell = c->notify_value;
+    Ring *r = static_cast<Ring *>(ring);
+    *(volatile uint32_t *)r->bell = r->value;
+    delete r;
   }
 };
 
@@ -148,6 +153,7 @@ class BufItemPool {
           hipHostMalloc((void **)&h, sizeof(T) * (size_t)num, hipHostMallocMapped) != hipSuccess ||
           hipHostGetDevicePointer((void **)&d, h, 0) != hipSuccess) {
         std::printf("BufItemPool: no pinned memory for %d items on device %d\n", num, type);
+        if (h) (void)hipHostFree(h);
         if (prev >= 0) (void)hipSetDevice(prev);
         return nullptr;
       }
