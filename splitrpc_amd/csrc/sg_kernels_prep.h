@@ -60,9 +60,9 @@ struct PrepArgs {
   u32x4 *desc;             // {slot, len, offset in request, request}
   uint64_t *req_size;
   uint64_t *req_off;
-  // The bump-ring cursor is one device word.  The descriptor pass only reads
-  // it and leaves the advanced value in *next_cursor; the copy kernel of the
-  // same call, which does not read the cursor, commits it.
+  // The plain word of the bump-ring cursor.  The descriptor pass only reads it
+  // and leaves the advanced value in *next_cursor; the copy kernel of the same
+  // call, which does not read the cursor, commits it.
   const uint64_t *cursor;
   uint64_t *next_cursor;
   uint64_t *offsets_out;
