@@ -113,11 +113,19 @@ class Pool:
         context (and stream) per direction (src/p2p_rpc_sg_engine.h:185-196);
         an echo answered in place reads what its gather wrote and stays on one."""
         dw = self.items[i % len(self.items)]
+        if ctx_tx is not None and self.w.tx_in_place:
+            # An echo answered in place reads what its gather wrote and takes the descriptors that
+            # gather built, so both calls of a step stay on one context; consecutive steps (other
+            # rings, other arenas) take the two contexts in turns and overlap on their streams.
+            c = ctx_tx if (i & 1) else ctx
+            dw.gather(c, flags | self.extra_flags, rule=self.rule)
+            dw.scatter(c, flags | self.extra_flags, fuse=self.rule, reuse=True)
+            return
         dw.gather(ctx, flags | self.extra_flags, rule=self.rule)
-        if ctx_tx is not None and not self.w.tx_in_place:
+        if ctx_tx is not None:
             dw.scatter(ctx_tx, flags | self.extra_flags, fuse=self.rule)
         else:
-            # an echo answered in place (the mixed workload) takes the descriptors its gather just built
+            # on one stream; an echo takes the descriptors its gather just built
             dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule, reuse=True)
 
 
@@ -583,7 +591,9 @@ def main() -> int:
                    "requests_per_step": pool.n_req, "header_profile": "REF64" if a.ref64 else "BL58",
                    "descriptor_pass": "general (prefix scan)" if a.general else
                    "fused where the workload has one size (fragmenting rule declared and checked)",
-                   "streams": "one" if (a.one_stream or w.tx_in_place) else
+                   "streams": "one" if a.one_stream else
+                   "both calls of a step on one context (the echo reads what its gather wrote), consecutive "
+                   "steps on two contexts and streams in turns" if w.tx_in_place else
                    "gather and scatter calls on a stream each (a copy context per direction)",
                    "timing": f"median of 5 runs of {a.steps} steps", "flags": w.flags,
                    "tx_slots": "ring order" if a.tx_in_order else "random permutation of the TX ring"},
