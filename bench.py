@@ -332,6 +332,70 @@ def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, 
     return dt
 
 
+def device_pipeline(w, dw, bursts=(256, 1024, 4096)) -> dict:
+    """The receive path end to end on the device, burst after burst and no
+    host wait in between: sg_hip_reassemble files a burst's arrivals (requests
+    that stay incomplete wait on the device), sg_hip_gather_batch gathers the
+    requests the burst completed (their number stays on the device),
+    sg_hip_scatter_batch answers them.  All arrivals of one default call's
+    worth of requests, in arrival order; wall time over the whole stream."""
+    import numpy as np
+    import torch
+    from splitrpc_amd import capi
+    from splitrpc_amd.engine import AppRef, RingRef, SgContext, to_dev
+    if w.in_tensor_sizes or w.out_tensor_sizes or w.tx_in_place or len(set(int(x) for x in w.req_sizes)) != 1:
+        return None
+    dev = "cuda:0"
+    size, rsize = int(w.req_sizes[0]), int(w.resp_sizes[0])
+    per, per_resp = -(-size // w.mtu), -(-rsize // w.mtu)
+    n_arr = int(dw.arrivals.numel())
+    out = {"arrivals": n_arr, "requests": dw.n_req}
+    for burst in bursts:
+        bound = burst // per + 2                      # requests one burst can complete
+        ctx = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=max(65536, bound * per))
+        ctx.reassemble_reset()
+        i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
+        fs, fl, rf, hdr, counts = i32(max(65536, bound * per)), i32(max(65536, bound * per)), i32(4097 + dw.n_req), \
+            i32(4096 + dw.n_req), i32(4)
+        req_cap, resp_cap = 4 * bound * size, 4 * bound * rsize
+        req_arena = torch.zeros(req_cap, dtype=torch.uint8, device=dev)
+        resp_arena = torch.zeros(resp_cap, dtype=torch.uint8, device=dev)
+        tx_ring = torch.zeros(bound * per_resp * w.slot_size, dtype=torch.uint8, device=dev)
+        tx = RingRef(tx_ring, bound * per_resp, w.slot_size, w.profile)
+        tx_slot = to_dev(np.arange(bound * per_resp, dtype=np.uint32), dev)
+        resp_first = to_dev((np.arange(bound + 1) * per_resp).astype(np.uint32), dev)
+        A = capi.F_ASYNC
+        ga = ctx.gather_args(dw.rx, fs, None, rf, bound, bound * per, AppRef(arena=req_arena, cap=req_cap), None,
+                             flags=A | capi.F_RULE_FRAGS, fixed_req_size=size, mtu=w.mtu, counts=counts)
+        sa = ctx.scatter_args(dw.rx, tx, tx_slot, None, resp_first, None, rsize, bound, bound * per_resp, w.mtu,
+                              AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A, hdr_src_req=hdr, counts=counts)
+        ras = [ctx.reassemble_args(dw.rx, dw.arrivals[b:b + burst], min(burst, n_arr - b), fs, fl, rf,
+                                   req_hdr_slot=hdr, counts_out=counts, flags=A) for b in range(0, n_arr, burst)]
+        torch.cuda.synchronize()
+        best = None
+        for rep in range(3):
+            ctx.reassemble_reset()
+            t0 = time.perf_counter()
+            for k, ra in enumerate(ras):
+                ctx.reassemble_raw(ra)
+                ctx.gather_batch_raw(ga)
+                ctx.scatter_batch_raw(sa)
+                if k % 64 == 63:
+                    ctx.sync()
+            ctx.sync()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        left = int(counts.cpu()[3])
+        out[str(burst)] = {"us_per_burst": round(best / len(ras) * 1e6, 2), "arrivals_per_sec": round(n_arr / best, 1),
+                           "requests_per_sec": round(dw.n_req / best, 1),
+                           "payload_Gbit_per_sec": round(8.0 * size * dw.n_req / best / 1e9, 1),
+                           "requests_left_in_flight": left}
+        ctx.close()
+        del fs, fl, rf, hdr, counts, req_arena, resp_arena, tx_ring
+        torch.cuda.empty_cache()
+    return out
+
+
 def roofline_of(pool: Pool, kt, traffic_known: bool = True) -> dict:
     """Both copy kernels of a workload against the HBM peak: algorithmic bytes
     per call over the average duration of the call's copy kernels (HIP events
@@ -481,6 +545,8 @@ def main() -> int:
     reassembly["us_per_burst_of_64_queued"] = round((time.perf_counter() - t0) / max(1, len(queued)) * 1e6, 2)
     ctx.reassemble_reset()
     del ra_fs, ra_fl, ra_rf
+    _log("device pipeline")
+    pipeline = device_pipeline(w, dw0) if not a.ref64 else None
 
     # how the dominant kernel and the whole step scale with the batches laid side by side in one call
     by_bpl = {}
@@ -615,6 +681,7 @@ def main() -> int:
         "single_batch_call": single,
         "per_request_call": per_req,
         "device_reassembly": reassembly,
+        "device_pipeline": pipeline,
         "other_workloads": sweep,
     }
     if not a.no_cpu:
