@@ -587,10 +587,16 @@ __device__ __forceinline__ uint32_t row_sum(uint32_t v)
   return v;
 }
 
-// Sum over the L lanes of a group.
+// Sum over the L lanes of a group (8: half a row, the first three steps of row_sum).
 template <int L>
 __device__ __forceinline__ uint32_t group_sum(uint32_t v)
 {
+  if (L == 8) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xb1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4e, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false);  // row_half_mirror
+    return v;
+  }
   v = row_sum(v);
   if (L == 32) v += __shfl_xor(v, 16, 64);
   return v;
@@ -600,7 +606,8 @@ __device__ __forceinline__ uint32_t group_sum(uint32_t v)
 // L aligned source chunks per step yielding L - 1 destination chunks (the
 // group's last lane has no upper neighbour of its own: the wave shift hands it
 // a foreign lane's chunk, which it does not use).  Lanes 0..15 of the group
-// carry one head byte and one tail byte each.
+// carry one head byte and one tail byte each; the lanes of a group of 8 carry
+// two of each (bytes gl and gl + 8).
 template <int L>
 struct GroupRun {
   const uint8_t *sa;
@@ -608,7 +615,8 @@ struct GroupRun {
   uint8_t *dst;
   uint32_t body, lim, p;
   uint32_t head_b, tail_b, tail_off;
-  bool has_head, has_tail;
+  uint32_t head_b2, tail_b2;  // L == 8 only
+  bool has_head, has_tail, has_head2, has_tail2;
   u32x4 v0, v1;
 };
 
@@ -627,6 +635,10 @@ __device__ __forceinline__ void group_run_begin(GroupRun<L> &r, const uint8_t *s
   r.tail_off = head + (body << 4) + gl;
   r.head_b = r.has_head ? src[gl] : 0u;
   r.tail_b = r.has_tail ? src[r.tail_off] : 0u;
+  r.has_head2 = L < 16 && gl + 8 < head;
+  r.has_tail2 = L < 16 && gl + 8 < tail;
+  r.head_b2 = r.has_head2 ? src[gl + 8] : 0u;
+  r.tail_b2 = r.has_tail2 ? src[r.tail_off + 8] : 0u;
   const uint8_t *s = src + head;
   r.d = dst + head;
   r.p = (uint32_t)(uintptr_t)s & 15u;
@@ -655,8 +667,8 @@ template <int L>
 __device__ __forceinline__ void group_run_cancel(GroupRun<L> &r)
 {
   r.body = 0;
-  r.has_head = false;
-  r.has_tail = false;
+  r.has_head = r.has_head2 = false;
+  r.has_tail = r.has_tail2 = false;
 }
 
 // Returns this lane's share of the little-endian 16-bit word sum with CSUM.
@@ -702,6 +714,16 @@ __device__ __forceinline__ uint32_t group_run_end(GroupRun<L> &r, uint32_t gl)
     r.dst[r.tail_off] = (uint8_t)r.tail_b;
     if (CSUM) acc += ((uintptr_t)(r.dst + r.tail_off) & 1u) ? (r.tail_b << 8) : r.tail_b;
   }
+  if (L < 16) {
+    if (r.has_head2) {
+      r.dst[gl + 8] = (uint8_t)r.head_b2;
+      if (CSUM) acc += ((uintptr_t)(r.dst + gl + 8) & 1u) ? (r.head_b2 << 8) : r.head_b2;
+    }
+    if (r.has_tail2) {
+      r.dst[r.tail_off + 8] = (uint8_t)r.tail_b2;
+      if (CSUM) acc += ((uintptr_t)(r.dst + r.tail_off + 8) & 1u) ? (r.tail_b2 << 8) : r.tail_b2;
+    }
+  }
   return acc;
 }
 
@@ -724,17 +746,24 @@ __device__ __forceinline__ uint32_t hdr_src_word(uint32_t h)
   return h;
 }
 
+// W = words per lane: 2 on the first 16 lanes of a group of 16 or 32, 4 on the 8 lanes of a group of 8
+// (lane j holds words W j .. W j + W - 1).
+template <int W>
 struct SmallHdr {
-  uint32_t w0, w1;  // words 2j and 2j+1 as fetched
+  uint32_t w[W];  // as fetched
 };
 
-__device__ __forceinline__ SmallHdr small_hdr_fetch(const uint8_t *in, uint32_t j, uint32_t hl, bool swap, bool live)
+template <int W>
+__device__ __forceinline__ SmallHdr<W> small_hdr_fetch(const uint8_t *in, uint32_t j, uint32_t hl, bool swap, bool live)
 {
-  SmallHdr h{0u, 0u};
+  SmallHdr<W> h;
   const uint32_t n_words = hl >> 1;
   const uint16_t *w = reinterpret_cast<const uint16_t *>(in);  // rings and templates start at even addresses
-  if (live && 2 * j < n_words) h.w0 = w[swap ? hdr_src_word(2 * j) : 2 * j];
-  if (live && 2 * j + 1 < n_words) h.w1 = w[swap ? hdr_src_word(2 * j + 1) : 2 * j + 1];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const uint32_t x = W * j + k;
+    h.w[k] = (live && x < n_words) ? w[swap ? hdr_src_word(x) : x] : 0u;
+  }
   return h;
 }
 
@@ -763,24 +792,36 @@ __device__ __forceinline__ uint32_t small_hdr_word(uint32_t v, uint32_t h, const
 // lane's index in its group; lanes 16.. of a 32-lane group take part in the
 // sums only.  `live` says whether the group has a frame at all; payload_sum is
 // the group-wide sum of the payload's little-endian words (full UDP checksum).
-template <int L>
-__device__ __forceinline__ void small_hdr_finish(SmallHdr s, uint8_t *out, uint32_t j, const HdrFields &f,
+template <int L, int W>
+__device__ __forceinline__ void small_hdr_finish(SmallHdr<W> s, uint8_t *out, uint32_t j, const HdrFields &f,
                                                  uint32_t payload_sum, bool live)
 {
+  static_assert(W * (L < 16 ? L : 16) == 32, "the header's 32 words over the lanes that hold it");
   const uint32_t n_words = f.hl >> 1;
   const uint32_t Lx = (f.hl - 42u) + f.payload_len;
   const uint32_t tot = (28u + Lx) & 0xffffu, ulen = (8u + Lx) & 0xffffu;
-  const uint32_t h0 = 2 * j, h1 = 2 * j + 1;
-  const bool on0 = live && j < 16 && h0 < n_words, on1 = live && j < 16 && h1 < n_words;
-  uint32_t v0 = on0 ? small_hdr_word(s.w0, h0, f, tot, ulen) : 0u;
-  uint32_t v1 = on1 ? small_hdr_word(s.w1, h1, f, tot, ulen) : 0u;
+  uint32_t h[W], v[W];
+  bool on[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    h[k] = W * j + k;
+    on[k] = live && j < 32 / W && h[k] < n_words;
+    v[k] = on[k] ? small_hdr_word(s.w[k], h[k], f, tot, ulen) : 0u;
+  }
   const uint32_t kAnyCsum = 0x7u;  // IPV4 | PSEUDO | FULL
   if (f.flags & kAnyCsum) {
-    auto in = [](uint32_t h, uint32_t a, uint32_t b) { return h >= a && h < b; };
-    const uint32_t s_ip = group_sum<L>((in(h0, 7, 17) && h0 != 12 ? v0 : 0u) + (in(h1, 7, 17) && h1 != 12 ? v1 : 0u));
-    const uint32_t s_addr = group_sum<L>((in(h0, 13, 17) ? v0 : 0u) + (in(h1, 13, 17) ? v1 : 0u));
-    // word 7 = bytes 14, 15 (version/ihl first); word 11 = bytes 22, 23 (protocol second)
-    const uint32_t pick = group_sum<L>((h1 == 7 ? (v1 & 0xffu) : 0u) + (h1 == 11 ? (v1 & 0xff00u) : 0u));
+    auto in = [](uint32_t x, uint32_t a, uint32_t b) { return x >= a && x < b; };
+    uint32_t t_ip = 0, t_addr = 0, t_pick = 0;
+#pragma unroll
+    for (int k = 0; k < W; k++) {
+      t_ip += in(h[k], 7, 17) && h[k] != 12 ? v[k] : 0u;
+      t_addr += in(h[k], 13, 17) ? v[k] : 0u;
+      // word 7 = bytes 14, 15 (version/ihl first); word 11 = bytes 22, 23 (protocol second)
+      t_pick += (h[k] == 7 ? (v[k] & 0xffu) : 0u) + (h[k] == 11 ? (v[k] & 0xff00u) : 0u);
+    }
+    const uint32_t s_ip = group_sum<L>(t_ip);
+    const uint32_t s_addr = group_sum<L>(t_addr);
+    const uint32_t pick = group_sum<L>(t_pick);
     const uint32_t b14 = pick & 0xffu, proto = pick >> 8;
     uint32_t udp = 0xffffffffu, ipc = 0xffffffffu;
     if (f.flags & (1u << 1)) {  // raw pseudo sum, reference style
@@ -789,20 +830,26 @@ __device__ __forceinline__ void small_hdr_finish(SmallHdr s, uint8_t *out, uint3
       udp = fold16(s_addr + (proto << 8) + bswap16(l));
     }
     if (f.flags & (1u << 2)) {  // finished UDP checksum
-      const uint32_t s_l4 = group_sum<L>(((in(h0, 17, 20) || in(h0, 21, n_words)) ? v0 : 0u) +
-                                         ((in(h1, 17, 20) || in(h1, 21, n_words)) ? v1 : 0u));
+      uint32_t t_l4 = 0;
+#pragma unroll
+      for (int k = 0; k < W; k++) t_l4 += (in(h[k], 17, 20) || in(h[k], 21, n_words)) ? v[k] : 0u;
+      const uint32_t s_l4 = group_sum<L>(t_l4);
       uint32_t t = s_addr + (proto << 8) + bswap16(ulen) + s_l4;
       t = fold16(fold16(t) + fold16(payload_sum));
       udp = (~t) & 0xffffu;
       if (udp == 0) udp = 0xffffu;
     }
     if (f.flags & (1u << 0)) ipc = (~fold16(s_ip)) & 0xffffu;
-    if (h0 == 20 && udp != 0xffffffffu) v0 = udp;
-    if (h0 == 12 && ipc != 0xffffffffu) v0 = ipc;
+#pragma unroll
+    for (int k = 0; k < W; k++) {
+      if (h[k] == 20 && udp != 0xffffffffu) v[k] = udp;
+      if (h[k] == 12 && ipc != 0xffffffffu) v[k] = ipc;
+    }
   }
   uint16_t *w = reinterpret_cast<uint16_t *>(out);
-  if (on0) w[h0] = (uint16_t)v0;
-  if (on1) w[h1] = (uint16_t)v1;
+#pragma unroll
+  for (int k = 0; k < W; k++)
+    if (on[k]) w[h[k]] = (uint16_t)v[k];
 }
 
 // ---- the header as 16-bit words, one per lane -------------------------------

@@ -402,8 +402,11 @@ static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
 
 // Lanes a short frame of at most `bytes` payload bytes is given (two steps of L - 1
 // chunks without looping), or 0 where a whole wavefront per frame is the better deal.
-static uint32_t small_lanes(uint64_t bytes)
+static uint32_t small_lanes(uint64_t bytes, bool scatter = false)
 {
+  // (groups of 8 lanes exist in the scatter only: tiny responses -- a class index, a few logits -- are
+  // common, tiny request fragments are not)
+  if (scatter && bytes <= 2 * 7 * 16) return 8;
   if (bytes <= 2 * 15 * 16) return 16;
   if (bytes <= 2 * 31 * 16) return 32;
   return 0;
@@ -424,7 +427,9 @@ static void launch_scatter_small_as(hipStream_t st, const ScatterArgs &sa, uint3
 {
   const uint32_t per_wave = kWave / lanes;
   const uint32_t grid = (n_frames + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
-  if (lanes == 16 && full_csum) k_scatter_small<16, true, ADV><<<grid, kBlock, 0, st>>>(sa);
+  if (lanes == 8 && full_csum) k_scatter_small<8, true, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else if (lanes == 8) k_scatter_small<8, false, ADV><<<grid, kBlock, 0, st>>>(sa);
+  else if (lanes == 16 && full_csum) k_scatter_small<16, true, ADV><<<grid, kBlock, 0, st>>>(sa);
   else if (lanes == 16) k_scatter_small<16, false, ADV><<<grid, kBlock, 0, st>>>(sa);
   else if (full_csum) k_scatter_small<32, true, ADV><<<grid, kBlock, 0, st>>>(sa);
   else k_scatter_small<32, false, ADV><<<grid, kBlock, 0, st>>>(sa);
@@ -1033,8 +1038,8 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     const uint64_t last_frame = a->fixed_resp_size - (per - 1) * a->mtu;
     uint32_t small_all = 0, small_last = 0;
     if (!(a->flags & SG_F_NO_SMALL)) {
-      small_all = small_lanes(full_frame);
-      if (!small_all && last_frame < a->mtu && small_last_pays(per, a->n_req, a->flags, true)) small_last = small_lanes(last_frame);
+      small_all = small_lanes(full_frame, true);
+      if (!small_all && last_frame < a->mtu && small_last_pays(per, a->n_req, a->flags, true)) small_last = small_lanes(last_frame, true);
     }
     // the call's last kernel that reads the cursor advances it where the call is self-advancing;
     // a kernel before that one has no writer beside it and reads the plain word

@@ -979,7 +979,7 @@ __global__ __launch_bounds__(kBlock) void k_udp_finish(ScatterArgs a)
   *reinterpret_cast<uint16_t *>(a.tx + (size_t)slot * a.tx_slot_size + 40) = (uint16_t)c;
 }
 
-// Scatter of SHORT frames, 64 / L frames per wavefront (L = 16 or 32 lanes per
+// Scatter of SHORT frames, 64 / L frames per wavefront (L = 8, 16 or 32 lanes per
 // frame): the fused form of k_scatter -- responses of one size cut by the
 // fragmenting rule -- for frames of a few hundred bytes, where one wavefront per
 // frame spends most of its time on addressing and header arithmetic that 48 of
@@ -1090,7 +1090,8 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
   }
   // header words and payload chunks are fetched together; a TX slot that is its own header
   // source still holds the request header then (the payload goes past the header only)
-  const SmallHdr sh = small_hdr_fetch(hin, gl, hl, !from_template, live && gl < 16);
+  constexpr int W = L == 8 ? 4 : 2;  // header words per lane
+  const SmallHdr<W> sh = small_hdr_fetch<W>(hin, gl, hl, !from_template, live && gl < 32 / W);
   if (early) {
     group_run_rebase<L>(run, slot + hl);
     if (!plain) group_run_cancel<L>(run);  // a frame the tables have just ruled out
@@ -1107,7 +1108,7 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
     }
   }
   const uint32_t psum = FULL_CSUM ? group_sum<L>(acc) : 0u;
-  small_hdr_finish<L>(sh, slot, gl, hf, psum, live);
+  small_hdr_finish<L, W>(sh, slot, gl, hf, psum, live);
 }
 
 // Every frame of the call is short.
