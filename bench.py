@@ -605,7 +605,7 @@ def main() -> int:
             _log(f"sweep: {wc.name} x {b}")
             c2, c2_tx = contexts(wc, b)
             pc = Pool(wc, b, a.rotate_mb, extra, rule=rule)
-            sc = timed(c2, pc, max(20, a.steps // 4), max(5, a.warmup // 4), c2_tx, reps=3)
+            sc = timed(c2, pc, a.steps, a.warmup, c2_tx)
             kc = kernel_times(c2, pc, 50)
             rps[wc.name] = round(pc.n_req / sc, 1)
             sweep[wc.name] = {"batches_per_launch": b, "ms_per_step": round(sc * 1e3, 5),
