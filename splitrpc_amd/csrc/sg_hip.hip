@@ -402,11 +402,13 @@ static void magic_div(uint64_t d, uint32_t *mul, uint32_t *shift)
 
 // Lanes a short frame of at most `bytes` payload bytes is given (two steps of L - 1
 // chunks without looping), or 0 where a whole wavefront per frame is the better deal.
-static uint32_t small_lanes(uint64_t bytes, bool scatter = false)
+// Groups of 8 lanes pay up to 128 bytes (131072 single-fragment requests and their responses,
+// 4 -> 8 to a wavefront: gather 18.4 -> 13.3 us at 40 bytes, 20.5 -> 18.6 us at 128, 24.6 -> 24.9 us
+// at 200; scatter 26.2 -> 21.7 us at 40, 25.6 -> 23.9 us at 128, 29.2 -> 32.0 us at 224); `eight`:
+// the caller has kernels for such groups.
+static uint32_t small_lanes(uint64_t bytes, bool eight = true)
 {
-  // (groups of 8 lanes exist in the scatter only: tiny responses -- a class index, a few logits -- are
-  // common, tiny request fragments are not)
-  if (scatter && bytes <= 2 * 7 * 16) return 8;
+  if (eight && bytes <= 128) return 8;
   if (bytes <= 2 * 15 * 16) return 16;
   if (bytes <= 2 * 31 * 16) return 32;
   return 0;
@@ -470,7 +472,8 @@ static void launch_gather_rule(hipStream_t st, const GatherRuleArgs &ga, uint32_
   if (small_all) {
     const uint32_t per_wave = kWave / small_all;
     const uint32_t sgrid = (n_items + per_wave * kWavesPerBlock - 1) / (per_wave * kWavesPerBlock);
-    if (small_all == 16) k_gather_small<16, ADV><<<sgrid, kBlock, 0, st>>>(ga);
+    if (small_all == 8) k_gather_small<8, ADV><<<sgrid, kBlock, 0, st>>>(ga);
+    else if (small_all == 16) k_gather_small<16, ADV><<<sgrid, kBlock, 0, st>>>(ga);
     else k_gather_small<32, ADV><<<sgrid, kBlock, 0, st>>>(ga);
   } else if (small_last == 16) {
     if (ga.pieces > 1) k_gather_rule<true, 16, ADV><<<grid, kBlock, 0, st>>>(ga);
@@ -840,7 +843,8 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     uint32_t small_all = 0, small_last = 0;
     if (!(a->flags & SG_F_NO_SMALL)) {
       small_all = small_lanes(full_frag);
-      if (!small_all && last_frag < a->mtu && small_last_pays(per, a->n_req, a->flags, false)) small_last = small_lanes(last_frag);
+      // (a short last fragment rides in k_gather_rule, which has no groups of 8)
+      if (!small_all && last_frag < a->mtu && small_last_pays(per, a->n_req, a->flags, false)) small_last = small_lanes(last_frag, false);
     }
     ga.per_launch = small_last ? (uint32_t)per - 1 : (uint32_t)per;
     magic_div(ga.per_launch, &ga.lmul, &ga.lshift);
@@ -1038,8 +1042,8 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     const uint64_t last_frame = a->fixed_resp_size - (per - 1) * a->mtu;
     uint32_t small_all = 0, small_last = 0;
     if (!(a->flags & SG_F_NO_SMALL)) {
-      small_all = small_lanes(full_frame, true);
-      if (!small_all && last_frame < a->mtu && small_last_pays(per, a->n_req, a->flags, true)) small_last = small_lanes(last_frame, true);
+      small_all = small_lanes(full_frame);
+      if (!small_all && last_frame < a->mtu && small_last_pays(per, a->n_req, a->flags, true)) small_last = small_lanes(last_frame);
     }
     // the call's last kernel that reads the cursor advances it where the call is self-advancing;
     // a kernel before that one has no writer beside it and reads the plain word

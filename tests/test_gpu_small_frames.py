@@ -47,10 +47,10 @@ def _check(ctx, w, extra, cap_slack=0, cursor=0, templates=False):
 
 @pytest.mark.parametrize("path", list(PATHS))
 @pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64], ids=["bl58", "ref64"])
-@pytest.mark.parametrize("last", [1, 15, 16, 17, 100, 223, 224, 225, 239, 240, 479, 480, 481, 700, 991, 992, 993, 1399])
+@pytest.mark.parametrize("last", [1, 15, 16, 17, 100, 127, 128, 129, 239, 240, 479, 480, 481, 700, 991, 992, 993, 1399])
 def test_remainder_fragment_of_every_length(ctx, last, profile, path):
     """Requests and responses of two full frames plus a remainder of `last`
-    bytes: 16 lanes up to 480 bytes (8 in the scatter up to 224), 32 up to 992,
+    bytes: 16 lanes up to 480 bytes (8 in the scatter up to 128), 32 up to 992,
     a wavefront beyond."""
     size = 2 * 1400 + last
     w = synth.make_custom([size] * 11, [size] * 11, seed=last, profile=profile,
@@ -72,19 +72,14 @@ def test_calls_made_of_short_frames_only(ctx, size, mtu, flags, path):
 @pytest.mark.parametrize("profile", [synth.HDR_BL58, synth.HDR_REF64], ids=["bl58", "ref64"])
 @pytest.mark.parametrize("flags", [0, synth.F_IPV4_CSUM | synth.F_UDP_CSUM_FULL])
 def test_single_frame_responses_of_every_small_size(ctx, profile, flags):
-    """Responses of one short frame, eight to a wavefront up to 224 bytes and
-    four beyond: every size class and every phase of the source (responses
-    packed back to back start at all offsets modulo 16), edge bytes on both
-    sides of the aligned chunks included."""
-    for size in list(range(1, 50)) + list(range(50, 260, 7)) + [223, 224, 225, 226]:
-        w = synth.make_custom([64] * 19, [size] * 19, seed=1000 + size, profile=profile, flags=flags)
+    """Requests and responses of one short frame, eight to a wavefront up to
+    128 bytes and four beyond: every size class and every phase (payloads packed
+    back to back start at all offsets modulo 16), edge bytes on both sides of
+    the aligned chunks included."""
+    for size in list(range(1, 50)) + list(range(50, 260, 7)) + [127, 128, 129, 130]:
+        w = synth.make_custom([size] * 19, [size] * 19, seed=1000 + size, profile=profile, flags=flags)
         print(f"case single short frame size={size} profile={profile} flags={flags}", flush=True)
-        dw = DeviceWorkload(w)
-        ctx.set_cursor(1, 0)
-        dw.scatter(ctx)
-        exp_tx, _, _ = expected_scatter(w, None)
-        got = dw.tx_ring.cpu().numpy()
-        assert np.array_equal(got, exp_tx), f"size {size}: " + first_diff(got, exp_tx)
+        _check(ctx, w, 0, cap_slack=77, cursor=5)
 
 
 @pytest.mark.parametrize("path", list(PATHS))
