@@ -240,7 +240,17 @@ __device__ __forceinline__ uint32_t ra_word(const uint32_t *p)
   return FUSED ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
 }
 
-__device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint32_t *take)
+// What a thread knows of its arrival from one step to the next.  The four-kernel form keeps it in
+// device memory (arr_cell / arr_len / arr_fidx / arr_pack); a burst handled by one workgroup keeps
+// it in registers: every thread only ever reads its own entries, and a store followed by a load of
+// the same word is a memory round trip the burst's latency is made of.
+struct RaMine {
+  uint32_t slot = 0, cell = kRaNoCell, len = 0, fidx = 0;
+  unsigned long long pack = 0;
+};
+
+template <bool FUSED>
+__device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint32_t *take, RaMine &mine)
 {
   const uint32_t n = ra_n(a);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -252,6 +262,7 @@ __device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint
   bool pending = false;
   if (in_range) {
     const uint32_t slot = a.arrivals[i];
+    mine.slot = slot;
     if (slot >= a.n_slots) {
       refuse(a.status, a.status_flag, kStBadSlot);
     } else {
@@ -319,10 +330,15 @@ __device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint
   }
   // the cells this wavefront has claimed get their records (a lane claims one cell at most)
   ra_open_cells(a, opened != kRaNoCell, opened, lane, take);
+  mine.cell = cell;
+  mine.len = len;
+  mine.fidx = fidx;
   if (in_range) {
-    a.arr_cell[i] = cell;
-    a.arr_len[i] = len;
-    a.arr_fidx[i] = fidx;
+    if (!FUSED) {
+      a.arr_cell[i] = cell;
+      a.arr_len[i] = len;
+      a.arr_fidx[i] = fidx;
+    }
     if (cell == kRaNoCell && token != 0) refuse(a.status, a.status_flag, kStPoolFull);  // bucket full
   }
   // arrivals that belong to no request: token 0, refused, no room
@@ -333,7 +349,8 @@ __device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint
 __global__ __launch_bounds__(kRaTakeBlock) void k_ra_insert(RaArgs a)
 {
   __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
-  ra_insert_step(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take);
+  RaMine mine;
+  ra_insert_step<false>(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take, mine);
 }
 
 __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell, unsigned long long acc)
@@ -343,18 +360,19 @@ __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell, unsi
 
 // Returns the workgroup's packed (requests, fragments) total.
 template <bool FUSED>
-__device__ __forceinline__ uint64_t ra_flag_step(const RaArgs &a, uint32_t i, uint64_t *wave_tot)
+__device__ __forceinline__ uint64_t ra_flag_step(const RaArgs &a, uint32_t i, uint64_t *wave_tot, RaMine &mine)
 {
   const uint32_t n = ra_n(a);
   unsigned long long pack = 0;
   if (i < n) {
-    const uint32_t cell = a.arr_cell[i];
+    const uint32_t cell = FUSED ? mine.cell : a.arr_cell[i];
     const uint32_t r = cell != kRaNoCell ? a.rec[cell] : kRaNoRec;
     if (r != kRaNoRec) {
-      const uint32_t fidx = a.arr_fidx[i];
+      const uint32_t fidx = FUSED ? mine.fidx : a.arr_fidx[i];
       if (fidx < SG_MAX_BI_SIZE) {
         // rr_emplace_mbuf: the entry goes where its sequence number says
-        a.tab[(size_t)r * SG_MAX_BI_SIZE + fidx] = (unsigned long long)a.arrivals[i] | ((unsigned long long)a.arr_len[i] << 32);
+        a.tab[(size_t)r * SG_MAX_BI_SIZE + fidx] =
+            (unsigned long long)(FUSED ? mine.slot : a.arrivals[i]) | ((unsigned long long)(FUSED ? mine.len : a.arr_len[i]) << 32);
       } else {
         refuse(a.status, a.status_flag, kStBadTable);  // beyond what a request's tables hold (src/p2p_bufs.h:10)
       }
@@ -368,14 +386,16 @@ __device__ __forceinline__ uint64_t ra_flag_step(const RaArgs &a, uint32_t i, ui
   }
   uint64_t tot;
   const uint64_t ex = block_exclusive_scan<kRaBlock>(pack, wave_tot, &tot);
-  if (i < n) a.arr_pack[i] = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
+  mine.pack = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
+  if (!FUSED && i < n) a.arr_pack[i] = mine.pack;
   return tot;
 }
 
 __global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
 {
   __shared__ uint64_t wave_tot[kRaBlock / kWave];
-  const uint64_t tot = ra_flag_step<false>(a, blockIdx.x * kRaBlock + threadIdx.x, wave_tot);
+  RaMine mine;
+  const uint64_t tot = ra_flag_step<false>(a, blockIdx.x * kRaBlock + threadIdx.x, wave_tot, mine);
   if (threadIdx.x == 0) a.blk[blockIdx.x] = tot;
 }
 
@@ -436,7 +456,7 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
 // to the free ring, the cell is emptied.  The request's rank and first fragment
 // index hang on that arrival (arr_pack there plus its workgroup's scanned total).
 template <bool FUSED>
-__device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32_t *take, bool overflow)
+__device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32_t *take, bool overflow, const RaMine &mine)
 {
   const uint32_t n = ra_n(a);
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -444,8 +464,8 @@ __device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32
   unsigned long long v = 0;
   bool completes = false;
   if (i < n) {
-    cell = a.arr_cell[i];
-    const unsigned long long p = a.arr_pack[i];
+    cell = FUSED ? mine.cell : a.arr_cell[i];
+    const unsigned long long p = FUSED ? mine.pack : a.arr_pack[i];
     completes = cell != kRaNoCell && (p >> 63) && !overflow;
     if (completes) v = (p & ~(1ull << 63)) + (FUSED ? 0ull : a.blk[i / kRaBlock]);  // one workgroup: nothing before it
     // the position of a request's last arrival counts per call
@@ -524,7 +544,7 @@ __device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32
 __global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
 {
   __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
-  ra_emit_step<false>(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take, a.words[kRaOverflow] != 0);
+  ra_emit_step<false>(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take, a.words[kRaOverflow] != 0, RaMine());
 }
 
 // A burst of at most kRaTakeBlock arrivals: the four steps by one workgroup in one launch.
@@ -535,12 +555,13 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_burst(RaArgs a)
   __shared__ uint64_t wave_tot[kRaBlock / kWave];
   __shared__ uint32_t overflow;
   const uint32_t i = threadIdx.x;
-  ra_insert_step(a, i, take);
+  RaMine mine;
+  ra_insert_step<true>(a, i, take, mine);
   __syncthreads();
-  const uint64_t tot = ra_flag_step<true>(a, i, wave_tot);
+  const uint64_t tot = ra_flag_step<true>(a, i, wave_tot, mine);
   if (threadIdx.x == 0) overflow = ra_scan_finish<true>(a, tot);
   __syncthreads();
-  ra_emit_step<true>(a, i, take, overflow != 0);
+  ra_emit_step<true>(a, i, take, overflow != 0, mine);
 }
 
 // Empties the table: every cell, every record, all records back in the ring.
