@@ -202,3 +202,46 @@ def test_small_and_large_calls_in_turns():
     got = arena.cpu().numpy()
     assert np.array_equal(got, want), first_diff(got, want)
     c.close()
+
+
+def test_two_contexts_working_side_by_side():
+    """A context per direction, each on a stream of its own, queued without
+    waits (what the benchmark's step does): one gathers a ResNet-sized batch
+    round after round while the other scatters the responses of a LeNet-sized
+    one; arenas the batches do not divide, so every call starts somewhere else.
+    Arena, TX ring and both cursors are held against the oracle at the end."""
+    wg, ws = synth.make_workload(2, 6), synth.make_workload(1, 300)
+    dg, ds = DeviceWorkload(wg), DeviceWorkload(ws)
+    cap_g = 2 * int(wg.req_sizes.sum()) + 1001
+    arena_g = torch.zeros(cap_g, dtype=torch.uint8, device=DEV)
+    cap_s = int(ws.resp_sizes.sum()) + 333
+    resp_np = np.random.default_rng(9).integers(0, 256, cap_s, dtype=np.uint8)
+    arena_s = to_dev(resp_np, DEV)
+    g, s = SgContext(0, max_reqs=4096, max_frames=1 << 16), SgContext(0, max_reqs=4096, max_frames=1 << 16)
+    ga = g.gather_args(dg.rx, dg.frag_slot, None, dg.req_first, dg.n_req, dg.n_frags, AppRef(arena=arena_g, cap=cap_g),
+                       None, flags=capi.F_ASYNC | capi.F_RULE_FRAGS, fixed_req_size=int(wg.req_sizes[0]), mtu=wg.mtu)
+    sa = s.scatter_args(ds.rx, ds.tx, ds.tx_slot, ds.hdr_src_slot, ds.resp_first, None, int(ws.resp_sizes[0]), ds.n_req,
+                        ds.n_frames, ws.mtu, AppRef(arena=arena_s, cap=cap_s), None, ws.flags | capi.F_ASYNC)
+    g.set_cursor(0, 77)
+    s.set_cursor(1, 5)
+    torch.cuda.synchronize()
+    rounds = 7
+    for _ in range(rounds):
+        g.gather_batch_raw(ga)
+        s.scatter_batch_raw(sa)
+    g.sync()
+    s.sync()
+    want = np.zeros(cap_g, np.uint8)
+    cur_g, cur_s = 77, 5
+    tx = None
+    for _ in range(rounds):
+        want, _, cur_g = oracle.gather(wg, arena_cap=cap_g, cursor=cur_g, out=want)
+        tx = ws.tx_ring_init.copy()
+        _, cur_s = oracle.scatter(ws, ws.ring, tx, resp_np, arena_cap=cap_s, cursor=cur_s)
+    got = arena_g.cpu().numpy()
+    assert np.array_equal(got, want), first_diff(got, want)
+    got = ds.tx_ring.cpu().numpy()
+    assert np.array_equal(got, tx), first_diff(got, tx)
+    assert g.get_cursor(0) == cur_g and s.get_cursor(1) == cur_s
+    g.close()
+    s.close()
