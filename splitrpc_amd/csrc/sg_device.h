@@ -101,9 +101,10 @@ __device__ __forceinline__ T sload_here(const T *p)
 //    The queue word becomes visible before the stamp (a fence between the two
 //    stores; readers take a cell in one scalar load), so a cell that shows the
 //    new version also shows the whole new stamp.  Finding the live cell costs a
-//    wavefront some twenty scalar instructions, which the scalar-bound kernels
-//    of large calls feel (5 % on 400 000 response frames): the host picks this
-//    form for calls of few wavefronts and the trailing kernel for the others.
+//    wavefront two 8-dword scalar loads and some twenty scalar instructions
+//    (the gather of 220672 fragments alone 104.2 -> 106.7 us), so the kernels
+//    that do it are instances of their own (ADV) and the host picks them for
+//    calls of up to 65536 wavefronts, the trailing kernel for larger ones.
 // The plain word and the live cell hold the same value whenever no kernel that
 // writes them is running: whoever advances the cursor writes both (the plain
 // word is read by no wavefront of a self-advancing kernel, the cells by none of
