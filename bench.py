@@ -283,6 +283,39 @@ def per_request_calls(ctx, dw, calls: int = 300):
             "GBps": round((2 * size + 16 * int(skbs[0].num_items)) / dt / 1e9, 2)}
 
 
+def native_loop_time(ctx, ctx_tx, pool: "Pool", steps: int):
+    """Seconds per step when the loop that issues the calls is native code
+    (sgh_step_loop_gpu of libsg_host.so: what a C++ shunter thread does, without
+    the interpreter between the calls); the argument sets are the ones the
+    Python loop has used."""
+    import ctypes as C
+    from splitrpc_amd import capi
+    if pool.w.tx_in_place:
+        return None
+    host = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(__file__)), "splitrpc_amd", "libsg_host.so"))
+    fn = host.sgh_step_loop_gpu
+    fn.restype = C.c_double
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32]
+    tx = ctx_tx if ctx_tx is not None else ctx
+    for i in range(len(pool.items)):
+        pool.step(ctx, i, capi.F_ASYNC, ctx_tx)      # every item has its argument sets
+    ctx.sync()
+    tx.sync()
+    gas = [next(v for k, v in dw._args.items() if k[0] == "g") for dw in pool.items]
+    sas = [next(v for k, v in dw._args.items() if k[0] == "s") for dw in pool.items]
+    n = len(pool.items)
+    ga = (C.c_void_p * n)(*[C.addressof(a) for a in gas])
+    sa = (C.c_void_p * n)(*[C.addressof(a) for a in sas])
+    runs = []
+    for rep in range(5):
+        dt = fn(ctx.h, tx.h, ga, sa, n, steps)
+        if dt < 0:
+            raise RuntimeError(f"sgh_step_loop_gpu failed: {dt}")
+        runs.append(dt / steps)
+    runs.sort()
+    return runs[len(runs) // 2]
+
+
 def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, replays: int = 50,
                     streams: int = 1):
     """Seconds per step of the single-batch call when `steps` steps are recorded
@@ -583,6 +616,11 @@ def main() -> int:
                   "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in k1.items()},
                   "k_gather_GBps": round(p1.gather_bytes / (k1["k_gather"][0] * 1e-3) / 1e9, 1)
                   if k1["k_gather"][0] > 0 else None}
+        nl = native_loop_time(ctx, ctx_tx, p1, max(a.steps, 200))
+        if nl is not None:
+            single["native_loop_ms_per_step"] = round(nl * 1e3, 5)
+            single["native_loop_GBps"] = round(b1 / nl / 1e9, 1)
+            single["native_loop_requests_per_sec"] = round(p1.n_req / nl, 1)
         del p1
         for n_streams in (1, 2, 4):
             sg = graph_step_time(w, extra, rule, a.rotate_mb, streams=n_streams)

@@ -4,6 +4,7 @@
 // others are pure host logic.
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cstring>
 #include <thread>
 #include <vector>
@@ -453,5 +454,30 @@ void *sgh_mempool_req_base(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p
 uint64_t sgh_mempool_req_bytes(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_req_addr_pool_size(); }
 void *sgh_mempool_resp_base(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_resp_addr_range(); }
 uint64_t sgh_mempool_resp_bytes(void *p) { return static_cast<P2pRpcAppRrMemPool *>(p)->get_resp_addr_pool_size(); }
+
+// `steps` steps of the batched hot path from a native loop, as a shunter thread would issue
+// them: step i is one asynchronous gather call on `g` and one asynchronous scatter call on `s`
+// (the same context, or one per direction) with the i-th of `n` prepared argument sets, taken
+// in turns; both contexts are waited for at the end.  Returns the seconds the loop took, or a
+// negative error code.
+double sgh_step_loop_gpu(sg_hip_ctx *g, sg_hip_ctx *s, const sg_gather_args *const *ga,
+                         const sg_scatter_args *const *sa, uint32_t n, uint32_t steps)
+{
+  if (!g || !s || !ga || !sa || n == 0) return (double)SG_E_INVAL;
+  int rc = sg_hip_sync(g);
+  if (rc == SG_OK && s != g) rc = sg_hip_sync(s);
+  if (rc != SG_OK) return (double)rc;
+  const auto t0 = std::chrono::steady_clock::now();
+  for (uint32_t i = 0; i < steps; i++) {
+    rc = sg_hip_gather_batch(g, ga[i % n]);
+    if (rc != SG_OK) return (double)rc;
+    rc = sg_hip_scatter_batch(s, sa[i % n]);
+    if (rc != SG_OK) return (double)rc;
+  }
+  rc = sg_hip_sync(g);
+  if (rc == SG_OK && s != g) rc = sg_hip_sync(s);
+  if (rc != SG_OK) return (double)rc;
+  return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
 
 }  // extern "C"
