@@ -42,6 +42,8 @@ MEASURED_TRAFFIC = {
     (4, 8, "k_gather"): 661.9e6, (4, 8, "k_scatter"): 676.0e6,
     (5, 4, "k_gather"): 817.6e6, (5, 4, "k_scatter"): 549.3e6,
 }
+# the same for the reference's own 64-byte header (bench.py --ref64)
+MEASURED_TRAFFIC_REF64 = {}
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 
@@ -129,12 +131,44 @@ class Pool:
             dw.scatter(ctx, flags | self.extra_flags, fuse=self.rule, reuse=True)
 
 
-def timed(ctx, pool: Pool, steps: int, warmup: int, ctx_tx=None, reps: int = 5):
-    """Seconds per step: `warmup` untimed steps, then `reps` timed runs of
-    exactly `steps` steps each, bracketed by synchronization on both sides; the
-    median run is reported (one run of 20 steps of 0.1 ms is a 2 ms sample)."""
+MIN_TIMED_MS = 50.0
+
+
+def stat_line(ns) -> list:
+    """[N, Mean, p90, p95, p99, min, max] of nanosecond samples, the summary the
+    reference prints for its GDelay / SDelay vectors (print_stat,
+    src/utils/stats_utils.h:69-79; a percentile is the sample at index
+    round(p * (N - 1)) of the sorted samples, :10-21)."""
+    v = sorted(int(x) for x in ns)
+    if not v:
+        return [0, 0.0, 0.0, 0.0, 0.0, 0, 0]
+    pick = lambda p: float(v[int(round(p * (len(v) - 1)))])
+    return [len(v), round(sum(v) / len(v), 2), pick(0.90), pick(0.95), pick(0.99), v[0], v[-1]]
+
+
+class Timing(float):
+    """Seconds per step (the median run, by the events on the streams), with
+    what it was taken from."""
+    host_clock = 0.0   # the same runs by the host's clock around a drain
+    runs = 0
+    timed_ms = 0.0
+
+
+def timed(ctx, pool: Pool, steps: int, warmup: int, ctx_tx=None, reps: int = 5, min_ms: float = MIN_TIMED_MS,
+          shunt: bool = False) -> Timing:
+    """Seconds per step: `warmup` untimed steps, then timed runs of exactly
+    `steps` steps each, every run bracketed by synchronization on both sides --
+    at least `reps` runs and as many as it takes to have `min_ms` milliseconds
+    timed in all (one run of 20 steps of 0.1 ms is a 2 ms sample).  A run is
+    clocked twice: by events recorded on the streams the calls go to (the first
+    before the run's first call, the last behind its last call on either
+    stream), and by the host's clock around the run and the drain behind it.
+    The median run by the events is the figure; the host clock's median, which
+    carries the cost of the drain itself, rides along."""
     import torch
     from splitrpc_amd import capi
+
+    streams = [torch.cuda.ExternalStream(c.stream, device="cuda:0") for c in (ctx, ctx_tx) if c is not None]
 
     def drain():
         ctx.sync()
@@ -142,28 +176,54 @@ def timed(ctx, pool: Pool, steps: int, warmup: int, ctx_tx=None, reps: int = 5):
             ctx_tx.sync()
         torch.cuda.synchronize()
 
+    def step(i):
+        if shunt:
+            pool.items[i % len(pool.items)].shunt(ctx, capi.F_ASYNC | pool.extra_flags, rule=pool.rule)
+        else:
+            pool.step(ctx, i, capi.F_ASYNC, ctx_tx)
+
     # every rotated copy is touched at least once before the clock starts
     for i in range(max(warmup, len(pool.items))):
-        pool.step(ctx, i, capi.F_ASYNC, ctx_tx)
+        step(i)
     drain()
-    runs = []
-    for rep in range(reps):
+    ev_runs, host_runs, total = [], [], 0.0
+    while len(ev_runs) < reps or total < min_ms * 1e-3:
+        e0 = torch.cuda.Event(enable_timing=True)
+        ends = [torch.cuda.Event(enable_timing=True) for _ in streams]
         t0 = time.perf_counter()
+        e0.record(streams[0])
         for i in range(steps):
-            pool.step(ctx, warmup + i, capi.F_ASYNC, ctx_tx)
+            step(warmup + i)
+        for e, st in zip(ends, streams):
+            e.record(st)
         drain()
-        runs.append((time.perf_counter() - t0) / steps)
-    runs.sort()
-    return runs[len(runs) // 2]
+        host = time.perf_counter() - t0
+        ev = max(e0.elapsed_time(e) for e in ends) * 1e-3
+        ev_runs.append(ev / steps)
+        host_runs.append(host / steps)
+        total += ev
+        if len(ev_runs) >= 2000:
+            break
+    ev_runs.sort()
+    host_runs.sort()
+    t = Timing(ev_runs[len(ev_runs) // 2])
+    t.host_clock = host_runs[len(host_runs) // 2]
+    t.runs = len(ev_runs)
+    t.timed_ms = total * 1e3
+    return t
 
 
-def kernel_times(ctx, pool: Pool, steps: int):
+def kernel_times(ctx, pool: Pool, steps: int, shunt: bool = False):
     """Average duration of each kernel from HIP events recorded around every
-    launch on the stream the kernels run on."""
+    launch on the stream the kernels run on.  `shunt`: one launch per step that
+    carries both directions (counted under k_gather)."""
     from splitrpc_amd import capi
     ctx.set_profiling(True)
     for i in range(steps):
-        pool.step(ctx, i, capi.F_ASYNC)
+        if shunt:
+            pool.items[i % len(pool.items)].shunt(ctx, capi.F_ASYNC | pool.extra_flags, rule=pool.rule)
+        else:
+            pool.step(ctx, i, capi.F_ASYNC)
     out = {}
     for which, name in ((0, "k_prep"), (1, "k_gather"), (2, "k_scatter")):
         ms, n = ctx.kernel_time(which)
@@ -273,14 +333,18 @@ def per_request_calls(ctx, dw, calls: int = 300):
     fn = ctx.lib.sg_hip_gather
     for i in range(20):
         assert fn(ctx.h, C.byref(skbs[i % len(skbs)])) == 0
+    lat = []
     t0 = time.perf_counter()
     for i in range(calls):
+        a = time.perf_counter_ns()
         fn(ctx.h, C.byref(skbs[i % len(skbs)]))
+        lat.append(time.perf_counter_ns() - a)
     dt = (time.perf_counter() - t0) / calls
     size = int(w.req_sizes[0])
     return {"us_per_gather_call": round(dt * 1e6, 2), "runs_per_request": int(skbs[0].num_items),
             "request_bytes": size, "requests_per_sec": round(1.0 / dt, 1),
-            "GBps": round((2 * size + 16 * int(skbs[0].num_items)) / dt / 1e9, 2)}
+            "GBps": round((2 * size + 16 * int(skbs[0].num_items)) / dt / 1e9, 2),
+            "latency_ns_[N,Mean,p90,p95,p99,min,max]": stat_line(lat)}
 
 
 def native_loop_time(ctx, ctx_tx, pool: "Pool", steps: int):
@@ -316,8 +380,113 @@ def native_loop_time(ctx, ctx_tx, pool: "Pool", steps: int):
     return runs[len(runs) // 2]
 
 
+def _host_lib():
+    import ctypes as C
+    host = C.CDLL(os.path.join(ROOT, "splitrpc_amd", "libsg_host.so"))
+    host.sgh_shunt_loop_gpu.restype = C.c_double
+    host.sgh_shunt_loop_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
+    host.sgh_engine_loop_gpu.restype = C.c_int
+    host.sgh_engine_loop_gpu.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
+                                         C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint64,
+                                         C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint32, C.c_uint64, C.c_uint64,
+                                         C.c_uint32, C.c_uint32, C.c_void_p]
+    return host
+
+
+def native_shunt_loop(ctxs, pool: "Pool", steps: int, latency: bool = False):
+    """One sg_hip_shunt_batch call per step (both directions in one launch)
+    from a native loop over `ctxs`, taken in turns so that len(ctxs) calls are
+    in flight (sgh_shunt_loop_gpu of libsg_host.so).  Returns seconds per step
+    (median of 5 loops); with `latency` (one context) every call is made
+    synchronous and the calls' nanoseconds come back as well."""
+    import ctypes as C
+    import numpy as np
+    from splitrpc_amd import capi
+    if pool.w.tx_in_place:
+        return None
+    host = _host_lib()
+    for dw in pool.items:
+        dw.shunt(ctxs[0], capi.F_ASYNC | pool.extra_flags, rule=pool.rule)  # builds and keeps the argument sets
+    ctxs[0].sync()
+    gas = [next(v for k, v in dw._args.items() if k[0] == "g") for dw in pool.items]
+    sas = [next(v for k, v in dw._args.items() if k[0] == "s") for dw in pool.items]
+    for g_, s_ in zip(gas, sas):
+        g_.flags |= capi.F_ASYNC
+        s_.flags |= capi.F_ASYNC
+    n = len(pool.items)
+    ga = (C.c_void_p * n)(*[C.addressof(x) for x in gas])
+    sa = (C.c_void_p * n)(*[C.addressof(x) for x in sas])
+    hs = (C.c_void_p * len(ctxs))(*[c.h for c in ctxs])
+    if latency:
+        lat = np.zeros(steps, np.uint64)
+        dt = host.sgh_shunt_loop_gpu(hs, 1, ga, sa, n, steps, lat.ctypes.data_as(C.c_void_p))
+        if dt < 0:
+            raise RuntimeError(f"sgh_shunt_loop_gpu failed: {dt}")
+        return dt / steps, lat
+    runs = []
+    for rep in range(5):
+        dt = host.sgh_shunt_loop_gpu(hs, len(ctxs), ga, sa, n, steps, None)
+        if dt < 0:
+            raise RuntimeError(f"sgh_shunt_loop_gpu failed: {dt}")
+        runs.append(dt / steps)
+    runs.sort()
+    return runs[len(runs) // 2]
+
+
+def host_engine_batched(pool: "Pool", steps: int) -> dict:
+    """The batched calls of the C++ drop-in, P2pRpcSgHipEngine::gather_batch(P2pRpcRr **) and
+    scatter_batch(P2pRpcRr **), over the requests of one default call held as P2pRpcRr objects
+    (sgh_engine_loop_gpu of libsg_host.so): with the engine walking every fragment on the host,
+    and with the requests' fragment tables kept where the device reads them.  Response headers
+    come from the connections' templates here (fresh response buffers, rr_set_hdr)."""
+    import ctypes as C
+    import numpy as np
+    w = pool.w
+    if w.in_tensor_sizes or w.out_tensor_sizes or w.tx_in_place or len(set(int(x) for x in w.req_sizes)) != 1:
+        return None
+    host = _host_lib()
+    items = pool.items[:2]
+    dw = items[0]
+    bases = np.array([[d.ring.data_ptr(), d.tx_ring.data_ptr(), d.req_arena.data_ptr(), d.resp_arena.data_ptr()]
+                      for d in items], np.uint64).reshape(-1)
+    fs = np.ascontiguousarray(dw.frag_slot.cpu().numpy().view(np.uint32))
+    fl = np.ascontiguousarray(dw.frag_len.cpu().numpy().view(np.uint32))
+    ts = np.ascontiguousarray(dw.tx_slot.cpu().numpy().view(np.uint32))
+    per, per_resp = dw.n_frags // dw.n_req, dw.n_frames // dw.n_req
+    pv = lambda x: x.ctypes.data_as(C.c_void_p)
+    out = {"requests": dw.n_req, "fragments": dw.n_frags, "response_frames": dw.n_frames}
+    total = pool.gather_bytes + pool.scatter_bytes
+    for mode, name in ((0, "tables_walked_by_the_host"), (1, "tables_pulled_by_the_device")):
+        res = np.zeros(16, np.float64)
+        rc = host.sgh_engine_loop_gpu(0, mode, len(items), pv(bases), dw.rx.n_slots, w.slot_size, w.profile, pv(fs),
+                                      pv(fl), dw.n_req, per, int(w.req_sizes[0]), dw.req_app.cap, w.mtu,
+                                      dw.tx.n_slots, pv(ts), per_resp, int(w.resp_sizes[0]), dw.resp_app.cap,
+                                      w.flags, steps, pv(res))
+        if rc != 0:
+            raise RuntimeError(f"sgh_engine_loop_gpu mode {mode} failed: {rc}")
+        sec = float(res[0])
+        out[name] = {"us_per_step": round(sec * 1e6, 2), "GBps": round(total / sec / 1e9, 1),
+                     "frac_of_hbm_peak": round(total / sec / 1e9 / HBM_PEAK_GBS, 4),
+                     "requests_per_sec": round(dw.n_req / sec, 1),
+                     "host_us_per_gather_batch_call": round(float(res[2]) * 1e-3, 2),
+                     "host_us_per_scatter_batch_call": round(float(res[9]) * 1e-3, 2),
+                     "gather_batch_host_ns_[N,Mean,p90,p95,p99,min,max]": [round(float(x), 2) for x in res[1:8]],
+                     "scatter_batch_host_ns_[N,Mean,p90,p95,p99,min,max]": [round(float(x), 2) for x in res[8:15]]}
+    # the reference's own call through the same engine: one synchronous gather(rr, stub) per request
+    res = np.zeros(16, np.float64)
+    rc = host.sgh_engine_loop_gpu(0, 2, len(items), pv(bases), dw.rx.n_slots, w.slot_size, w.profile, pv(fs), pv(fl),
+                                  dw.n_req, per, int(w.req_sizes[0]), dw.req_app.cap, w.mtu, dw.tx.n_slots, pv(ts),
+                                  per_resp, int(w.resp_sizes[0]), dw.resp_app.cap, w.flags, 2000, pv(res))
+    if rc != 0:
+        raise RuntimeError(f"sgh_engine_loop_gpu mode 2 failed: {rc}")
+    out["per_request_gather"] = {"us_per_call": round(float(res[0]) * 1e6, 2),
+                                 "requests_per_sec": round(1.0 / float(res[0]), 1),
+                                 "GDelay_ns_[N,Mean,p90,p95,p99,min,max]": [round(float(x), 2) for x in res[1:8]]}
+    return out
+
+
 def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, replays: int = 50,
-                    streams: int = 1):
+                    streams: int = 1, shunt: bool = False):
     """Seconds per step of the single-batch call when `steps` steps are recorded
     into one HIP graph per stream and the graphs are replayed: the launch-bound
     loop without the per-launch host cost.  With `streams` > 1 that many
@@ -333,21 +502,28 @@ def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, 
         ctx = SgContext(0, max_reqs=max(4096, w.n_req), max_frames=max(65536, w.n_frags, w.n_resp_frames),
                         stream=stream.cuda_stream)
         pool = Pool(w, 1, max(64, rotate_mb // streams), extra, rule=rule)
+
+        def one(i, ctx=ctx, pool=pool):
+            if shunt:
+                pool.items[i % len(pool.items)].shunt(ctx, capi.F_ASYNC | pool.extra_flags, rule=pool.rule)
+            else:
+                pool.step(ctx, i, capi.F_ASYNC)
+
         for i in range(len(pool.items)):
-            pool.step(ctx, i, capi.F_ASYNC)
+            one(i)
         ctx.sync()
-        lanes.append((stream, ctx, pool))
+        lanes.append((stream, ctx, pool, one))
     torch.cuda.synchronize()
     graphs = []
-    for stream, ctx, pool in lanes:
+    for stream, ctx, pool, one in lanes:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, stream=stream):
             for i in range(steps):
-                pool.step(ctx, i, capi.F_ASYNC)
+                one(i)
         graphs.append(g)
 
     def replay_all():
-        for (stream, _, _), g in zip(lanes, graphs):
+        for (stream, _, _, _), g in zip(lanes, graphs):
             with torch.cuda.stream(stream):
                 g.replay()
 
@@ -359,37 +535,58 @@ def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, 
         replay_all()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / (replays * steps * streams)
-    for _, ctx, _ in lanes:
+    for _, ctx, _, _ in lanes:
         ctx.sync()
         ctx.close()
     return dt
 
 
-def device_pipeline(w, dw, bursts=(256, 1024, 4096)) -> dict:
+def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 65536, 0)) -> dict:
     """The receive path end to end on the device, burst after burst and no
-    host wait in between: sg_hip_reassemble files a burst's arrivals (requests
-    that stay incomplete wait on the device), sg_hip_gather_batch gathers the
-    requests the burst completed (their number stays on the device),
-    sg_hip_scatter_batch answers them.  All arrivals of one default call's
-    worth of requests, in arrival order; wall time over the whole stream."""
+    host wait in between, from a native loop (sgh_pipeline_loop_gpu of
+    libsg_host.so): sg_hip_reassemble files a burst's arrivals (requests that
+    stay incomplete wait on the device), then the requests the burst completed
+    are gathered and answered (their number stays on the device):
+    sg_hip_shunt_batch, one launch for both directions where the burst is small
+    enough, else a gather and a scatter call.  The stream of arrivals is that
+    of `calls` default calls' worth of requests (the pool's ring copies in
+    turns), in arrival order; wall time over the whole stream (burst 0 = a
+    whole call's arrivals per burst).  Two forms:
+      one_stream   the calls of a burst one after the other on one context
+      overlapped   the reassembly on a context (stream) of its own, its output
+                   tables double-buffered, events between the two streams: burst
+                   k + 1 is filed while burst k is gathered and answered"""
+    import ctypes as C
     import numpy as np
     import torch
     from splitrpc_amd import capi
     from splitrpc_amd.engine import AppRef, RingRef, SgContext, to_dev
+    w = pool.w
     if w.in_tensor_sizes or w.out_tensor_sizes or w.tx_in_place or len(set(int(x) for x in w.req_sizes)) != 1:
         return None
+    host = _host_lib()
+    host.sgh_pipeline_loop_gpu.restype = C.c_double
+    host.sgh_pipeline_loop_gpu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
     dev = "cuda:0"
+    items = pool.items
+    dw = items[0]
     size, rsize = int(w.req_sizes[0]), int(w.resp_sizes[0])
     per, per_resp = -(-size // w.mtu), -(-rsize // w.mtu)
     n_arr = int(dw.arrivals.numel())
-    out = {"arrivals": n_arr, "requests": dw.n_req}
+    out = {"arrivals_per_call": n_arr, "requests_per_call": dw.n_req, "calls": calls}
+    total_bytes = (pool.gather_bytes + pool.scatter_bytes) * calls
     for burst in bursts:
-        bound = burst // per + 2                      # requests one burst can complete
-        ctx = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=max(65536, bound * per))
-        ctx.reassemble_reset()
+        burst = burst or n_arr
+        if burst > n_arr:
+            continue
+        bound = min(burst // per + 2, dw.n_req)           # requests one burst can complete
+        mf = max(65536, bound * per, burst)
+        ctx_ra = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=mf)
+        ctx_sg = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=mf)
         i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
-        fs, fl, rf, hdr, counts = i32(max(65536, bound * per)), i32(max(65536, bound * per)), i32(4097 + dw.n_req), \
-            i32(4096 + dw.n_req), i32(4)
+        # reassembly output, twice: while the copy reads one set the next burst fills the other
+        sets = [dict(fs=i32(mf), fl=i32(mf), rf=i32(4097 + dw.n_req), hdr=i32(4096 + dw.n_req), counts=i32(4))
+                for _ in range(2)]
         req_cap, resp_cap = 4 * bound * size, 4 * bound * rsize
         req_arena = torch.zeros(req_cap, dtype=torch.uint8, device=dev)
         resp_arena = torch.zeros(resp_cap, dtype=torch.uint8, device=dev)
@@ -398,33 +595,54 @@ def device_pipeline(w, dw, bursts=(256, 1024, 4096)) -> dict:
         tx_slot = to_dev(np.arange(bound * per_resp, dtype=np.uint32), dev)
         resp_first = to_dev((np.arange(bound + 1) * per_resp).astype(np.uint32), dev)
         A = capi.F_ASYNC
-        ga = ctx.gather_args(dw.rx, fs, None, rf, bound, bound * per, AppRef(arena=req_arena, cap=req_cap), None,
-                             flags=A | capi.F_RULE_FRAGS, fixed_req_size=size, mtu=w.mtu, counts=counts)
-        sa = ctx.scatter_args(dw.rx, tx, tx_slot, None, resp_first, None, rsize, bound, bound * per_resp, w.mtu,
-                              AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A, hdr_src_req=hdr, counts=counts)
-        ras = [ctx.reassemble_args(dw.rx, dw.arrivals[b:b + burst], min(burst, n_arr - b), fs, fl, rf,
-                                   req_hdr_slot=hdr, counts_out=counts, flags=A) for b in range(0, n_arr, burst)]
-        torch.cuda.synchronize()
-        best = None
-        for rep in range(3):
-            ctx.reassemble_reset()
-            t0 = time.perf_counter()
-            for k, ra in enumerate(ras):
-                ctx.reassemble_raw(ra)
-                ctx.gather_batch_raw(ga)
-                ctx.scatter_batch_raw(sa)
-                if k % 64 == 63:
-                    ctx.sync()
-            ctx.sync()
-            dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
-        left = int(counts.cpu()[3])
-        out[str(burst)] = {"us_per_burst": round(best / len(ras) * 1e6, 2), "arrivals_per_sec": round(n_arr / best, 1),
-                           "requests_per_sec": round(dw.n_req / best, 1),
-                           "payload_Gbit_per_sec": round(8.0 * size * dw.n_req / best / 1e9, 1),
-                           "requests_left_in_flight": left}
-        ctx.close()
-        del fs, fl, rf, hdr, counts, req_arena, resp_arena, tx_ring
+        ras, gas, sas = [], [], []
+        by_item = {}
+        for call in range(calls):
+            it = items[call % len(items)]
+            for b in range(0, n_arr, burst):
+                j = len(ras) & 1
+                t = sets[j]
+                key = (call % len(items), j)
+                if key not in by_item:
+                    by_item[key] = (
+                        ctx_sg.gather_args(it.rx, t["fs"], None, t["rf"], bound, bound * per,
+                                           AppRef(arena=req_arena, cap=req_cap), None, flags=A | capi.F_RULE_FRAGS,
+                                           fixed_req_size=size, mtu=w.mtu, counts=t["counts"]),
+                        ctx_sg.scatter_args(it.rx, tx, tx_slot, None, resp_first, None, rsize, bound, bound * per_resp,
+                                            w.mtu, AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A,
+                                            hdr_src_req=t["hdr"], counts=t["counts"]))
+                ras.append(ctx_sg.reassemble_args(it.rx, it.arrivals[b:b + burst], min(burst, n_arr - b), t["fs"],
+                                                  t["fl"], t["rf"], req_hdr_slot=t["hdr"], counts_out=t["counts"],
+                                                  flags=A))
+                gas.append(by_item[key][0])
+                sas.append(by_item[key][1])
+        n_bursts = len(ras)
+        arr = lambda xs: (C.c_void_p * len(xs))(*[C.addressof(x) for x in xs])
+        c_ras, c_gas, c_sas = arr(ras), arr(gas), arr(sas)
+        res = {}
+        for form in ("one_stream", "overlapped"):
+            c_ra = ctx_sg if form == "one_stream" else ctx_ra
+            best = None
+            for rep in range(3):
+                c_ra.reassemble_reset()
+                torch.cuda.synchronize()
+                dt = host.sgh_pipeline_loop_gpu(c_ra.h, ctx_sg.h, c_ras, c_gas, c_sas, n_bursts,
+                                                1 if form == "overlapped" else 0)
+                if dt < 0:
+                    raise RuntimeError(f"sgh_pipeline_loop_gpu failed: {dt} {ctx_sg.lib.sg_hip_last_error(ctx_sg.h)}")
+                best = dt if best is None else min(best, dt)
+            left = int(sets[(n_bursts - 1) & 1]["counts"].cpu()[3])
+            res[form] = {"us_per_burst": round(best / n_bursts * 1e6, 2),
+                         "arrivals_per_sec": round(n_arr * calls / best, 1),
+                         "requests_per_sec": round(dw.n_req * calls / best, 1),
+                         "payload_Gbit_per_sec": round(8.0 * size * dw.n_req * calls / best / 1e9, 1),
+                         "GBps": round(total_bytes / best / 1e9, 1),
+                         "frac_of_hbm_peak": round(total_bytes / best / 1e9 / HBM_PEAK_GBS, 4),
+                         "requests_left_in_flight": left}
+        out[str(burst)] = res
+        ctx_ra.close()
+        ctx_sg.close()
+        del sets, req_arena, resp_arena, tx_ring, gas, sas, ras, by_item
         torch.cuda.empty_cache()
     return out
 
@@ -515,7 +733,8 @@ def main() -> int:
         del src, dst
 
     sec = timed(ctx, pool, a.steps, a.warmup, ctx_tx)
-    _log(f"timed: {sec * 1e6:.1f} us per step (median of 5 runs of {a.steps} steps)")
+    _log(f"timed: {sec * 1e6:.1f} us per step by the streams' events, {sec.host_clock * 1e6:.1f} us by the host clock "
+         f"(medians of {sec.runs} runs of {a.steps} steps, {sec.timed_ms:.1f} ms timed)")
     kt = kernel_times(ctx, pool, min(a.steps, 100))
     total_bytes = pool.gather_bytes + pool.scatter_bytes
     value = total_bytes / sec / 1e9
@@ -556,10 +775,14 @@ def main() -> int:
     for b in range(0, n_b, 64):
         ctx.reassemble(dw0.rx, dw0.arrivals[b:b + 64], min(64, n_b - b), ra_fs, ra_fl, ra_rf, **ra_kw)
     ctx.reassemble_reset()
+    lat = []
     t0 = time.perf_counter()
     for b in range(0, n_b, 64):
+        t1 = time.perf_counter_ns()
         ctx.reassemble(dw0.rx, dw0.arrivals[b:b + 64], min(64, n_b - b), ra_fs, ra_fl, ra_rf, **ra_kw)
+        lat.append(time.perf_counter_ns() - t1)
     reassembly["us_per_burst_of_64"] = round((time.perf_counter() - t0) / max(1, (n_b + 63) // 64) * 1e6, 2)
+    reassembly["burst_of_64_latency_ns_[N,Mean,p90,p95,p99,min,max]"] = stat_line(lat)
     ctx.reassemble_reset()
     # the same bursts queued without waiting for each one's counts (they stay on the device, where the
     # gather reads them): what a burst costs the stream
@@ -579,7 +802,7 @@ def main() -> int:
     ctx.reassemble_reset()
     del ra_fs, ra_fl, ra_rf
     _log("device pipeline")
-    pipeline = device_pipeline(w, dw0) if not a.ref64 else None
+    pipeline = device_pipeline(pool) if not a.ref64 else None
 
     # how the dominant kernel and the whole step scale with the batches laid side by side in one call
     by_bpl = {}
@@ -604,13 +827,20 @@ def main() -> int:
             torch.cuda.empty_cache()
 
     _log("single-batch call")
-    # the single-batch call of the same workload, for the record
+    # the single-batch call of the same workload -- the call BASELINE's config words literally
     single = None
     if bpl != 1 and not a.no_single:
         p1 = Pool(w, 1, a.rotate_mb, extra, rule=rule)
+        b1 = p1.gather_bytes + p1.scatter_bytes
+
+        def fig(sec_per_step):
+            return {"us_per_step": round(sec_per_step * 1e6, 3), "GBps": round(b1 / sec_per_step / 1e9, 1),
+                    "frac_of_hbm_peak": round(b1 / sec_per_step / 1e9 / HBM_PEAK_GBS, 4),
+                    "requests_per_sec": round(p1.n_req / sec_per_step, 1)}
+
+        # two calls per step, a context (stream) per direction
         s1 = timed(ctx, p1, a.steps, a.warmup, ctx_tx)
         k1 = kernel_times(ctx, p1, min(a.steps, 100))
-        b1 = p1.gather_bytes + p1.scatter_bytes
         single = {"ms_per_step": round(s1 * 1e3, 5), "GBps": round(b1 / s1 / 1e9, 2),
                   "requests_per_sec": round(p1.n_req / s1, 1),
                   "kernel_us": {k: round(v[0] * 1e3, 3) for k, v in k1.items()},
@@ -621,6 +851,24 @@ def main() -> int:
             single["native_loop_ms_per_step"] = round(nl * 1e3, 5)
             single["native_loop_GBps"] = round(b1 / nl / 1e9, 1)
             single["native_loop_requests_per_sec"] = round(p1.n_req / nl, 1)
+        if not w.tx_in_place:
+            # one call and ONE launch per step (sg_hip_shunt_batch: the scatter's frames ride in the gather's grid)
+            ks = kernel_times(ctx, p1, min(a.steps, 100), shunt=True)
+            one = {"python_loop_one_stream": fig(timed(ctx, p1, a.steps, a.warmup, None, shunt=True)),
+                   "kernel_us": round(ks["k_gather"][0] * 1e3, 3),
+                   "kernel_frac_of_hbm_peak": round(b1 / (ks["k_gather"][0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+                   if ks["k_gather"][0] > 0 else None}
+            more = [SgContext(0, max_reqs=4096, max_frames=65536) for _ in range(3)]
+            n_native = max(a.steps, 400)
+            for n_ctx in (1, 2, 4):
+                one[f"native_loop_{n_ctx}_stream{'s' if n_ctx > 1 else ''}"] = fig(
+                    native_shunt_loop(([ctx] + more)[:n_ctx], p1, n_native))
+            dt, lat = native_shunt_loop([ctx], p1, 1000, latency=True)
+            one["synchronous_call"] = {"us_per_call": round(dt * 1e6, 2),
+                                       "latency_ns_[N,Mean,p90,p95,p99,min,max]": stat_line(lat)}
+            for c in more:
+                c.close()
+            single["one_launch_per_step"] = one
         del p1
         for n_streams in (1, 2, 4):
             sg = graph_step_time(w, extra, rule, a.rotate_mb, streams=n_streams)
@@ -628,7 +876,18 @@ def main() -> int:
             single[key + "_ms_per_step"] = round(sg * 1e3, 5)
             single[key + "_GBps"] = round(b1 / sg / 1e9, 1)
             single[key + "_requests_per_sec"] = round(w.n_req / sg, 1)
+            if not w.tx_in_place:
+                sg = graph_step_time(w, extra, rule, a.rotate_mb, streams=n_streams, shunt=True)
+                single["one_launch_per_step"][key] = {
+                    "us_per_step": round(sg * 1e6, 3), "GBps": round(b1 / sg / 1e9, 1),
+                    "frac_of_hbm_peak": round(b1 / sg / 1e9 / HBM_PEAK_GBS, 4),
+                    "requests_per_sec": round(w.n_req / sg, 1)}
             torch.cuda.empty_cache()
+
+    host_engine = None
+    if not a.no_single:
+        _log("C++ engine, batched calls over P2pRpcRr objects")
+        host_engine = host_engine_batched(pool, max(50, min(a.steps, 200)))
 
     _log("per-request calls")
     per_req = per_request_calls(ctx, pool.items[0]) if not w.in_tensor_sizes else None
@@ -670,9 +929,16 @@ def main() -> int:
         # the headline workload again with the reference's own 64-byte header
         wr = synth.make_workload(a.workload, profile=synth.HDR_REF64)
         pr = Pool(wr, bpl, a.rotate_mb, extra, rule=rule)
-        sr = timed(ctx, pr, max(20, a.steps // 4), max(5, a.warmup // 4), ctx_tx, reps=3)
+        sr = timed(ctx, pr, a.steps, a.warmup, ctx_tx)
+        kr = kernel_times(ctx, pr, 50)
+        roofs = roofline_of(pr, kr, False)
+        for name in roofs:
+            roofs[name]["traffic"] = MEASURED_TRAFFIC_REF64.get((a.workload, bpl, name)) if traffic_known else None
         sweep[wr.name + "_ref64_headers"] = {"batches_per_launch": bpl, "ms_per_step": round(sr * 1e3, 5),
-                                             "GBps": round((pr.gather_bytes + pr.scatter_bytes) / sr / 1e9, 2)}
+                                             "GBps": round((pr.gather_bytes + pr.scatter_bytes) / sr / 1e9, 2),
+                                             "frac_of_hbm_peak": round((pr.gather_bytes + pr.scatter_bytes) / sr / 1e9
+                                                                       / HBM_PEAK_GBS, 4),
+                                             "kernels": roofs}
         del pr
 
     out = {
@@ -683,6 +949,9 @@ def main() -> int:
         "steps": a.steps,
         "warmup": a.warmup,
         "ms_per_step": round(sec * 1e3, 5),
+        "ms_per_step_host_clock": round(sec.host_clock * 1e3, 5),
+        "timed_runs": sec.runs,
+        "timed_ms": round(sec.timed_ms, 2),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -699,7 +968,10 @@ def main() -> int:
                    "both calls of a step on one context (the echo reads what its gather wrote), consecutive "
                    "steps on two contexts and streams in turns" if w.tx_in_place else
                    "gather and scatter calls on a stream each (a copy context per direction)",
-                   "timing": f"median of 5 runs of {a.steps} steps", "flags": w.flags,
+                   "timing": f"median of {sec.runs} runs of {a.steps} steps each ({sec.timed_ms:.0f} ms timed), every run "
+                             "between synchronization on both sides; a run is clocked by events on the streams "
+                             "(ms_per_step, value) and by the host clock around the run and its drain "
+                             "(ms_per_step_host_clock)", "flags": w.flags,
                    "tx_slots": "ring order" if a.tx_in_order else "random permutation of the TX ring"},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "requests_per_sec": rps,
@@ -718,6 +990,7 @@ def main() -> int:
         "roofline_by_batches_per_launch": by_bpl,
         "single_batch_call": single,
         "per_request_call": per_req,
+        "host_engine_batched": host_engine,
         "device_reassembly": reassembly,
         "device_pipeline": pipeline,
         "other_workloads": sweep,

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SG_HIP_ABI_VERSION 2
+#define SG_HIP_ABI_VERSION 3
 
 /* Error codes. */
 #define SG_OK 0
@@ -73,10 +73,13 @@ extern "C" {
                                           same slots (tx_slot == its frag_slot), same lengths, same
                                           requests in the same arena (an echo, answered in place or not):
                                           its descriptors and arena offsets are used as they stand and no
-                                          descriptor pass runs.  Held against that pass's counts; a call
-                                          that does not match is refused with SG_E_DATA.  resp_size is
-                                          not read; the response cursor ends up where the request cursor
-                                          did */
+                                          descriptor pass runs.  Held against what that pass recorded: its
+                                          counts, its arena (base and capacity) and the slot size its
+                                          lengths were checked against -- a call with other counts, another
+                                          arena or a TX ring of smaller slots moves nothing -- and every
+                                          frame against this call's TX ring and mtu; either way the call
+                                          reports SG_E_DATA.  resp_size is not read; the response cursor
+                                          ends up where the request cursor did */
 #define SG_F_ASYNC (1u << 16)          /* enqueue only; completion through sg_hip_sync() */
 #define SG_F_NO_XCD_REMAP (1u << 17)   /* launch-order = item order (for experiments) */
 #define SG_F_NO_SMALL (1u << 18)       /* one wavefront per frame even for short frames (for experiments) */
@@ -194,8 +197,10 @@ typedef struct sg_gather_args {
    * index, which lives on the device (sg_hip_set_slot_index).  A slot found in
    * another state is still overwritten and the call reports SG_E_DATA: the
    * caller keeps at most n_slot_states requests between gather and scatter, as
-   * the reference's flow control does (:117).  The words may live in device
-   * memory or in pinned host memory the worker's loop polls.  NULL: no ring. */
+   * the reference's flow control does (:117).  A call that refuses any part of
+   * its input (SG_E_DATA) publishes no states and leaves the index where it
+   * was.  The words may live in device memory or in pinned host memory the
+   * worker's loop polls.  NULL: no ring. */
   uint32_t *slot_state; /* device-addressable, n_slot_states words, or NULL */
   uint32_t n_slot_states;
   uint32_t reserved2;
@@ -349,6 +354,12 @@ int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_te
  * recorded into a HIP graph -- any number of them, replayed from any stream --
  * therefore continue the ring on every replay.  Calls on one context must
  * not overlap in time (one stream, or streams ordered by events).
+ * What a self-advancing launch knows itself by is its queue's address, its
+ * dispatch id there and the context's own count of such calls; sg_hip_create
+ * launches two probes and keeps to the kernel behind the call for good if the
+ * runtime does not hand out distinct pairs.  A caller that brings its own
+ * stream and destroys and re-creates it between calls needs nothing further:
+ * the count goes on where the new queue's dispatch ids start over.
  *
  * The cursor after a refusal.  A call the host refuses (SG_E_INVAL) launches
  * nothing and leaves the cursor alone.  With a descriptor pass (no
@@ -361,6 +372,70 @@ int sg_hip_set_hdrs(sg_hip_ctx *ctx, const sg_hbufs *hdrs, const uint8_t *hdr_te
  * descriptor-pass calls queued behind a refused one move nothing either. */
 int sg_hip_gather_batch(sg_hip_ctx *ctx, const sg_gather_args *args);
 int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
+
+/* One pass of the shunter's loop in one call: the gather of the requests that
+ * became ready and the scatter of the responses that are done, which the
+ * reference issues one after the other on every turn of shunter_loop
+ * (src/splitrpc_server/p2p_rpc_dpdk_server.cc:117-150 and :158-189).  The
+ * result is that of sg_hip_gather_batch(ctx, gather) followed by
+ * sg_hip_scatter_batch(ctx, scatter).  Where both halves are single-kernel
+ * calls of one wavefront per fragment that advance their cursors themselves
+ * (SG_F_RULE_FRAGS gather and a scatter of one response size, fragments and
+ * frames of at most 2016 bytes, no slot ring, no short-frame kernels of their
+ * own) and neither touches the other's memory (the TX ring apart from the RX
+ * ring, the response buffers apart from the request buffers), both travel in
+ * ONE launch: a call of a batch or two costs more in launches than in bytes,
+ * and this halves them.  Any other pair of calls is made as two calls, gather
+ * first.  Synchronous unless both argument blocks carry SG_F_ASYNC. */
+int sg_hip_shunt_batch(sg_hip_ctx *ctx, const sg_gather_args *gather, const sg_scatter_args *scatter);
+
+/* Fragment tables the device reads where the receive thread writes them.
+ * The reference's receive thread files every fragment in its request's table
+ * as it arrives (P2pRpcRr::rr_emplace_mbuf, src/p2p_rpc_rr_ng.h:96-105) and the
+ * shunter later walks those tables fragment by fragment on the host
+ * (gather_skbs, src/p2p_rpc_sg_engine.h:19-45).  With one sg_frag_table per
+ * request in memory the device can read (pinned host memory), written at the
+ * same place in the same order, a batched call needs no per-fragment work on
+ * the host: it names one table per request, and sg_hip_pack_tables pulls the
+ * tables into the CSR arrays sg_hip_gather_batch / sg_hip_scatter_batch take.
+ *   off[i]  (payload address of fragment i - pkt_base) / 2, pkt_base being any
+ *           even address at or below the packet memory (8 GiB are in reach);
+ *           0xffffffff: no such fragment
+ *   len[i]  payload bytes of fragment i
+ * An entry that is not the payload start of a slot of `ring` comes out as slot
+ * 0xffffffff, which the batched calls refuse with SG_E_DATA. */
+typedef struct sg_frag_table {
+  uint32_t off[SG_MAX_BI_SIZE];
+  uint32_t len[SG_MAX_BI_SIZE];
+} sg_frag_table; /* 8 KiB */
+
+typedef struct sg_pack_args {
+  const sg_frag_table *tables; /* device-addressable, n_tables, 16-byte aligned */
+  uint32_t n_tables;
+  uint32_t n_req;
+  const uint32_t *table_idx;   /* device-addressable, n_req: the table of each request */
+  const uint32_t *req_first;   /* device-addressable, n_req + 1: running sum of the requests' fragment counts */
+  uint32_t n_frags;            /* == req_first[n_req] */
+  uint32_t reserved;
+  uint64_t pkt_base;
+  sg_ring_desc ring;           /* the ring the fragments lie in (its header profile gives the payload offset) */
+  uint32_t *frag_slot;         /* device out, n_frags */
+  uint32_t *frag_len;          /* device out, n_frags, or NULL */
+  uint32_t *req_first_out;     /* device out, n_req + 1, or NULL */
+  /* words copied along by the same launch (what else the call behind needs on the device:
+   * tokens, response sizes, header templates), or NULL / 0 */
+  const uint32_t *blob_src;    /* device-addressable */
+  uint32_t *blob_dst;          /* device */
+  uint32_t blob_words;
+  uint32_t reserved2;
+  void *stream;                /* hipStream_t to launch on; NULL: the context's.  On a stream of its own the
+                                  pull of the next call's tables runs beside the current call's copy (the
+                                  caller orders the two streams with an event) */
+} sg_pack_args;
+
+/* Launches only; nothing is waited for.  n_req == 0 with blob_words != 0 brings the words along
+ * and nothing else.  No counterpart call in the reference. */
+int sg_hip_pack_tables(sg_hip_ctx *ctx, const sg_pack_args *args);
 
 /* The gather call for callers that cannot allocate.  No counterpart in the
  * reference: it is for code running under HIP graph capture, tight serving

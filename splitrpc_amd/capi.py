@@ -35,7 +35,7 @@ F_FORCE_SMALL = 1 << 19
 F_SELF_ADVANCE = 1 << 20
 F_TAIL_KERNEL = 1 << 21
 
-ABI_VERSION = 2  # SG_HIP_ABI_VERSION of include/sg_hip.h these mirrors were written against
+ABI_VERSION = 3  # SG_HIP_ABI_VERSION of include/sg_hip.h these mirrors were written against
 MAX_BI_SIZE = 1024
 MAX_TENSORS = 4
 
@@ -45,7 +45,7 @@ SYMBOLS = [
     "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_set_hdrs", "sg_hip_gather_batch",
     "sg_hip_scatter_batch", "sg_hip_reassemble", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
     "sg_hip_kernel_time", "sg_hip_gather_batch_static", "sg_hip_reassemble_reset", "sg_hip_reassemble_evict",
-    "sg_hip_set_slot_index", "sg_hip_get_slot_index",
+    "sg_hip_set_slot_index", "sg_hip_get_slot_index", "sg_hip_shunt_batch", "sg_hip_pack_tables",
 ]
 
 SLOT_FREE, SLOT_RX_COMPLETE, SLOT_WORK_COMPLETE, SLOT_TX_COMPLETE = 0, 1, 2, 3
@@ -99,6 +99,18 @@ class ScatterArgs(C.Structure):
                 ("n_slot_states", C.c_uint32), ("reserved2", C.c_uint32)]
 
 
+class FragTable(C.Structure):
+    _fields_ = [("off", C.c_uint32 * MAX_BI_SIZE), ("len", C.c_uint32 * MAX_BI_SIZE)]
+
+
+class PackArgs(C.Structure):
+    _fields_ = [("tables", C.c_void_p), ("n_tables", C.c_uint32), ("n_req", C.c_uint32), ("table_idx", C.c_void_p),
+                ("req_first", C.c_void_p), ("n_frags", C.c_uint32), ("reserved", C.c_uint32),
+                ("pkt_base", C.c_uint64), ("ring", RingDesc), ("frag_slot", C.c_void_p), ("frag_len", C.c_void_p),
+                ("req_first_out", C.c_void_p), ("blob_src", C.c_void_p), ("blob_dst", C.c_void_p),
+                ("blob_words", C.c_uint32), ("reserved2", C.c_uint32), ("stream", C.c_void_p)]
+
+
 class ReassembleArgs(C.Structure):
     _fields_ = [("ring", RingDesc), ("arrivals", C.c_void_p), ("len_nic", C.c_void_p),
                 ("n_arrivals", C.c_uint32), ("flags", C.c_uint32), ("req_size", C.c_uint64),
@@ -144,6 +156,8 @@ def load() -> C.CDLL:
                                     C.c_uint32, C.c_uint32]
     lib.sg_hip_gather_batch.argtypes = [P, C.POINTER(GatherArgs)]
     lib.sg_hip_scatter_batch.argtypes = [P, C.POINTER(ScatterArgs)]
+    lib.sg_hip_shunt_batch.argtypes = [P, C.POINTER(GatherArgs), C.POINTER(ScatterArgs)]
+    lib.sg_hip_pack_tables.argtypes = [P, C.POINTER(PackArgs)]
     lib.sg_hip_gather_batch_static.argtypes = [C.c_int, P, C.POINTER(GatherArgs), P, P]
     lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32 * 4)]
     lib.sg_hip_reassemble_reset.argtypes = [P]

@@ -140,9 +140,14 @@ __device__ __forceinline__ void cursor_put(uint64_t *p, bool cells, uint64_t v)
 // dispatch packet there, both handed to every wavefront in scalar registers.  (The dispatch id
 // has no builtin of its own: the declaration names the compiler's intrinsic.)
 extern "C" __device__ unsigned long long sg_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
-__device__ __forceinline__ uint64_t launch_queue()
+// `seq`: the calling context's count of calls, folded into the 16 bits a queue address leaves
+// unused.  A queue that is destroyed and created again at the same address starts its dispatch
+// ids over; the context's count goes on, so the launch that gets an old id back still does not
+// take the last call's stamp for its own.  (Replays of one graph carry one count and differ by
+// their dispatch ids.)
+__device__ __forceinline__ uint64_t launch_queue(uint32_t seq)
 {
-  return (uint64_t)(uintptr_t)__builtin_amdgcn_queue_ptr();
+  return (uint64_t)(uintptr_t)__builtin_amdgcn_queue_ptr() ^ ((uint64_t)seq << 48);
 }
 __device__ __forceinline__ uint64_t launch_stamp()
 {
@@ -151,7 +156,7 @@ __device__ __forceinline__ uint64_t launch_stamp()
 
 // The live value as a wavefront of a self-advancing kernel sees it (wave-uniform, through the
 // scalar cache).  *live: the cell it came from, *stamp: that cell's stamp.
-__device__ __forceinline__ uint64_t cursor_take(const uint64_t *p, uint32_t *live, uint64_t *stamp)
+__device__ __forceinline__ uint64_t cursor_take(const uint64_t *p, uint32_t seq, uint32_t *live, uint64_t *stamp)
 {
   // a cell is one 8-dword scalar load
   const u32x8 c0 = sload_here(reinterpret_cast<const u32x8 *>(p)), c1 = sload_here(reinterpret_cast<const u32x8 *>(p + kCurCell));
@@ -159,7 +164,7 @@ __device__ __forceinline__ uint64_t cursor_take(const uint64_t *p, uint32_t *liv
   const uint64_t v1 = (uint64_t)c1[1] << 32 | c1[0], q1 = (uint64_t)c1[3] << 32 | c1[2], s1 = (uint64_t)c1[5] << 32 | c1[4];
   // this launch's own write, once visible, is the newer cell: one comparison decides
   const uint32_t n = cursor_newer(s0, s1);
-  const bool own = (n ? q1 : q0) == launch_queue() && ((n ? s1 : s0) & ~3ull) == launch_stamp();
+  const bool own = (n ? q1 : q0) == launch_queue(seq) && ((n ? s1 : s0) & ~3ull) == launch_stamp();
   const uint32_t l = own ? n ^ 1u : n;
   *live = l;
   *stamp = l ? s1 : s0;
@@ -168,12 +173,12 @@ __device__ __forceinline__ uint64_t cursor_take(const uint64_t *p, uint32_t *liv
 
 // The successor, by ONE thread of the launch.  (Vector stores: nothing is ever
 // written through the scalar cache.)
-__device__ __forceinline__ void cursor_advance(uint64_t *p, uint32_t live, uint64_t live_stamp, uint64_t value)
+__device__ __forceinline__ void cursor_advance(uint64_t *p, uint32_t seq, uint32_t live, uint64_t live_stamp, uint64_t value)
 {
   uint64_t *cell = p + (live ^ 1u) * kCurCell;
   p[kCurPlain] = value;  // no wavefront of a self-advancing kernel reads the plain word
   cell[kCurValue] = value;
-  cell[kCurQueue] = launch_queue();
+  cell[kCurQueue] = launch_queue(seq);
   __threadfence();
   __hip_atomic_store(cell + kCurStamp, launch_stamp() | ((live_stamp + 1u) & 3ull), __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);

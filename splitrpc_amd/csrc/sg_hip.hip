@@ -38,6 +38,7 @@ using namespace sg;
 #include "sg_kernels_prep.h"
 #include "sg_kernels_copy.h"
 #include "sg_kernels_reassemble.h"
+#include "sg_kernels_pack.h"
 
 // ---------------------------------------------------------------------------
 // scratch of the allocation-free entry point
@@ -51,8 +52,9 @@ constexpr size_t kStaticReq = sizeof(uint64_t) * (size_t)SG_STATIC_MAX_REQS;
 constexpr size_t kStaticTile = sizeof(uint64_t) * (SG_STATIC_MAX_REQS / kPartMin + 2);
 constexpr size_t kStaticWords = 256;  // cursors, staged cursors, status, refusal flag
 // 64-bit words a context keeps beside its scratch: two cursors of kCurWords each, their staged
-// successors, the two slot indices (one word), the descriptor tag (two words)
+// successors, the two slot indices (one word), the descriptor tag (four words)
 constexpr size_t kCtxWords = 2 * kCurWords + 8;
+static_assert(2 + 1 + kTagWords / 2 <= 8, "the words behind the cursors");
 constexpr size_t kStaticBytes = kStaticDesc + 2 * kStaticReq + kStaticTile + kStaticWords;
 }  // namespace
 static __device__ __align__(256) uint8_t scratch[kStaticBytes];
@@ -83,8 +85,10 @@ struct Scratch {
   // plain words (the allocation-free entry point, whose caller may bring the word)
   bool cursor_cells = false;
   uint32_t *slot_idx[2] = {nullptr, nullptr};  // next slot of the application ring to fill / to serve
-  uint32_t *desc_tag = nullptr;    // {generation, requests, items} of the descriptors in `desc`
+  uint32_t *desc_tag = nullptr;    // kTag* words: what the descriptors in `desc` were made of and held against
   uint32_t *desc_gen = nullptr;    // host counter behind the generation (one per scratch)
+  uint32_t *call_seq = nullptr;    // host count of self-advancing launches (a context's; part of their stamps)
+  bool stamps_ok = false;          // launches on this device tell themselves apart by queue and dispatch id
   uint32_t *csum_part = nullptr;   // kPartStride words per frame (two-phase UDP checksum of long frames)
   uint32_t *csum_valid = nullptr;  // one mark per frame, zero between calls
   uint32_t *status = nullptr;
@@ -106,6 +110,7 @@ struct sg_hip_ctx {
   uint64_t *cursors = nullptr;
   uint32_t *csum_scratch = nullptr;  // csum_part and csum_valid
   uint32_t desc_gen = 0;
+  uint32_t call_seq = 0;
   uint32_t *status = nullptr;
   Scratch sc;
   // pinned staging for the per-request entry points (device reads it in place)
@@ -267,7 +272,7 @@ const uint64_t *plain_cursor(const Scratch &sc, int which)
 constexpr uint64_t kSelfAdvanceMaxWaves = 65536;
 bool self_advancing(const Scratch &sc, bool packed, const void *slot_state, uint64_t waves, uint32_t flags)
 {
-  if (flags & SG_F_TAIL_KERNEL) return false;
+  if ((flags & SG_F_TAIL_KERNEL) || !sc.stamps_ok) return false;
   return packed && sc.cursor_cells && !slot_state && (waves <= kSelfAdvanceMaxWaves || (flags & SG_F_SELF_ADVANCE));
 }
 
@@ -487,6 +492,24 @@ static void launch_gather_rule(hipStream_t st, const GatherRuleArgs &ga, uint32_
   }
 }
 
+// One direction's share of a launch that carries both (sg_hip_shunt_batch).
+struct ShuntHalf {
+  GatherRuleArgs g;
+  ScatterArgs s;
+  uint32_t g_grid = 0, s_grid = 0;
+  bool full_csum = false;
+};
+constexpr int kNoShare = 1;  // the call needs kernels of its own
+
+// What a self-advancing launch tells itself from every other launch by, as one wavefront sees it.
+__global__ void k_stamp_probe(uint64_t *out)
+{
+  if (threadIdx.x == 0) {
+    out[0] = launch_queue(0);
+    out[1] = launch_stamp();
+  }
+}
+
 extern "C" {
 
 int sg_hip_abi_version(void) { return SG_HIP_ABI_VERSION; }
@@ -538,6 +561,18 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   c->h_status[0] = c->h_status[1] = 0;
   c->h_flag = c->h_status + 1;
   HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
+  // The self-advancing cursor rests on every launch seeing a queue address and a dispatch id of
+  // its own.  Two probe launches show whether this runtime hands them out: if their pairs agree,
+  // or come back empty, calls on this context keep to the kernel behind the call.
+  {
+    volatile uint64_t *probe = c->h_ptrs;
+    probe[0] = probe[1] = probe[2] = probe[3] = 0;
+    k_stamp_probe<<<1, kWave, 0, c->stream>>>(c->h_ptrs);
+    k_stamp_probe<<<1, kWave, 0, c->stream>>>(c->h_ptrs + 2);
+    HIP_TRY(nullptr, hipGetLastError());
+    HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
+    c->sc.stamps_ok = probe[0] != 0 && probe[2] != 0 && !(probe[0] == probe[2] && probe[1] == probe[3]);
+  }
   Scratch &sc = c->sc;
   sc.max_reqs = c->max_reqs;
   sc.max_frames = c->max_frames;
@@ -554,6 +589,7 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   sc.slot_idx[1] = sc.slot_idx[0] + 1;
   sc.desc_tag = reinterpret_cast<uint32_t *>(c->cursors + 2 * kCurWords + 3);
   sc.desc_gen = &c->desc_gen;
+  sc.call_seq = &c->call_seq;
   sc.csum_part = c->csum_scratch;
   sc.csum_valid = c->csum_scratch + (size_t)c->max_frames * kPartStride;
   sc.status = c->status;
@@ -788,11 +824,16 @@ int sg_hip_set_hdrs(sg_hip_ctx *c, const sg_hbufs *hdrs, const uint8_t *hdr_temp
 
 // The gather call proper.  `c` may be null (allocation-free entry point): then
 // errors go to the creation-error text, nothing is profiled and nothing waits.
-static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const sg_gather_args *a)
+// `half` (sg_hip_shunt_batch): nothing is launched; a call that can share a launch with the other
+// direction leaves its kernel arguments there and returns SG_OK, any other returns kNoShare.
+// `zero_words` (allocation-free entry point): two status words to clear ahead of the first kernel,
+// once the host has found nothing to refuse.
+static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const sg_gather_args *a,
+                       ShuntHalf *half = nullptr, uint32_t *zero_words = nullptr)
 {
   int rc = check_ring(c, a->ring, "rx");
   if (rc != SG_OK) return rc;
-  if (a->n_req == 0) return SG_OK;
+  if (a->n_req == 0) return half ? kNoShare : SG_OK;
   if (a->n_req > sc.max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u", a->n_req, sc.max_reqs);
   if (a->n_frags > sc.max_frames) return fail(c, SG_E_INVAL, "n_frags %u > max_frames %u", a->n_frags, sc.max_frames);
   if ((!a->frag_slot && a->n_frags) || !a->req_first) return fail(c, SG_E_INVAL, "null fragment tables");
@@ -877,6 +918,16 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     ga.opts = (remap ? kOptRemap : 0u) | (app.mirrored ? kOptMirrored : 0u) |
               (app.n_tensors > 1 ? kOptMultiTensor : 0u) | (small_last ? kOptSmallLast : 0u) |
               ((((uintptr_t)a->ring.base | a->ring.slot_size) & 15u) ? 0u : kOptHdrChunk);
+    if (half) {
+      // one wavefront per fragment, the cursor advanced by the kernel itself: the shape k_shunt carries
+      if (!self_advance || small_all || small_last || ga.pieces != 1) return kNoShare;
+      ga.call_seq = ++*sc.call_seq;
+      half->g = ga;
+      half->g_grid = grid;
+      return SG_OK;
+    }
+    if (self_advance) ga.call_seq = ++*sc.call_seq;
+    if (zero_words) k_zero_words<<<1, kBlock, 0, st>>>(zero_words, 2);
     rc = prof_begin(c, 1);
     if (rc != SG_OK) return rc;
     if (self_advance) launch_gather_rule<true>(st, ga, grid, small_all, small_last, n_items);
@@ -888,10 +939,12 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
     return finish(c, a->flags);
   }
 
+  if (half) return kNoShare;  // a descriptor pass: kernels of its own
   PrepArgs p;
   memset(&p, 0, sizeof p);
   p.mode = 0;
   p.n_req = a->n_req;
+  p.arena_base = (uint64_t)(uintptr_t)app.arena;
   p.ring = static_cast<const uint8_t *>(a->ring.base);
   p.n_slots = a->ring.n_slots;
   p.slot_size = a->ring.slot_size;
@@ -918,6 +971,7 @@ static int gather_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const s
   }
   p.status = sc.status;
   p.status_flag = sc.flag;
+  if (zero_words) k_zero_words<<<1, kBlock, 0, st>>>(zero_words, 2);
   rc = launch_prep(c, sc, st, p);
   if (rc != SG_OK) return rc;
 
@@ -961,14 +1015,15 @@ int sg_hip_gather_batch(sg_hip_ctx *c, const sg_gather_args *a)
   return gather_impl(c, c->sc, c->stream, a);
 }
 
-static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const sg_scatter_args *a)
+static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const sg_scatter_args *a,
+                        ShuntHalf *half = nullptr)
 {
   int rc = check_ring(c, a->rx, "rx");
   if (rc != SG_OK) return rc;
   rc = check_ring(c, a->tx, "tx");
   if (rc != SG_OK) return rc;
   if (a->rx.hdr_profile != a->tx.hdr_profile) return fail(c, SG_E_INVAL, "rx and tx rings differ in header profile");
-  if (a->n_req == 0) return SG_OK;
+  if (a->n_req == 0) return half ? kNoShare : SG_OK;
   if (a->n_req > sc.max_reqs) return fail(c, SG_E_INVAL, "n_req %u > max_reqs %u", a->n_req, sc.max_reqs);
   if (a->n_frames > sc.max_frames) return fail(c, SG_E_INVAL, "n_frames %u > max_frames %u", a->n_frames, sc.max_frames);
   if (!a->resp_first || (a->n_frames && (!a->tx_slot || (!a->hdr_src_slot && !a->hdr_src_req && !a->hdr_templates))))
@@ -1049,6 +1104,19 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     // a kernel before that one has no writer beside it and reads the plain word
     const bool self_advance = self_advancing(sc, packed, a->slot_state, (uint64_t)n_items * sa.pieces, a->flags);
     sa.rule.cursor = const_cast<uint64_t *>(plain_cursor(sc, 1));
+    if (half) {
+      // one wavefront per frame in one kernel that advances the cursor itself
+      const bool own_small_launch = !small_all && small_last;
+      if (!self_advance || small_all || own_small_launch || sa.pieces != 1) return kNoShare;
+      sa.rule.call_seq = ++*sc.call_seq;
+      magic_div(sa.rule.per_launch, &sa.rule.lmul, &sa.rule.lshift);
+      geometry((uint64_t)n_items, !(a->flags & SG_F_NO_XCD_REMAP), &grid, &sa.remap);
+      half->s = sa;
+      half->s_grid = grid;
+      half->full_csum = full_csum;
+      return SG_OK;
+    }
+    if (self_advance) sa.rule.call_seq = ++*sc.call_seq;
     rc = prof_begin(c, 2);
     if (rc != SG_OK) return rc;
     if (small_all) {
@@ -1080,10 +1148,12 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
     return finish(c, a->flags);
   }
 
+  if (half) return kNoShare;  // a descriptor pass: kernels of its own
   PrepArgs p;
   memset(&p, 0, sizeof p);
   p.mode = 1;
   p.n_req = a->n_req;
+  p.arena_base = (uint64_t)(uintptr_t)app.arena;
   p.n_slots = a->tx.n_slots;
   p.slot_size = a->tx.slot_size;
   p.hl = hl;
@@ -1157,6 +1227,7 @@ static int scatter_impl(sg_hip_ctx *c, const Scratch &sc, hipStream_t st, const 
       sa.offsets_out = a->offsets_out;
     }
     sa.app = app;
+    sa.rule.mtu = a->mtu;  // reused descriptors are held against it
     sa.pieces = pieces_for(a->mtu);
     uint32_t grid;
     const bool full_csum = (a->flags & SG_F_UDP_CSUM_FULL) != 0;
@@ -1180,6 +1251,119 @@ int sg_hip_scatter_batch(sg_hip_ctx *c, const sg_scatter_args *a)
   if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
   DeviceGuard g(c->device);
   return scatter_impl(c, c->sc, c->stream, a);
+}
+
+// ---- both directions in one launch ---------------------------------------------
+
+static bool ranges_overlap(const void *a, uint64_t an, const void *b, uint64_t bn)
+{
+  const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+  return a0 < b0 + bn && b0 < a0 + an;
+}
+
+int sg_hip_shunt_batch(sg_hip_ctx *c, const sg_gather_args *g, const sg_scatter_args *s)
+{
+  if (!c || !g || !s) return fail(c, SG_E_INVAL, "null argument");
+  DeviceGuard guard(c->device);
+  const uint32_t async = g->flags & s->flags & SG_F_ASYNC;
+  // what the scatter writes (TX slots) and reads (responses) against what the gather reads (RX
+  // slots) and writes (requests): halves that touch each other's memory run one after the other
+  bool apart = !ranges_overlap(s->tx.base, (uint64_t)s->tx.n_slots * s->tx.slot_size, g->ring.base,
+                               (uint64_t)g->ring.n_slots * g->ring.slot_size);
+  if (g->app.n_tensors == 0 && s->app.n_tensors == 0)
+    apart = apart && !ranges_overlap(s->app.arena, s->app.arena_cap, g->app.arena, g->app.arena_cap);
+  else if (g->app.n_tensors == 0 || s->app.n_tensors == 0)
+    apart = false;  // an arena against tensors: not looked into
+  else
+    for (uint32_t i = 0; i < g->app.n_tensors; i++)
+      for (uint32_t j = 0; j < s->app.n_tensors; j++)
+        apart = apart && g->app.tensor_base[i] != s->app.tensor_base[j];
+  // Both halves are looked at before either is launched: a call the host refuses launches nothing.
+  // A half that cannot share a launch leaves no trace; both are then made as calls of their own.
+  ShuntHalf h;
+  const uint32_t seq0 = c->call_seq;
+  const int rg = gather_impl(c, c->sc, c->stream, g, &h);
+  if (rg < 0) return rg;
+  const int rs = scatter_impl(c, c->sc, c->stream, s, &h);
+  if (rs < 0) return rs;
+  if (apart && rg == SG_OK && rs == SG_OK) {
+    ShuntArgs sh;
+    sh.g = h.g;
+    sh.s = h.s;
+    sh.s_blocks = h.s_grid;
+    int rc = prof_begin(c, 1);
+    if (rc != SG_OK) return rc;
+    if (h.full_csum) k_shunt<true><<<h.g_grid + h.s_grid, kBlock, 0, c->stream>>>(sh);
+    else k_shunt<false><<<h.g_grid + h.s_grid, kBlock, 0, c->stream>>>(sh);
+    rc = prof_end(c);
+    if (rc != SG_OK) return rc;
+    return finish(c, async);
+  }
+  c->call_seq = seq0;
+  int rc = gather_impl(c, c->sc, c->stream, g);
+  if (rc != SG_OK) return rc;
+  return scatter_impl(c, c->sc, c->stream, s);
+}
+
+// ---- fragment tables pulled from where the receive thread keeps them -----------
+
+int sg_hip_pack_tables(sg_hip_ctx *c, const sg_pack_args *a)
+{
+  if (!c || !a) return fail(c, SG_E_INVAL, "null argument");
+  if (a->blob_words && (!a->blob_src || !a->blob_dst)) return fail(c, SG_E_INVAL, "null blob");
+  if (a->n_req == 0 && a->blob_words) {
+    // no tables, only words to bring along
+    DeviceGuard g(c->device);
+    PackArgs p;
+    memset(&p, 0, sizeof p);
+    p.blob_src = a->blob_src;
+    p.blob_dst = a->blob_dst;
+    p.blob_words = a->blob_words;
+    const uint32_t blocks = (a->blob_words + 4 * kBlock - 1) / (4 * kBlock);
+    k_pack_tables<64><<<blocks > 256 ? 256u : blocks, kBlock, 0, a->stream ? static_cast<hipStream_t>(a->stream) : c->stream>>>(p);
+    HIP_TRY(c, hipGetLastError());
+    return SG_OK;
+  }
+  int rc = check_ring(c, a->ring, "packet");
+  if (rc != SG_OK) return rc;
+  if (a->n_req == 0) return SG_OK;
+  if (!a->tables || !a->table_idx || !a->req_first || (a->n_frags && !a->frag_slot)) return fail(c, SG_E_INVAL, "null tables");
+  const uint32_t hl = hdr_len_of(a->ring.hdr_profile);
+  if ((a->pkt_base & 1u) || (uint64_t)(uintptr_t)a->ring.base < a->pkt_base)
+    return fail(c, SG_E_INVAL, "pkt_base must be even and at or below the ring");
+  if ((uintptr_t)a->tables & 15u) return fail(c, SG_E_INVAL, "fragment tables must start at a 16-byte aligned address");
+  DeviceGuard g(c->device);
+  PackArgs p;
+  memset(&p, 0, sizeof p);
+  p.tables = a->tables;
+  p.table_idx = a->table_idx;
+  p.req_first = a->req_first;
+  p.n_req = a->n_req;
+  p.n_frags = a->n_frags;
+  p.n_tables = a->n_tables;
+  p.delta = (uint64_t)(uintptr_t)a->ring.base + hl - a->pkt_base;
+  p.ring_bytes = (uint64_t)a->ring.n_slots * a->ring.slot_size;
+  p.slot_size = a->ring.slot_size;
+  p.n_slots = a->ring.n_slots;
+  p.frag_slot = a->frag_slot;
+  p.frag_len = a->frag_len;
+  p.req_first_out = a->req_first_out;
+  p.blob_src = a->blob_src;
+  p.blob_dst = a->blob_dst;
+  p.blob_words = a->blob_words;
+  hipStream_t st = a->stream ? static_cast<hipStream_t>(a->stream) : c->stream;
+  // lanes per request by the average number of fragments (a lane takes four entries per step).  A
+  // wavefront per request even for the longest tables: the pull is bound by the bus, and the fewer
+  // wavefronts wait on it, the more slots are left to the copy kernel that runs beside it.
+  const uint32_t avg = a->n_frags / a->n_req;
+  const uint32_t lanes = avg <= 32 ? 16u : 64u;
+  p.req_blocks = (a->n_req + kBlock / lanes - 1) / (kBlock / lanes);
+  const uint32_t copy_blocks = a->blob_words ? (a->blob_words + 4 * kBlock - 1) / (4 * kBlock) : 0u;
+  const uint32_t grid = p.req_blocks + (copy_blocks > 64 ? 64u : copy_blocks);
+  if (lanes == 16) k_pack_tables<16><<<grid, kBlock, 0, st>>>(p);
+  else k_pack_tables<64><<<grid, kBlock, 0, st>>>(p);
+  HIP_TRY(c, hipGetLastError());
+  return SG_OK;
 }
 
 // ---- allocation-free gather ---------------------------------------------------
@@ -1239,9 +1423,9 @@ int sg_hip_gather_batch_static(int device_id, void *stream, const sg_gather_args
   sc.slot_idx[0] = w32 + 2;  // the array's own producer index, for callers that pass a slot ring
   sc.slot_idx[1] = w32 + 3;
   // descriptors, request totals, offsets and the staged cursor are written by this call's own
-  // kernels before they are read; the array's own status word would carry the last call's refusals
-  if (!status) k_zero_words<<<1, kBlock, 0, st>>>(w32, 2);
-  return gather_impl(nullptr, sc, st, a);
+  // kernels before they are read; the array's own status word would carry the last call's
+  // refusals: it is cleared ahead of the call's first kernel, once the host has nothing to refuse
+  return gather_impl(nullptr, sc, st, a, nullptr, status ? nullptr : w32);
 }
 
 // ---- reassembly ----------------------------------------------------------------

@@ -22,9 +22,9 @@ namespace {
 // which share the cache lines at their common destination boundary -- meet in
 // one L2, while all XCDs still walk the same region of memory together.
 constexpr uint32_t kXcdRun = 32;
-__device__ __forceinline__ uint32_t item_of_wave(bool remap)
+__device__ __forceinline__ uint32_t item_of_wave(bool remap, uint32_t block)
 {
-  uint32_t g = blockIdx.x;
+  uint32_t g = block;
   if (remap) {
     const uint32_t xcd = g % kXcds, k = g / kXcds;
     g = ((k / kXcdRun) * kXcds + xcd) * kXcdRun + (k % kXcdRun);
@@ -77,7 +77,10 @@ __global__ __launch_bounds__(kBlock) void k_finish(FinishArgs a)
     const uint64_t c = cursor_get(a.cursor, a.cursor_cells != 0);
     cursor_put(a.cursor, a.cursor_cells != 0, (c % a.cap + ((uint64_t)n * a.size) % a.cap) % a.cap);
   }
-  if (a.state) {
+  // A call that refused part of its input publishes no slot states and leaves the ring index: a
+  // worker that polls the words must not be handed a request with a hole in it.  (The cursor of a
+  // call without a descriptor pass has moved all the same, as documented.)
+  if (a.state && !refused) {
     const uint32_t i0 = *a.slot_idx % a.n_states;
     uint32_t bad = 0;
     for (uint32_t k = threadIdx.x; k < n; k += kBlock) {
@@ -112,6 +115,7 @@ struct RuleArgs {
   uint32_t per_launch;
   uint32_t div_mul, div_shift;  // item / per_req == (item * div_mul) >> div_shift for item < 2^27
   uint32_t lmul, lshift;        // the same for per_launch
+  uint32_t call_seq;            // ADV: the context's count of calls, part of the launch's stamp
   // The plain cursor word.  In the self-advancing kernels (ADV) it is a context's, the live value
   // is in the cells that word belongs to, and the launch writes the successor (it is the call's
   // last kernel that reads the cursor; no k_finish follows).
@@ -156,7 +160,7 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
   uint64_t c0 = app.n_tensors == 0 ? sload_here(g.cursor) : 0;
   uint64_t cur_stamp = 0;
   uint32_t cur_live = 0;
-  if (ADV && app.n_tensors == 0) c0 = cursor_take(g.cursor - kCurPlain, &cur_live, &cur_stamp);
+  if (ADV && app.n_tensors == 0) c0 = cursor_take(g.cursor - kCurPlain, g.call_seq, &cur_live, &cur_stamp);
   *off = *i * g.mtu;
   const uint64_t rem = g.size - *off;
   *len = (uint32_t)(rem <= g.mtu ? rem : g.mtu);
@@ -166,7 +170,7 @@ __device__ __forceinline__ uint32_t rule_desc(const RuleArgs &g, const AppDev &a
   if (app.n_tensors == 0) {
     if (c0 >= app.cap) c0 %= app.cap;  // only after a set_cursor beyond the capacity
     // the successor depends on the cursor, the size and the count only: it is out before a bad item is dropped
-    if (ADV && writer) cursor_advance(g.cursor - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, g.size, app.cap));
+    if (ADV && writer) cursor_advance(g.cursor - kCurPlain, g.call_seq, cur_live, cur_stamp, cursor_bump(c0, n_req, g.size, app.cap));
     uint64_t o = c0 + (uint64_t)*r * g.size;
     if (g.single_wrap) o = o >= app.cap ? o - app.cap : o;  // n_req * size <= capacity
     else o %= app.cap;
@@ -321,7 +325,7 @@ __global__ __launch_bounds__(kBlock) void k_gather(GatherArgs a)
   SG_PIN(desc); SG_PIN(req_off); SG_PIN(ring); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_items);
   SG_PIN(remap); SG_PIN(status); SG_PIN(pieces); SG_PIN(counts);
   if (counts) n_items = dev_count(counts, 1, n_items);
-  const uint32_t w = item_of_wave(remap != 0);
+  const uint32_t w = item_of_wave(remap != 0, blockIdx.x);
   const uint32_t item = LONG ? w / pieces : w;
   const uint32_t piece = LONG ? w - item * pieces : 0;
   const uint32_t lane = threadIdx.x & (kWave - 1);
@@ -402,7 +406,7 @@ struct alignas(64) GatherRuleArgs {
   // wavefront reads one entry instead of walking them itself.  n_plan == 0: no plan (too many
   // fragments per request, or tensors of 4 GiB and more per request).
   uint32_t n_plan;
-  uint32_t plan_pad;
+  uint32_t call_seq;  // ADV: the context's count of calls, part of the launch's stamp
   alignas(64) FragPlan plan[kPlanMax];  // an entry is one 8-dword scalar load: inside one cache line
 };
 constexpr uint32_t kOptRemap = 1u, kOptMirrored = 2u, kOptMultiTensor = 8u;
@@ -412,18 +416,21 @@ constexpr uint32_t kOptHdrChunk = 16u;
 constexpr uint32_t kOptSmallLast = 32u;  // the last fragment of every request is left to k_gather_small
 
 template <int L, bool ADV>
-__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave, bool may_advance);
+__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave, bool may_advance, size_t kernarg_base = 0);
 
 // SMALL: lanes per remainder fragment (16 or 32) when the last fragment of every
 // request is short -- the wavefronts behind those of the full fragments then move
 // 64 / SMALL remainder fragments each, in the same launch (a launch of their own
 // would be all latency: tens of megabytes at most); 0: no such wavefronts.
 // ADV: the kernel takes the cursor from a context's cells and advances it itself (no k_finish follows).
+// `block`: the workgroup's number among those of this work; `kernarg_base`: where `a` lies in the
+// running kernel's argument block (the plan is read through the argument pointer).
 template <bool LONG, int SMALL, bool ADV>
-__global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
+__device__ __forceinline__ void gather_rule_body(const GatherRuleArgs &a, uint32_t block, size_t kernarg_base)
 {
   const uint8_t *ring = a.ring;
   const uint32_t *frag_slot = a.frag_slot;
+  const uint32_t *frag_len = a.frag_len;
   uint8_t *dst = a.dst;
   uint64_t *cursor_in = a.cursor;
   const uint64_t size = a.size, cap = a.cap;
@@ -434,14 +441,14 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   uint32_t n_items = a.n_items, n_req = a.n_req;
   SG_PIN(ring); SG_PIN(frag_slot); SG_PIN(dst); SG_PIN(cursor_in); SG_PIN(size); SG_PIN(cap);
   SG_PIN(n_items); SG_PIN(per_req); SG_PIN(mtu); SG_PIN(slot_size); SG_PIN(hl); SG_PIN(n_slots);
-  SG_PIN(pieces); SG_PIN(opts); SG_PIN(div_mul); SG_PIN(div_shift); SG_PIN(counts);
+  SG_PIN(pieces); SG_PIN(opts); SG_PIN(div_mul); SG_PIN(div_shift); SG_PIN(counts); SG_PIN(frag_len);
   if (counts) {
     // counts left on the device by the reassembly: the launch was sized for n_req requests at most
     n_req = dev_count(counts, 0, n_req);
     n_items = n_req * per_req;
   }
 
-  uint32_t w = item_of_wave((opts & kOptRemap) != 0);
+  uint32_t w = item_of_wave((opts & kOptRemap) != 0, block);
   const bool first_wave = w == 0;
   const uint32_t pl = a.per_launch;
   if (SMALL) {
@@ -452,7 +459,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     const uint32_t blk = (uint32_t)(((uint64_t)w * a.pmul) >> a.pshift);
     const uint32_t j = w - blk * a.period;
     if (j == a.period - 1) {
-      gather_small_wave<(SMALL ? SMALL : 16), ADV>(a, blk, false);  // wavefront 0 of the full fragments advances the cursor
+      gather_small_wave<(SMALL ? SMALL : 16), ADV>(a, blk, false, kernarg_base);  // wavefront 0 of the full fragments advances the cursor
       return;
     }
     w = blk * (a.period - 1) + j;
@@ -474,10 +481,14 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   }
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t slot = sload(frag_slot + item);
+  // where lengths come from a table (the reference's header carries none), the entry is asked for
+  // with the slot's: read at the end, where it is held against the rule, it would lengthen the
+  // wavefront's life by a round trip of its own
+  const uint32_t tab_len = frag_len ? sload(frag_len + item) : 0u;
   uint64_t c0 = cap ? sload(cursor_in) : 0;
   uint64_t cur_stamp = 0;
   uint32_t cur_live = 0;
-  if (ADV && cap) c0 = cursor_take(cursor_in - kCurPlain, &cur_live, &cur_stamp);
+  if (ADV && cap) c0 = cursor_take(cursor_in - kCurPlain, a.call_seq, &cur_live, &cur_stamp);
   const uint32_t off = i * mtu;
   const uint32_t rem = (uint32_t)size - off;  // sizes are below 4 GiB (checked by the host)
   const uint32_t len = rem <= mtu ? rem : mtu;
@@ -494,7 +505,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     // the successor depends on the cursor, the size and the count only: it is out before a
     // fragment with a bad slot index is dropped
     if (ADV && first_wave && lane == 0)
-      cursor_advance(cursor_in - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, size, cap));
+      cursor_advance(cursor_in - kCurPlain, a.call_seq, cur_live, cur_stamp, cursor_bump(c0, n_req, size, cap));
     ro = c0 + (uint64_t)r * size;
     ro = ro >= cap ? ro - cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
     if (lane == 0 && piece == 0 && a.offsets_out) {
@@ -513,7 +524,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   } else if (opts & kOptMultiTensor) {
     // tensor-major buffers: a fragment inside one tensor still takes the fast path
     if (a.n_plan) {
-      const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(GatherRuleArgs, plan))) + i);
+      const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(kernarg_base + offsetof(GatherRuleArgs, plan))) + i);
       plan_kind = fp[7];
       plain = plan_kind == 0;
       to = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
@@ -535,7 +546,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
   // The header words that hold the fragment's real length are fetched together
   // with the payload, so that checking them does not lengthen the wavefront's
   // life by another memory round trip.
-  const bool check_hdr = piece == 0 && a.frag_len == nullptr;
+  const bool check_hdr = piece == 0 && frag_len == nullptr;
   uint32_t hv = 0;
   u32x4 hc = {0u, 0u, 0u, 0u};
   if (check_hdr) {
@@ -579,11 +590,17 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
     uint32_t bad = 0;
     // payload_len is the u32 at byte 54: bytes 6..9 of the chunk that starts at byte 48
     const uint32_t hdr_len = (opts & kOptHdrChunk) ? ((hc[1] >> 16) | (hc[2] << 16)) : hv;
-    const bool as_ruled = (check_hdr ? hdr_len : sload(a.frag_len + item)) == len;
+    const bool as_ruled = (check_hdr ? hdr_len : tab_len) == len;
     if (!as_ruled) bad |= kStNotRule;
     if (i == 0 && sload(a.first + r) != item) bad |= kStBadTable;
     if (bad && lane == 0) refuse(a.status, a.status_flag, bad);
   }
+}
+
+template <bool LONG, int SMALL, bool ADV>
+__global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
+{
+  gather_rule_body<LONG, SMALL, ADV>(a, blockIdx.x, 0);
 }
 
 // Gather of SHORT fragments, 64 / L fragments per wavefront (L = 16 or 32 lanes
@@ -592,7 +609,7 @@ __global__ __launch_bounds__(kBlock) void k_gather_rule(GatherRuleArgs a)
 // fragment of every request (the remainder; the full fragments then go through
 // k_gather_rule).  Addressing is per lane.
 template <int L, bool ADV>
-__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave, bool may_advance)
+__device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint32_t wave, bool may_advance, size_t kernarg_base)
 {
   constexpr uint32_t G = kWave / L;
   // every argument of the common path in one burst of scalar loads
@@ -634,10 +651,10 @@ __device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint3
     uint64_t c0 = sload(a.cursor);
     uint64_t cur_stamp = 0;
     uint32_t cur_live = 0;
-    if (ADV) c0 = cursor_take(a.cursor - kCurPlain, &cur_live, &cur_stamp);
+    if (ADV) c0 = cursor_take(a.cursor - kCurPlain, a.call_seq, &cur_live, &cur_stamp);
     if (c0 >= a.cap) c0 %= a.cap;  // only after a set_cursor beyond the capacity
     if (ADV && may_advance && wave == 0 && lane == 0)
-      cursor_advance(a.cursor - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, a.size, a.cap));
+      cursor_advance(a.cursor - kCurPlain, a.call_seq, cur_live, cur_stamp, cursor_bump(c0, n_req, a.size, a.cap));
     ro = c0 + (uint64_t)r * a.size;
     ro = ro >= a.cap ? ro - a.cap : ro;  // the batch fits the arena (checked by the host): one wrap at most
     if (live && gl == 0 && a.offsets_out) {
@@ -665,7 +682,7 @@ __device__ __forceinline__ void gather_small_wave(const GatherRuleArgs &a, uint3
     } else if (a.opts & kOptMultiTensor) {
       if (last_only && a.n_plan) {
         // every group has the request's last fragment: one plan entry for the wavefront
-        const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(GatherRuleArgs, plan))) + (per_req - 1));
+        const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(kernarg_base + offsetof(GatherRuleArgs, plan))) + (per_req - 1));
         plain = fp[7] == 0;
         to = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
       } else {
@@ -746,10 +763,10 @@ struct alignas(64) ScatterArgs {
 // Where the payload of a frame comes from; false: not one contiguous piece.
 template <bool FUSED>
 __device__ __forceinline__ bool scatter_source(const ScatterArgs &a, uint64_t ro, uint32_t r, uint32_t i,
-                                               uint32_t off, uint32_t len, uint8_t **from)
+                                               uint32_t off, uint32_t len, uint8_t **from, size_t kernarg_base)
 {
   if (FUSED && a.n_plan) {
-    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(ScatterArgs, plan))) + i);
+    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(kernarg_base + offsetof(ScatterArgs, plan))) + i);
     *from = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
     return fp[7] == 0;
   }
@@ -773,8 +790,8 @@ constexpr uint32_t kPartStride = 8;  // words of csum_part per frame: up to 7 su
 // several wavefronts all the same, each leaving the sum of its bytes behind,
 // and k_udp_finish writes the checksum field afterwards.
 // ADV (fused only): the kernel takes the cursor from a context's cells and advances it itself.
-template <bool FULL_CSUM, bool FUSED, bool LONG, bool DEFER = false, bool ADV = false>
-__global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
+template <bool FULL_CSUM, bool FUSED, bool LONG, bool DEFER, bool ADV>
+__device__ __forceinline__ void scatter_body(const ScatterArgs &a, uint32_t block, size_t kernarg_base)
 {
   constexpr bool SPLIT = LONG && (!FULL_CSUM || DEFER);      // several wavefronts per frame
   constexpr bool WHOLE_LONG = LONG && FULL_CSUM && !DEFER;   // one wavefront walks all sub-runs of its frame
@@ -803,14 +820,22 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     SG_PIN(a.rule.item_slot); SG_PIN(a.rule.first); SG_PIN(a.rule.size); SG_PIN(a.rule.mtu);
     SG_PIN(a.rule.per_req); SG_PIN(a.rule.n_slots); SG_PIN(a.rule.single_wrap); SG_PIN(a.rule.cursor);
   }
-  const uint32_t w = item_of_wave(remap != 0);
+  const uint32_t w = item_of_wave(remap != 0, block);
   const uint32_t pieces = SPLIT ? n_pieces : 1u;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   // descriptor path: this kernel does not read the cursor and commits what the descriptor pass left
   if (!FUSED && a.reuse_gen && n_req) {
-    // the caller says these are the items the tagged descriptor pass described
-    if (sload(a.desc_tag) != a.reuse_gen || sload(a.desc_tag + 1) != n_req || sload(a.desc_tag + 2) != n_items) {
-      if (w == 0 && lane == 0) refuse(a.status, a.status_flag, kStBadTable);
+    // the caller says these are the items the tagged descriptor pass described: the tag holds that
+    // pass's generation and counts, the slot size its lengths were held against, and the arena its
+    // offsets lie in.  A call that departs from any of them moves nothing.
+    const u32x8 tg = sload(reinterpret_cast<const u32x8 *>(a.desc_tag));
+    uint32_t bad = 0;
+    if (tg[kTagGen] != a.reuse_gen || tg[kTagReqs] != n_req || tg[kTagItems] != n_items) bad |= kStBadTable;
+    if (tg[kTagSlotSize] > tx_slot_size) bad |= kStBadLen;  // lengths were only held against that slot size
+    const uint64_t t_base = (uint64_t)tg[kTagArena + 1] << 32 | tg[kTagArena], t_cap = (uint64_t)tg[kTagCap + 1] << 32 | tg[kTagCap];
+    if (t_base != (uint64_t)(uintptr_t)a.app.arena || t_cap != a.app.cap) bad |= kStBadSize;  // offsets of another arena
+    if (bad) {
+      if (w == 0 && lane == 0) refuse(a.status, a.status_flag, bad);
       return;
     }
   }
@@ -846,8 +871,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     nf = sload(first + r + 1) - f0;
     ro = a.app.n_tensors == 0 ? sload(req_off + r) : 0;
     if (a.reuse_gen) {
-      if (d[0] >= a.tx_n_slots) {  // described for another ring
-        if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, kStBadSlot);
+      if (d[0] >= a.tx_n_slots || d[1] > a.rule.mtu) {  // described for another ring, or cut at another mtu
+        if (lane == 0 && piece == 0) refuse(a.status, a.status_flag, d[0] >= a.tx_n_slots ? kStBadSlot : kStBadLen);
         return;
       }
       if (a.offsets_out && item == f0 && lane == 0 && piece == 0) a.offsets_out[r] = ro;
@@ -891,7 +916,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
     // a later piece of a long frame: payload only
     uint8_t *from;
     uint32_t part = 0;
-    if (d[1] && scatter_source<FUSED>(a, ro, r, item - f0, d[2], d[1], &from)) {
+    if (d[1] && scatter_source<FUSED>(a, ro, r, item - f0, d[2], d[1], &from, kernarg_base)) {
       uint32_t o, n;
       sub_run(slot + hl, d[1], piece, &o, &n);
       if (n) part = copy_run<DEFER>(from + o, slot + hl + o, n, lane);
@@ -909,7 +934,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   const uint32_t raw = hdrw_fetch(hin, lane, hl, !from_template);
   uint32_t hb = 0, acc = 0;
   uint8_t *from = nullptr;
-  const bool plain = d[1] != 0 && scatter_source<FUSED>(a, ro, r, item - f0, d[2], d[1], &from);
+  const bool plain = d[1] != 0 && scatter_source<FUSED>(a, ro, r, item - f0, d[2], d[1], &from, kernarg_base);
   RunState rs;
   uint32_t first_len = d[1];
   if (SPLIT && plain) {
@@ -941,6 +966,32 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   // the payload went past the header only, so a TX slot that is the header's own
   // source still held the request header when it was fetched above
   hdrw_store(slot, lane, hl, hb);
+}
+
+template <bool FULL_CSUM, bool FUSED, bool LONG, bool DEFER = false, bool ADV = false>
+__global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
+{
+  scatter_body<FULL_CSUM, FUSED, LONG, DEFER, ADV>(a, blockIdx.x, 0);
+}
+
+// One pass of the shunter's loop (src/splitrpc_server/p2p_rpc_dpdk_server.cc:117-189) in ONE
+// launch: the first s_blocks workgroups scatter the responses that are done (one response size),
+// the others gather the requests that became ready (declared rule), each half exactly as the
+// kernel of its own would.  For calls of a batch or two a launch costs more than the bytes it
+// moves; this halves the launches of a step.  Both halves advance their cursors themselves.
+// The scatter's wavefronts live longest (a header to fetch, rewrite and store besides the
+// payload) and are few: they are dispatched first so that they end with the others, not after.
+struct alignas(64) ShuntArgs {
+  GatherRuleArgs g;
+  ScatterArgs s;
+  uint32_t s_blocks;
+};
+
+template <bool FULL_CSUM>
+__global__ __launch_bounds__(kBlock) void k_shunt(ShuntArgs a)
+{
+  if (blockIdx.x >= a.s_blocks) gather_rule_body<false, 0, true>(a.g, blockIdx.x - a.s_blocks, offsetof(ShuntArgs, g));
+  else scatter_body<FULL_CSUM, true, false, false, true>(a.s, blockIdx.x, offsetof(ShuntArgs, s));
 }
 
 // Second phase of the full UDP checksum of long frames: one thread per frame
@@ -1039,10 +1090,10 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
     uint64_t c0 = sload(a.rule.cursor);
     uint64_t cur_stamp = 0;
     uint32_t cur_live = 0;
-    if (ADV) c0 = cursor_take(a.rule.cursor - kCurPlain, &cur_live, &cur_stamp);
+    if (ADV) c0 = cursor_take(a.rule.cursor - kCurPlain, a.rule.call_seq, &cur_live, &cur_stamp);
     if (c0 >= a.app.cap) c0 %= a.app.cap;  // only after a set_cursor beyond the capacity
     if (ADV && wave == 0 && lane == 0)
-      cursor_advance(a.rule.cursor - kCurPlain, cur_live, cur_stamp, cursor_bump(c0, n_req, a.rule.size, a.app.cap));
+      cursor_advance(a.rule.cursor - kCurPlain, a.rule.call_seq, cur_live, cur_stamp, cursor_bump(c0, n_req, a.rule.size, a.app.cap));
     uint64_t o = c0 + (uint64_t)r * a.rule.size;
     if (a.rule.single_wrap) o = o >= a.app.cap ? o - a.app.cap : o;
     else o %= a.app.cap;

@@ -36,6 +36,9 @@ struct AppDev {
   uint64_t cap;
 };
 
+// words of a descriptor tag
+constexpr uint32_t kTagGen = 0, kTagReqs = 1, kTagItems = 2, kTagSlotSize = 3, kTagArena = 4, kTagCap = 6, kTagWords = 8;
+
 struct PrepArgs {
   // mode 0 (gather): lengths from item_len[] or from the slot headers
   // mode 1 (scatter): lengths from the fragmenting rule over sizes[] / fixed_size
@@ -79,9 +82,11 @@ struct PrepArgs {
   // scan of many requests, which then needs no launch of its own to total the tiles); or nullptr
   uint64_t *part;
   // What this pass leaves for a later call that wants to reuse its descriptors
-  // (SG_F_REUSE_DESC): desc_tag = {gen, requests, items}.
+  // (SG_F_REUSE_DESC): desc_tag = {gen, requests, items, slot size the lengths were held
+  // against, arena base, arena capacity} (kTag*, eight 32-bit words).
   uint32_t *desc_tag;
   uint32_t gen;
+  uint64_t arena_base;
   uint32_t *status;
   volatile uint32_t *status_flag;  // pinned host word: non-zero once any kernel refused something
 };
@@ -206,9 +211,14 @@ __device__ __forceinline__ void prep_finish(const PrepArgs &a, uint32_t r, uint6
   if (bad) refuse(a.status, a.status_flag, bad);
   a.req_size[r] = total;
   if (r == 0 && a.desc_tag) {
-    a.desc_tag[0] = a.gen;
-    a.desc_tag[1] = a.n_req;
-    a.desc_tag[2] = a.n_items;
+    a.desc_tag[kTagGen] = a.gen;
+    a.desc_tag[kTagReqs] = a.n_req;
+    a.desc_tag[kTagItems] = a.n_items;
+    a.desc_tag[kTagSlotSize] = a.slot_size;
+    a.desc_tag[kTagArena] = (uint32_t)a.arena_base;
+    a.desc_tag[kTagArena + 1] = (uint32_t)(a.arena_base >> 32);
+    a.desc_tag[kTagCap] = (uint32_t)a.cap;
+    a.desc_tag[kTagCap + 1] = (uint32_t)(a.cap >> 32);
   }
   if (a.packed && a.fixed_offsets) {
     // bump ring with equal sizes: ret = base + off; off = (off + size) % capacity

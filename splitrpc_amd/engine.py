@@ -210,6 +210,15 @@ class SgContext:
         if rc != capi.SG_OK:
             self._check(rc)
 
+    def shunt_batch_raw(self, g: capi.GatherArgs, s: capi.ScatterArgs) -> None:
+        """One pass of the shunter's loop: gather and scatter, in one launch
+        where the two calls can share one."""
+        if not (g.flags & s.flags & capi.F_ASYNC):
+            self._after_torch()
+        rc = self.lib.sg_hip_shunt_batch(self.h, C.byref(g), C.byref(s))
+        if rc != capi.SG_OK:
+            self._check(rc)
+
     @staticmethod
     def reassemble_args(ring: RingRef, arrivals: torch.Tensor, n_arrivals: int, frag_slot: torch.Tensor,
                         frag_len: torch.Tensor, req_first: torch.Tensor, req_token: Optional[torch.Tensor] = None,
@@ -407,12 +416,14 @@ class DeviceWorkload:
             o += s
         return outs
 
-    def gather(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False,
-               fixed: bool = True, rule: bool = False) -> None:
-        """``fixed``: declare the common request size when all requests have one
-        (offsets are then multiples of it instead of a prefix scan).  ``rule``:
-        also state that fragments follow the fragmenting rule, which lets the
-        copy kernel work without a descriptor pass."""
+    def gather_call(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False,
+                    fixed: bool = True, rule: bool = False) -> capi.GatherArgs:
+        """The argument block of this workload's gather call (built once per
+        combination and kept).  ``fixed``: declare the common request size when
+        all requests have one (offsets are then multiples of it instead of a
+        prefix scan).  ``rule``: also state that fragments follow the
+        fragmenting rule, which lets the copy kernel work without a descriptor
+        pass."""
         key = ("g", use_frag_len, fixed, rule)
         a = self._args.get(key)
         if a is None:
@@ -425,16 +436,21 @@ class DeviceWorkload:
             a._base_flags = capi.F_RULE_FRAGS if (rule and fx) else 0
             self._args[key] = a
         a.flags = flags | a._base_flags
-        self._described = not (a._base_flags & capi.F_RULE_FRAGS)  # a descriptor pass ran
-        ctx.gather_batch_raw(a)
+        self._described = not (a._base_flags & capi.F_RULE_FRAGS)  # a descriptor pass runs
+        return a
 
-    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True,
-                templates: Optional[torch.Tensor] = None, tokens: Optional[torch.Tensor] = None,
-                reuse: bool = False) -> None:
-        """``templates`` (n_req x 64 uint8 on the device) takes the frame
-        headers from connection templates instead of request headers.
-        ``reuse``: an echo answered in place right after this workload's gather
-        reuses that call's descriptors where it ran a descriptor pass."""
+    def gather(self, ctx: SgContext, flags: int = 0, use_frag_len: bool = False,
+               fixed: bool = True, rule: bool = False) -> None:
+        ctx.gather_batch_raw(self.gather_call(ctx, flags, use_frag_len, fixed, rule))
+
+    def scatter_call(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True,
+                     templates: Optional[torch.Tensor] = None, tokens: Optional[torch.Tensor] = None,
+                     reuse: bool = False) -> capi.ScatterArgs:
+        """The argument block of this workload's scatter call.  ``templates``
+        (n_req x 64 uint8 on the device) takes the frame headers from
+        connection templates instead of request headers.  ``reuse``: an echo
+        answered in place right after this workload's gather reuses that call's
+        descriptors where it ran a descriptor pass."""
         if not fuse:
             flags |= capi.F_NO_FUSE
         if reuse and self.w.tx_in_place and getattr(self, "_described", False):
@@ -452,4 +468,16 @@ class DeviceWorkload:
                                  self.w.mtu, self.resp_app, self.resp_offsets, 0, templates, tokens)
             self._args[key] = a
         a.flags = self.w.flags | flags
-        ctx.scatter_batch_raw(a)
+        return a
+
+    def scatter(self, ctx: SgContext, flags: int = 0, fixed: bool = True, fuse: bool = True,
+                templates: Optional[torch.Tensor] = None, tokens: Optional[torch.Tensor] = None,
+                reuse: bool = False) -> None:
+        ctx.scatter_batch_raw(self.scatter_call(ctx, flags, fixed, fuse, templates, tokens, reuse))
+
+    def shunt(self, ctx: SgContext, flags: int = 0, rule: bool = True) -> None:
+        """Gather and scatter of this workload as one pass of the shunter's
+        loop (one launch where the two calls can share one)."""
+        g = self.gather_call(ctx, flags, rule=rule)
+        s = self.scatter_call(ctx, flags, fuse=rule)
+        ctx.shunt_batch_raw(g, s)

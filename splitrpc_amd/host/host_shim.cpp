@@ -200,7 +200,9 @@ int sgh_ring_stress(uint32_t n_threads, uint32_t per_thread, uint32_t capacity)
 // batched gather with per-request TX; 2 the batched gather and the batched TX
 // (headers from the connections' templates, written by the scatter kernel),
 // with the application slots' state words published by the device and walked
-// by the worker's batching window on the host.  The request arena
+// by the worker's batching window on the host; 3 the same with the requests'
+// fragment tables kept where the device reads them, so that the batched calls
+// walk no fragment on the host.  The request arena
 // (n_done * req_size bytes) and the TX ring are copied back for inspection.
 // Fixed-size requests (req_size) as in the reference.  Returns completed
 // requests or a negative error.
@@ -220,11 +222,22 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
   (void)hipMemcpy(d_tx, tx_ring_host, tx_bytes, hipMemcpyHostToDevice);
 
   int64_t done = 0;
+  bool tables_pulled = false;
   {
     P2pRpcRRPool pool(-1, profile);
     p2p_rpc_conn_info *srv = initialize_src_conn_info("b8:ce:f6:cc:6a:52,192.168.25.1,50051");
     pool.setup_and_init_rr_pool(srv, req_size);
     release_conn_info(srv);
+    P2pRpcSgHipEngine engine(device_id);
+    if (per_request == 3) {
+      // the requests' fragment tables where the device reads them: written below as fragments are
+      // filed, pulled by the batched calls
+      sg_frag_table *t = engine.frag_tables((uint32_t)pool.get_pool_size());
+      if (!t) return -18;
+      pool.attach_frag_tables(t, (size_t)pool.get_pool_size(), (uintptr_t)d_ring & ~(uintptr_t)1);
+      tables_pulled = true;
+      per_request = 2;
+    }
     for (uint32_t a = 0; a < n_arr; a++) {
       const uint32_t s = arrivals[a];
       uint8_t hdr[64];
@@ -242,7 +255,6 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
     const int n_app = (int)ready.size() + 3;  // the application ring wraps after a few slots
     P2pRpcAppRrPool app_pool(n_app, device_id, req_size, resp_size, want_mirror != 0);
     if (mirrored_out) *mirrored_out = app_pool.rr_mem_pool->mirrored() ? 1 : 0;
-    P2pRpcSgHipEngine engine(device_id);
     std::vector<P2pRpcAppRr *> slots;
     for (size_t k = 0; k < ready.size(); k++) slots.push_back(app_pool.get_next());
 
@@ -295,6 +307,8 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
         P2pRpcRr *r = ready[k];
         r->transport_mbufs->num_items = r->hdr_bufs->num_items = r->payload_bufs->num_items = 0;
         r->payload_size = 0;
+        // the response buffers lie in another allocation than the request's: its table counts from there now
+        if (tables_pulled) r->pkt_base = (uintptr_t)d_tx & ~(uintptr_t)1;
         size_t rem = resp_size;
         for (uint32_t i = 0; i < per; i++) {
           uint8_t *slot = d_tx + (size_t)tx_slot[(uint32_t)k * per + i] * slot_size;
@@ -437,6 +451,22 @@ int sgh_copy_ctx_gpu(int device_id, uint64_t src, uint64_t dst, uint64_t len)
   return ok;
 }
 
+// MetaAppCtx::AppRrRunNotify with the word set by ANOTHER thread `delay_us` later, against a bound
+// of `timeout_ns`.  Bit 0: the wait saw the value; bit 1: it gave up (and counted the timeout).
+int sgh_notify_wait(uint32_t delay_us, uint64_t timeout_ns)
+{
+  AppCtx c;
+  c.notify_timeout_ns = timeout_ns;
+  volatile uint32_t word = 0;
+  std::thread setter([&] {
+    std::this_thread::sleep_for(std::chrono::microseconds(delay_us));
+    word = RX_COMPLETE;
+  });
+  const bool seen = c.AppRrRunNotify(&word, RX_COMPLETE);
+  setter.join();
+  return (seen ? 1 : 0) | (c.notify_timeouts ? 2 : 0) | (c.AppRrRunReady(&word, RX_COMPLETE) ? 4 : 0);
+}
+
 // A double-mapped arena for callers outside C++ (the tests): the request
 // range of a P2pRpcAppRrMemPool.  Returns a handle, or NULL.
 void *sgh_mempool_create(int device_id, int n, uint64_t req_size, uint64_t resp_size, int want_mirror)
@@ -478,6 +508,215 @@ double sgh_step_loop_gpu(sg_hip_ctx *g, sg_hip_ctx *s, const sg_gather_args *con
   if (rc == SG_OK && s != g) rc = sg_hip_sync(s);
   if (rc != SG_OK) return (double)rc;
   return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
+
+// The C++ engine's calls as a shunter thread issues them, timed: `n_req` requests of `per_req`
+// fragments each (request r's fragment i in slot frag_slot[r * per_req + i] of the item's RX
+// ring) held as P2pRpcRr objects, and as many responses of `per_resp` frames in the item's TX
+// ring.  `items` are ring copies taken in turns (bases[4 * k + 0..3]: RX ring, TX ring, request
+// arena, response arena of item k).
+//   mode 0  batched: gather_batch(P2pRpcRr **) + scatter_batch(P2pRpcRr **) per step, the engine
+//           walking every fragment on the host
+//   mode 1  the same with the requests' fragment tables kept where the device reads them
+//   mode 2  the reference's call: one synchronous gather(rr, stub) per request, `steps` calls
+// out[0]: seconds per step (per call in mode 2) over the whole loop, the device drained at the
+// end; out[1..7] / out[8..14]: [N, mean, p90, p95, p99, min, max] of the nanoseconds the
+// calling thread spent inside each gather / scatter call.  Returns 0 or a negative error.
+int sgh_engine_loop_gpu(int device_id, int mode, uint32_t n_items, const uint64_t *bases, uint32_t n_slots,
+                        uint32_t slot_size, uint32_t profile, const uint32_t *frag_slot, const uint32_t *frag_len,
+                        uint32_t n_req, uint32_t per_req, uint64_t req_size, uint64_t req_cap, uint32_t mtu,
+                        uint32_t tx_n_slots, const uint32_t *tx_slot, uint32_t per_resp, uint64_t resp_size,
+                        uint64_t resp_cap, uint32_t flags, uint32_t steps, double *out)
+{
+  if (hipSetDevice(device_id) != hipSuccess) return -1;
+  if (!n_items || !n_req || !steps) return -2;
+  const uint32_t hl = rpc_header_len(profile);
+  const uint32_t n_rr = 2 * n_items * n_req;
+  P2pRpcSgHipEngine engine(device_id, n_req, n_req * (per_req > per_resp ? per_req : per_resp));
+  P2pRpcRRPool pool((int)n_rr + 1, profile);
+  p2p_rpc_conn_info *srv = initialize_src_conn_info("b8:ce:f6:cc:6a:52,192.168.25.1,50051");
+  pool.setup_and_init_rr_pool(srv, req_size);
+  release_conn_info(srv);
+  if (mode == 1) {
+    sg_frag_table *t = engine.frag_tables(n_rr);
+    if (!t) return -3;
+    pool.attach_frag_tables(t, n_rr, 0);
+  }
+  std::vector<std::vector<P2pRpcRr *>> rx(n_items), tx(n_items);
+  for (uint32_t k = 0; k < n_items; k++) {
+    const uintptr_t ring = (uintptr_t)bases[4 * k], txr = (uintptr_t)bases[4 * k + 1];
+    for (uint32_t r = 0; r < n_req; r++) {
+      // the receive thread's work: every fragment filed at its sequence number
+      P2pRpcRr *q = pool.consume_rr();
+      q->pkt_base = ring & ~(uintptr_t)1;
+      q->req_token = ((uint64_t)k << 32) | (r + 1);
+      for (uint32_t i = 0; i < per_req; i++) {
+        const uintptr_t slot = ring + (uintptr_t)frag_slot[r * per_req + i] * slot_size;
+        q->rr_emplace_mbuf(slot, slot, slot + hl, frag_len[r * per_req + i], (int)i);
+      }
+      rx[k].push_back(q);
+      // rr_alloc_mbufs: the response's buffers
+      P2pRpcRr *p = pool.consume_rr();
+      p->pkt_base = txr & ~(uintptr_t)1;
+      p->req_token = q->req_token;
+      size_t rem = resp_size;
+      for (uint32_t i = 0; i < per_resp; i++) {
+        const uintptr_t slot = txr + (uintptr_t)tx_slot[r * per_resp + i] * slot_size;
+        const size_t cur = rem <= mtu ? rem : mtu;
+        rem -= cur;
+        p->rr_append_mbuf(slot, slot, slot + hl, cur);
+      }
+      tx[k].push_back(p);
+    }
+  }
+  auto fill = [&](const std::vector<uint64_t> &v, double *o) {
+    const SgStatLine s = sg_stat_line(v);
+    for (int i = 0; i < 7; i++) o[i] = s.v[i];
+  };
+  int rc = 0;
+  if (mode == 2) {
+    for (uint32_t i = 0; i < 20 && i < steps; i++) engine.gather(rx[0][i % n_req], (uint8_t *)(uintptr_t)bases[2] + (i % n_req) * req_size);
+    engine.GDelay.clear();
+    engine.numSkbs.clear();
+    const uint64_t t0 = getCurNs();
+    for (uint32_t i = 0; i < steps; i++) {
+      const uint32_t k = i % n_items, r = (i / n_items) % n_req;
+      engine.gather(rx[k][r], (uint8_t *)(uintptr_t)bases[4 * k + 2] + r * req_size);
+      if (engine.last_rc != SG_OK) rc = -10;
+    }
+    out[0] = (double)(getCurNs() - t0) * 1e-9 / steps;
+    fill(engine.GDelay, out + 1);
+    fill(std::vector<uint64_t>(), out + 8);
+    engine.GDelay.clear();
+    engine.numSkbs.clear();
+  } else {
+    auto step = [&](uint32_t i) {
+      const uint32_t k = i % n_items;
+      SgRingView rv{sg_ring_desc{(void *)(uintptr_t)bases[4 * k], n_slots, slot_size, profile, 0}};
+      SgRingView tv{sg_ring_desc{(void *)(uintptr_t)bases[4 * k + 1], tx_n_slots, slot_size, profile, 0}};
+      sg_app_desc ra, ta;
+      std::memset(&ra, 0, sizeof ra);
+      std::memset(&ta, 0, sizeof ta);
+      ra.arena = (void *)(uintptr_t)bases[4 * k + 2];
+      ra.arena_cap = req_cap;
+      ta.arena = (void *)(uintptr_t)bases[4 * k + 3];
+      ta.arena_cap = resp_cap;
+      if (engine.gather_batch(rx[k].data(), n_req, rv, ra, nullptr, req_size, profile == SG_HDR_BL58 || frag_len ? mtu : 0,
+                              SG_F_ASYNC) != SG_OK)
+        rc = -11;
+      if (engine.scatter_batch(tx[k].data(), n_req, tv, ta, mtu, flags | SG_F_ASYNC) != SG_OK) rc = -12;
+    };
+    for (uint32_t i = 0; i < 2 * n_items && rc == 0; i++) step(i);
+    if (engine.sync() != SG_OK) rc = -13;
+    engine.GBatchHostNs.clear();
+    engine.SBatchHostNs.clear();
+    const uint64_t t0 = getCurNs();
+    for (uint32_t i = 0; i < steps && rc == 0; i++) step(i);
+    if (engine.sync() != SG_OK && rc == 0) rc = -14;
+    out[0] = (double)(getCurNs() - t0) * 1e-9 / steps;
+    fill(engine.GBatchHostNs, out + 1);
+    fill(engine.SBatchHostNs, out + 8);
+    engine.GBatchHostNs.clear();
+    engine.SBatchHostNs.clear();
+  }
+  for (auto &v : rx)
+    for (auto *q : v) pool.reap_rr(q);
+  for (auto &v : tx)
+    for (auto *q : v) pool.reap_rr(q);
+  return rc;
+}
+
+// `steps` passes of the shunter's loop as one sg_hip_shunt_batch call each, from a native loop
+// over `n_ctx` contexts (streams) taken in turns, so that up to n_ctx calls are in flight; pass i
+// uses the i-th of `n` prepared argument sets.  Returns the seconds the loop took (device drained
+// at the end) or a negative error code.  `lat_ns` (steps entries, or NULL): with n_ctx == 1 every
+// call is made synchronous and its nanoseconds are left there.
+double sgh_shunt_loop_gpu(sg_hip_ctx *const *ctxs, uint32_t n_ctx, const sg_gather_args *const *ga,
+                          const sg_scatter_args *const *sa, uint32_t n, uint32_t steps, uint64_t *lat_ns)
+{
+  if (!ctxs || !n_ctx || !ga || !sa || n == 0) return (double)SG_E_INVAL;
+  int rc = SG_OK;
+  for (uint32_t c = 0; c < n_ctx && rc == SG_OK; c++) rc = sg_hip_sync(ctxs[c]);
+  if (rc != SG_OK) return (double)rc;
+  const uint64_t t0 = getCurNs();
+  if (lat_ns && n_ctx == 1) {
+    for (uint32_t i = 0; i < steps; i++) {
+      const uint64_t a = getCurNs();
+      rc = sg_hip_shunt_batch(ctxs[0], ga[i % n], sa[i % n]);
+      if (rc == SG_OK) rc = sg_hip_sync(ctxs[0]);
+      if (rc != SG_OK) return (double)rc;
+      lat_ns[i] = getCurNs() - a;
+    }
+  } else {
+    for (uint32_t i = 0; i < steps; i++) {
+      rc = sg_hip_shunt_batch(ctxs[i % n_ctx], ga[i % n], sa[i % n]);
+      if (rc != SG_OK) return (double)rc;
+    }
+  }
+  for (uint32_t c = 0; c < n_ctx && rc == SG_OK; c++) rc = sg_hip_sync(ctxs[c]);
+  if (rc != SG_OK) return (double)rc;
+  return (double)(getCurNs() - t0) * 1e-9;
+}
+
+// The receive path on the device, burst after burst, from a native loop and without a host wait:
+// burst k is filed by sg_hip_reassemble(ra, ras[k]) and the requests it completed are gathered and
+// answered by sg_hip_shunt_batch(sg, ga[k], sa[k]) (their counts stay on the device).  With
+// `overlapped` the two contexts are different ones (a stream each), the reassembly's output tables
+// are two sets taken in turns (ras[k], ga[k], sa[k] name set k & 1) and events order the streams:
+// the copy of burst k waits for its tables, the reassembly of burst k + 2 for the copy of burst k
+// to have read them -- so burst k + 1 is filed while burst k is copied.  Returns the seconds the
+// loop took, both contexts drained, or a negative error code.
+double sgh_pipeline_loop_gpu(sg_hip_ctx *ra, sg_hip_ctx *sg, const sg_reassemble_args *const *ras,
+                             const sg_gather_args *const *ga, const sg_scatter_args *const *sa, uint32_t n_bursts,
+                             int overlapped)
+{
+  if (!ra || !sg || !ras || !ga || !sa) return (double)SG_E_INVAL;
+  if (overlapped && ra == sg) return (double)SG_E_INVAL;
+  hipStream_t s_ra = static_cast<hipStream_t>(sg_hip_stream(ra)), s_sg = static_cast<hipStream_t>(sg_hip_stream(sg));
+  hipEvent_t filled[2] = {nullptr, nullptr}, drained[2] = {nullptr, nullptr};
+  bool have_drained[2] = {false, false};
+  for (int j = 0; j < 2 && overlapped; j++)
+    if (hipEventCreateWithFlags(&filled[j], hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&drained[j], hipEventDisableTiming) != hipSuccess)
+      return (double)SG_E_HIP;
+  int rc = sg_hip_sync(ra);
+  if (rc == SG_OK && sg != ra) rc = sg_hip_sync(sg);
+  const uint64_t t0 = getCurNs();
+  // files burst k on the reassembly's stream (once the copy that last read its table set is through)
+  auto file = [&](uint32_t k) {
+    const int j = k & 1;
+    if (overlapped && have_drained[j] && hipStreamWaitEvent(s_ra, drained[j], 0) != hipSuccess) return SG_E_HIP;
+    int r = sg_hip_reassemble(ra, ras[k], nullptr);
+    if (r == SG_OK && overlapped && hipEventRecord(filled[j], s_ra) != hipSuccess) r = SG_E_HIP;
+    return r;
+  };
+  if (overlapped && n_bursts) rc = file(0);
+  for (uint32_t k = 0; k < n_bursts && rc == SG_OK; k++) {
+    const int j = k & 1;
+    if (overlapped) {
+      // burst k + 1 is queued ahead of the copy of burst k: when both become runnable together, the
+      // reassembly's few large workgroups are placed before the copy's many small ones fill the chip
+      if (k + 1 < n_bursts) rc = file(k + 1);
+      if (rc == SG_OK && hipStreamWaitEvent(s_sg, filled[j], 0) != hipSuccess) rc = SG_E_HIP;
+    } else {
+      rc = file(k);
+    }
+    if (rc == SG_OK) rc = sg_hip_shunt_batch(sg, ga[k], sa[k]);
+    if (rc == SG_OK && overlapped) {
+      if (hipEventRecord(drained[j], s_sg) != hipSuccess) rc = SG_E_HIP;
+      have_drained[j] = true;
+    }
+    // a caller takes the counts in now and then; it also keeps the queues from growing without bound
+    if (rc == SG_OK && (k & 255u) == 255u) rc = sg_hip_sync(sg);
+  }
+  if (rc == SG_OK) rc = sg_hip_sync(ra);
+  if (rc == SG_OK && sg != ra) rc = sg_hip_sync(sg);
+  const double dt = (double)(getCurNs() - t0) * 1e-9;
+  for (int j = 0; j < 2; j++) {
+    if (filled[j]) (void)hipEventDestroy(filled[j]);
+    if (drained[j]) (void)hipEventDestroy(drained[j]);
+  }
+  return rc == SG_OK ? dt : (double)rc;
 }
 
 }  // extern "C"

@@ -13,6 +13,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <climits>
 #include <cstdint>
 #include <cstdio>
@@ -28,14 +29,37 @@ class MetaAppCtx {
  public:
   MetaAppCtx() : curr_batch_size(1), next_batch_size(1) {}
 
-  // work queued after this call runs once *d_state == value (src/p2p_rpc_app_ctx.h:35-37): the
-  // calling thread waits for the word (it lives in pinned host memory) and only then goes on queueing
-  inline void AppRrRunNotify(volatile uint32_t *d_state, int value)
+  // Work queued after this call runs once *d_state == value (src/p2p_rpc_app_ctx.h:35-37).  The
+  // reference queues a wait on the stream and returns; here the CALLING THREAD waits for the word
+  // (it lives in pinned host memory) and only then goes on queueing.  So the word has to be set by
+  // somebody else -- another thread, or work that is already queued: a thread that calls this and
+  // means to set the word itself afterwards, as it may with the reference's queued wait, would wait
+  // for itself.  The wait is therefore bounded: after notify_timeout_ns (default 2 s; 0 = no
+  // bound) it gives up, reports, and returns false; notify_timeouts counts such returns.
+  inline bool AppRrRunNotify(volatile uint32_t *d_state, int value)
   {
-    while (*d_state != (uint32_t)value) __builtin_ia32_pause();
+    if (*d_state == (uint32_t)value) return true;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t spins = 0;; spins++) {
+      if (*d_state == (uint32_t)value) return true;
+      __builtin_ia32_pause();
+      if ((spins & 1023u) == 1023u && notify_timeout_ns) {
+        const auto waited = std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - t0).count();
+        if ((uint64_t)waited > notify_timeout_ns) {
+          notify_timeouts++;
+          std::printf("MetaAppCtx: waited %llu ns for a state word to become %d (it holds %u): giving up\n",
+                      (unsigned long long)waited, value, *d_state);
+          return false;
+        }
+      }
+    }
   }
   // the same on this context's doorbell (:40-42)
-  inline void AppRunNotify(int value) { AppRrRunNotify(d_door_bell, value); }
+  inline bool AppRunNotify(int value) { return AppRrRunNotify(d_door_bell, value); }
+  // the same without waiting: true when the word holds the value now
+  inline bool AppRrRunReady(volatile uint32_t *d_state, int value) const { return *d_state == (uint32_t)value; }
+  uint64_t notify_timeout_ns = 2000000000ull;
+  uint64_t notify_timeouts = 0;
   // the doorbell is set once what was queued before is done (:45-47)
   inline void AppCompleteNotify(uint32_t value = 2)
   {

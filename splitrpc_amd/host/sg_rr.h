@@ -12,6 +12,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "sg_hip.h"
 #include "sg_tables.h"
 #include "sg_wire.h"
 
@@ -33,6 +34,13 @@ class P2pRpcRr {
   p2p_bufs *payload_bufs;
   // copy engine scratch
   p2p_sk_buf *payload_sk_bufs;
+  // The payload table once more, in the form the device reads (sg_frag_table: 32-bit offsets from
+  // pkt_base and lengths), written entry for entry with payload_bufs where a table is attached.
+  // The table lives in memory the GPU can read (the copy engine allocates it, pinned), so a batched
+  // gather or scatter names the table and walks no fragment on the host.  No counterpart in the
+  // reference; nullptr: not kept.
+  sg_frag_table *frag_table = nullptr;
+  uintptr_t pkt_base = 0;
 
   explicit P2pRpcRr(p2p_rpc_conn_info *template_conn_info = nullptr, size_t _max_payload_size = 0)
       : req_token(0), payload_size(0), max_payload_size(_max_payload_size), rr_state(RR_CREATE),
@@ -69,6 +77,13 @@ class P2pRpcRr {
     payload_bufs->burst_items[idx] = payload_buf;
     payload_bufs->item_size[idx] = item_size;
     payload_bufs->num_items++;
+    if (frag_table) {
+      // an address the 32-bit form cannot hold becomes an entry the device refuses
+      const uintptr_t d = payload_buf - pkt_base;
+      const bool fits = payload_buf >= pkt_base && !(d & 1u) && (d >> 33) == 0 && (d >> 1) != 0xffffffffu;
+      frag_table->off[idx] = fits ? (uint32_t)(d >> 1) : 0xffffffffu;
+      frag_table->len[idx] = (uint32_t)item_size;
+    }
   }
 
   // at the end, whatever the frame id (src/p2p_rpc_rr_ng.h:85-93)
@@ -191,6 +206,7 @@ class P2pRpcRRPool {
   P2pRpcRr *proto_rr;
   int pool_size;
   uint32_t hdr_profile;
+  uintptr_t frag_pkt_base = 0;  // what the rrs' fragment tables count from when they file a request
 
  public:
   // _pool_size == -1: RR_POOL_SIZE rrs; else _pool_size - 1 (as the reference counts)
@@ -230,6 +246,22 @@ class P2pRpcRRPool {
     for (int i = 0; i < pool_size; i++) rr_pool.push_back(rr_clone_alloc(proto_rr));
     for (int i = 0; i < pool_size; i++)
       if (free_rr_pool->enqueue(rr_pool[i]) != 0) std::printf("P2pRpcRRPool: Free pool full!\n");
+  }
+
+  // Gives rr i of the pool table i of `tables` (n of them, in memory the GPU reads; see
+  // P2pRpcSgHipEngine::frag_tables) and the address its 32-bit offsets count from.  Rrs beyond n,
+  // and rrs the pool allocates later when it runs dry, keep none: batched calls walk those on the host.
+  // The 32-bit offsets reach 8 GiB: where response buffers come from memory further than that
+  // from the request buffers, whoever hands an rr its response buffers sets rr->pkt_base to that
+  // memory's base first (reap_rr sets it back).
+  void attach_frag_tables(sg_frag_table *tables, size_t n, uintptr_t pkt_base)
+  {
+    frag_pkt_base = pkt_base;
+    for (size_t i = 0; i < rr_pool.size(); i++) {
+      if (!rr_pool[i]) continue;
+      rr_pool[i]->frag_table = i < n ? tables + i : nullptr;
+      rr_pool[i]->pkt_base = pkt_base;
+    }
   }
 
   // cached rr of this token, or a fresh one filed under it (:97-109)
@@ -289,6 +321,7 @@ class P2pRpcRRPool {
     rr->payload_bufs->num_items = 0;
     rr->payload_size = 0;
     rr->req_token = 0;
+    rr->pkt_base = frag_pkt_base;
     if (free_rr_pool->enqueue(rr) == -ENOBUFS) {
       std::printf("Warning!, P2pRpcRRPool is full, de-allocating rr: %p\n", (void *)rr);
       for (auto &q : rr_pool)

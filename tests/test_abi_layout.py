@@ -11,7 +11,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 MIRRORS = [("sg_hbufs", capi.HBufs), ("sg_sk_buf", capi.SkBuf), ("sg_hip_cfg", capi.Cfg),
            ("sg_ring_desc", capi.RingDesc), ("sg_app_desc", capi.AppDesc), ("sg_gather_args", capi.GatherArgs),
-           ("sg_scatter_args", capi.ScatterArgs), ("sg_reassemble_args", capi.ReassembleArgs)]
+           ("sg_scatter_args", capi.ScatterArgs), ("sg_reassemble_args", capi.ReassembleArgs),
+           ("sg_frag_table", capi.FragTable), ("sg_pack_args", capi.PackArgs)]
 
 
 def test_ctypes_mirrors_match_the_header(tmp_path):

@@ -709,3 +709,47 @@ def test_echo_scatter_reuses_the_descriptors_of_its_gather(ctx):
         fresh.scatter_batch_raw(a)
     assert e.value.code == capi.SG_E_INVAL
     fresh.close()
+
+
+def test_reused_descriptors_are_held_against_the_call_that_uses_them(ctx):
+    """SG_F_REUSE_DESC trusts nothing the describing pass did not check: a TX
+    ring of smaller slots, another arena, or a smaller mtu than the lengths
+    described are refused with SG_E_DATA -- the first two before a byte moves."""
+    sizes = [3000, 1400, 4200, 77, 2800, 1401]
+    w = synth.make_custom(sizes, sizes, seed=91, in_place=True)
+    dw = DeviceWorkload(w)
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    dw.gather(ctx, fixed=False)
+    assert getattr(dw, "_described")
+
+    def call(tx, mtu, app):
+        a = ctx.scatter_args(dw.rx, tx, dw.tx_slot, dw.hdr_src_slot, dw.resp_first, None, 0, dw.n_req, dw.n_frames,
+                             mtu, app, None, w.flags | capi.F_REUSE_DESC)
+        with pytest.raises(SgError) as e:
+            ctx.scatter_batch_raw(a)
+        return e.value
+
+    # a TX ring whose slots are smaller than the slots the lengths were held against
+    small = torch.full((w.n_slots * 1024,), 0x5A, dtype=torch.uint8, device=DEV)
+    e = call(RingRef(small, w.n_slots, 1024, w.profile), 900, dw.resp_app)
+    assert e.code == capi.SG_E_DATA and "longer than a slot" in str(e)
+    assert bool((small == 0x5A).all())
+    # the same requests, but in another arena than the one the offsets were made for
+    other = torch.zeros_like(dw.req_arena)
+    tx = torch.full((w.n_slots * w.slot_size,), 0x5A, dtype=torch.uint8, device=DEV)
+    e = call(RingRef(tx, w.n_slots, w.slot_size, w.profile), w.mtu, AppRef(arena=other, cap=dw.req_app.cap))
+    assert e.code == capi.SG_E_DATA and "destination" in str(e)
+    assert bool((tx == 0x5A).all())
+    # an arena of another capacity
+    e = call(RingRef(tx, w.n_slots, w.slot_size, w.profile), w.mtu, AppRef(arena=dw.req_arena, cap=dw.req_app.cap - 16))
+    assert e.code == capi.SG_E_DATA
+    assert bool((tx == 0x5A).all())
+    # a smaller mtu than the described lengths: the frames beyond it are refused
+    e = call(RingRef(tx, w.n_slots, w.slot_size, w.profile), 1000, dw.resp_app)
+    assert e.code == capi.SG_E_DATA and "longer than a slot" in str(e)
+    # and the matching call still goes through afterwards
+    exp, _, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    dw.scatter(ctx, fixed=False, reuse=True)
+    exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.req_app.cap)
+    assert np.array_equal(dw.ring.cpu().numpy(), exp_tx)

@@ -45,14 +45,14 @@ def p(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
 
-@pytest.mark.parametrize("per_request", [1, 0, 2], ids=["per-request", "batched", "batched-tx"])
+@pytest.mark.parametrize("per_request", [1, 0, 2, 3], ids=["per-request", "batched", "batched-tx", "tables-pulled"])
 @pytest.mark.parametrize("mirror", [1, 0], ids=["mirrored", "plain"])
 @pytest.mark.parametrize("cfg,n,profile", [(1, 12, synth.HDR_BL58), (2, 3, synth.HDR_BL58),
                                            (2, 2, synth.HDR_REF64), (5, 1, synth.HDR_BL58)])
 def test_one_burst_of_the_shunter(host, cfg, n, profile, mirror, per_request):
     w = synth.make_workload(cfg, n, profile=profile)
     flags = w.flags & ~synth.F_UDP_CSUM_FULL  # a header-only rewrite cannot see the payload
-    if per_request == 2:
+    if per_request >= 2:
         flags = w.flags                           # the batched TX writes headers with the payload in hand
     print(f"case serve cfg={cfg} n={n} profile={profile} mirror={mirror} per_request={per_request}", flush=True)
     req_size, resp_size = int(w.req_sizes[0]), int(w.resp_sizes[0])
@@ -73,7 +73,7 @@ def test_one_burst_of_the_shunter(host, cfg, n, profile, mirror, per_request):
     exp, _, _ = oracle.gather(w)
     assert np.array_equal(req_out, exp), first_diff(req_out, exp)
     exp_tx = w.tx_ring_init.copy()
-    if per_request == 2:
+    if per_request >= 2:
         # fresh response buffers: headers from the connections' templates (rr_set_hdr), the server
         # identity being the one the host layer was started with
         import socket

@@ -249,6 +249,32 @@ def test_slot_states_published_by_the_device():
         ctx.gather_batch_raw(ga)
     assert not states.cpu().numpy().any()
     assert ctx.get_slot_index(0) == pi
+    # the same bad fragment with the rule declared: the other fragments move and the cursor moves (no
+    # descriptor pass has looked at the batch beforehand), but no slot is published -- a worker that
+    # polls the words is never handed a request with a hole in it -- and the ring index stays
+    ga = ctx.gather_args(dw.rx, bad_dev, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app, dw.req_offsets,
+                         flags=capi.F_RULE_FRAGS, fixed_req_size=4200, mtu=w.mtu, slot_state=states)
+    c0 = ctx.get_cursor(0)
+    with pytest.raises(SgError) as e:
+        ctx.gather_batch_raw(ga)
+    assert e.value.code == capi.SG_E_DATA
+    assert not states.cpu().numpy().any()
+    assert ctx.get_slot_index(0) == pi
+    assert ctx.get_cursor(0) == (c0 + 5 * 4200) % dw.req_app.cap
+    # and on the TX side: a bad TX slot index with one response size
+    states.fill_(WORK)
+    bad_tx = w.tx_slot.copy()
+    bad_tx[1] = w.tx_n_slots + 4
+    bad_tx_dev = to_dev(bad_tx, DEV)
+    sa = ctx.scatter_args(dw.rx, dw.tx, bad_tx_dev, dw.hdr_src_slot, dw.resp_first, None, 3000, dw.n_req,
+                          dw.n_frames, w.mtu, dw.resp_app, dw.resp_offsets, w.flags, slot_state=states)
+    ci = ctx.get_slot_index(1)
+    with pytest.raises(SgError) as e:
+        ctx.scatter_batch_raw(sa)
+    assert e.value.code == capi.SG_E_DATA
+    assert bool((states == WORK).all())
+    assert ctx.get_slot_index(1) == ci
+    states.zero_()
     # more requests than the ring has slots: refused by the host
     small = torch.zeros(3, dtype=torch.int32, device=DEV)
     ga = ctx.gather_args(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, dw.req_app, slot_state=small)
@@ -360,3 +386,99 @@ def test_bursts_through_reassembly_gather_and_scatter_without_the_host(use_graph
         assert not states.cpu().numpy().any()
     assert done == n_reqs
     ctx.close()
+
+
+@pytest.mark.parametrize("burst", [7, 16, 40])
+def test_reassembly_on_a_stream_of_its_own_beside_the_copy(burst):
+    """The receive path with burst k + 1 being filed while burst k is gathered
+    and answered: the reassembly on one context (stream), gather + scatter
+    (sg_hip_shunt_batch) on another, the reassembly's output tables
+    double-buffered and events between the two streams -- every burst queued,
+    the host waiting for nothing until the end.  Final request arena, TX ring
+    and cursors against the oracle's reassembly, gather and scatter replayed
+    burst by burst."""
+    n_reqs, resp_size = 36, 3000
+    w = synth.make_custom([4200] * n_reqs, [resp_size] * n_reqs, seed=63,
+                          flags=synth.F_UDP_CSUM_PSEUDO | synth.F_IPV4_CSUM)
+    order = np.random.default_rng(14).permutation(w.arrivals)
+    efs, efl, erf, etok = oracle.reassemble(w, arrivals=order)
+    slot_req = {int(s): r for r in range(n_reqs) for s in efs[erf[r]:erf[r + 1]]}
+    per_req, per_resp = 3, synth.num_frames(resp_size, w.mtu)
+    ctx_ra = SgContext(0, max_reqs=64, max_frames=4096)
+    ctx_sg = SgContext(0, max_reqs=64, max_frames=4096)
+    ctx_ra.reassemble_reset()
+    s_ra = torch.cuda.ExternalStream(ctx_ra.stream, device=DEV)
+    s_sg = torch.cuda.ExternalStream(ctx_sg.stream, device=DEV)
+    sets = [Tables(64, 4096), Tables(64, 4096)]
+    rx = RingRef(torch.from_numpy(w.ring).to(DEV), w.n_slots, w.slot_size, w.profile)
+    bound = min(burst, n_reqs)  # a burst of b arrivals completes at most b requests
+    tx_slots = np.random.default_rng(15).permutation(bound * per_resp).astype(np.uint32)
+    tx_init = np.random.default_rng(16).integers(0, 256, bound * per_resp * w.slot_size, dtype=np.uint8)
+    tx_ring = torch.from_numpy(tx_init).to(DEV)
+    tx = RingRef(tx_ring, bound * per_resp, w.slot_size, w.profile)
+    req_cap, resp_cap = n_reqs * 4200 + 100, 7 * resp_size + 50  # every request of the run keeps its place
+    req_arena = torch.zeros(req_cap, dtype=torch.uint8, device=DEV)
+    resp_np = np.random.default_rng(17).integers(0, 256, resp_cap, dtype=np.uint8)
+    resp_arena = torch.from_numpy(resp_np).to(DEV)
+    arr = to_dev(np.ascontiguousarray(order, np.uint32), DEV)
+    tx_slot_dev = to_dev(tx_slots, DEV)
+    resp_first = to_dev((np.arange(bound + 1) * per_resp).astype(np.uint32), DEV)
+    A = capi.F_ASYNC
+    gas, sas = [], []
+    for t in sets:
+        gas.append(ctx_sg.gather_args(rx, t.fs, None, t.rf, bound, bound * per_req, AppRef(arena=req_arena, cap=req_cap),
+                                      None, flags=A | capi.F_RULE_FRAGS, fixed_req_size=4200, mtu=w.mtu,
+                                      counts=t.counts))
+        sas.append(ctx_sg.scatter_args(rx, tx, tx_slot_dev, None, resp_first, None, resp_size, bound,
+                                       bound * per_resp, w.mtu, AppRef(arena=resp_arena, cap=resp_cap), None,
+                                       w.flags | A, hdr_src_req=t.hdr, counts=t.counts))
+    start = req_cap - 5000
+    ctx_sg.set_cursor(0, start)
+    ctx_sg.set_cursor(1, 0)
+    torch.cuda.synchronize()
+    filled = [torch.cuda.Event(), torch.cuda.Event()]
+    drained = [None, None]
+    keep = []
+    for k, b in enumerate(range(0, len(order), burst)):
+        j = k & 1
+        t = sets[j]
+        n = min(burst, len(order) - b)
+        if drained[j] is not None:
+            s_ra.wait_event(drained[j])          # the copy of burst k - 2 has read this set
+        ra = ctx_ra.reassemble_args(rx, arr[b:b + n], n, t.fs, t.fl, t.rf, t.tok, req_hdr_slot=t.hdr,
+                                    counts_out=t.counts, flags=A)
+        keep.append(ra)
+        ctx_ra.reassemble_raw(ra)
+        filled[j].record(s_ra)
+        s_sg.wait_event(filled[j])               # the copy of burst k starts once its tables are in
+        ctx_sg.shunt_batch_raw(gas[j], sas[j])
+        drained[j] = torch.cuda.Event()
+        drained[j].record(s_sg)
+    ctx_ra.sync()
+    ctx_sg.sync()
+    torch.cuda.synchronize()
+    # the oracle, burst by burst
+    want_req = np.zeros(req_cap, np.uint8)
+    want_tx = tx_init.copy()
+    cur0, cur1, done = start, 0, 0
+    pos_done = np.zeros(n_reqs, int)
+    for b in range(0, len(order), burst):
+        for sl in order[b:b + burst]:
+            pos_done[slot_req[int(sl)]] += 1
+        now = int((pos_done == per_req).sum())
+        r0, r1 = done, now
+        if r1 > r0:
+            sub = _sub(w, efs[erf[r0]:erf[r1]], efl[erf[r0]:erf[r1]], erf[r0:r1 + 1] - erf[r0], None, tx_slots,
+                       efs[erf[r0:r1]], resp_size)
+            want_req, _, cur0 = oracle.gather(sub, arena_cap=req_cap, cursor=cur0, out=want_req)
+            sub.tx_n_slots = bound * per_resp
+            _, cur1 = oracle.scatter(sub, w.ring, want_tx, resp_np, arena_cap=resp_cap, cursor=cur1)
+        done = now
+    assert done == n_reqs
+    got = req_arena.cpu().numpy()
+    assert np.array_equal(got, want_req), first_diff(got, want_req)
+    got = tx_ring.cpu().numpy()
+    assert np.array_equal(got, want_tx), first_diff(got, want_tx)
+    assert ctx_sg.get_cursor(0) == cur0 and ctx_sg.get_cursor(1) == cur1
+    ctx_ra.close()
+    ctx_sg.close()

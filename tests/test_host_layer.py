@@ -152,6 +152,26 @@ def test_pointer_ring_multi_producer_multi_consumer(host):
 
 # ---------------------------------------------------------------- client patterns (load generator)
 
+def test_state_word_wait_is_bounded(host):
+    """AppRrRunNotify waits on the calling thread: the word has to be set by
+    somebody else.  Another thread setting it ends the wait; nobody setting it
+    in time ends it too, with a false return and a count."""
+    host.sgh_notify_wait.argtypes = [C.c_uint32, C.c_uint64]
+    assert host.sgh_notify_wait(2000, 2_000_000_000) == 1 | 4        # set after 2 ms: seen
+    assert host.sgh_notify_wait(200_000, 20_000_000) == 2 | 4        # set after 200 ms, bound 20 ms: gave up
+    assert host.sgh_notify_wait(0, 0) & 1                            # no bound: still returns once set
+
+
+def test_bench_has_measured_traffic_for_every_default_call():
+    """roofline.traffic comes from counter runs of the default calls: a default
+    that changes without a fresh counter run would silently report None."""
+    import bench
+    for cfg, bpl in bench.DEFAULT_BPL.items():
+        for kernel in ("k_gather", "k_scatter"):
+            assert (cfg, bpl, kernel) in bench.MEASURED_TRAFFIC, (cfg, bpl, kernel)
+            assert bench.MEASURED_TRAFFIC[(cfg, bpl, kernel)] > 0
+
+
 def test_client_patterns_and_checks_through_the_cpu_path():
     """The reference clients' request patterns and reply checks
     (lib_loadgen/echo_client.cc, vec_add_client.cc) around the oracle's gather

@@ -678,4 +678,4 @@ def test_c_abi_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert sorted(capi.SYMBOLS) == declared
-    assert lib.sg_hip_abi_version() == 2
+    assert lib.sg_hip_abi_version() == 3

@@ -1,5 +1,7 @@
-"""The allocation-free gather (sg_hip_gather_batch_static) against the context's
-sg_hip_gather_batch on the same inputs, bit for bit, through the C ABI.
+"""The allocation-free gather (sg_hip_gather_batch_static) against the CPU oracle
+and against the context's sg_hip_gather_batch on the same inputs, bit for bit,
+through the C ABI; that it leaves the device's free memory alone; and that a
+call recorded into a HIP graph replays.
 
 Collected last on purpose (the file name sorts behind the other tests): the
 static scratch array is shared by every call on the GPU, so these cases also
@@ -11,6 +13,7 @@ import numpy as np
 import pytest
 import torch
 
+import oracle
 from splitrpc_amd import capi, synth
 from splitrpc_amd.engine import AppRef, DeviceWorkload, SgContext, to_dev
 
@@ -75,10 +78,19 @@ def test_two_calls_in_a_row_the_second_smaller(mode):
         print(f"case no-alloc mode={mode} n_req={w.n_req} n_frags={w.n_frags} start={start}", flush=True)
         (a0, o0, c0, _), (a1, o1, c1, st) = _both_ways(ctx, w, cap, start, mode)
         assert st == 0
+        # against the oracle directly: the bytes of the batch where the bump ring puts them, the
+        # arena's fill everywhere else, the offsets and the cursor
+        exp, eoffs, ecur = oracle.gather(w, arena_cap=cap, cursor=start)
+        total = int(w.req_sizes.sum())
+        written = np.zeros(cap, bool)
+        written[(start + np.arange(total)) % cap] = True
+        assert np.array_equal(a1[written], exp[written])
+        assert bool((a1[~written] == 0x5A).all())
+        assert np.array_equal(o1, eoffs) and c1 == ecur
+        # and against the context's call
         assert np.array_equal(o0, o1)
         assert c0 == c1
         assert np.array_equal(a0, a1)
-        assert (a0 != 0x5A).sum() > 0.9 * int(w.req_sizes.sum())  # and it is not the fill that agrees
         start = c1
     ctx.close()
 
@@ -143,4 +155,68 @@ def test_limits_and_refusals():
     assert int(status[0]) != 0
     assert bool((dw.req_arena == 0xAB).all())
     assert int(cursor[0]) == 0
+    ctx.close()
+
+
+def test_calls_leave_device_memory_alone_and_replay_from_a_graph():
+    """What the entry point exists for: after a warm first call, further calls
+    change nothing in the device's free memory, and a call recorded into a HIP
+    graph on a stream replays -- twice, with eager work between -- continuing
+    the bump ring, like the context's call from the same positions."""
+    w = synth.make_custom([4200] * 50, [64] * 50, seed=41)
+    dw = DeviceWorkload(w)
+    total = int(w.req_sizes.sum())
+    cap = 3 * total + 555
+    arena = torch.zeros(cap, dtype=torch.uint8, device=DEV)
+    offs = torch.zeros(w.n_req + 1, dtype=torch.int64, device=DEV)
+    cursor = torch.zeros(1, dtype=torch.int64, device=DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ctx = SgContext(0)
+    for mode in ("rule", "scan"):
+        a = ctx.gather_args(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags, AppRef(arena=arena, cap=cap),
+                            offs, flags=capi.F_RULE_FRAGS if mode == "rule" else 0,
+                            fixed_req_size=4200 if mode == "rule" else 0, mtu=w.mtu)
+        cursor.zero_()
+        torch.cuda.synchronize()
+        assert _static_call(ctx.lib, a, cursor, status) == capi.SG_OK  # warm: looks up the array's address
+        torch.cuda.synchronize()
+        free0, _ = torch.cuda.mem_get_info()
+        for _ in range(5):
+            assert _static_call(ctx.lib, a, cursor, status) == capi.SG_OK
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        assert free1 == free0, f"{mode}: free device memory went from {free0} to {free1}"
+        assert int(status[0]) == 0
+        assert int(cursor[0]) == (6 * total) % cap
+        # one call recorded on a side stream, replayed twice
+        cursor.zero_()
+        s = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            rc = ctx.lib.sg_hip_gather_batch_static(0, C.c_void_p(s.cuda_stream), C.byref(a),
+                                                    C.c_void_p(cursor.data_ptr()), C.c_void_p(status.data_ptr()))
+        assert rc == capi.SG_OK, ctx.lib.sg_hip_last_error(None).decode()
+        pos = 0
+        for rep in range(2):
+            arena.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            exp, eoffs, nxt = oracle.gather(w, arena_cap=cap, cursor=pos)
+            got = arena.cpu().numpy()
+            assert np.array_equal(got, exp), f"{mode} replay {rep}"
+            assert np.array_equal(offs.cpu().numpy().view(np.uint64), eoffs)
+            assert int(cursor[0]) == nxt and int(status[0]) == 0
+            # the context's call from the same position
+            ctx.set_cursor(0, pos)
+            arena2 = torch.zeros_like(arena)
+            a2 = ctx.gather_args(dw.rx, dw.frag_slot, None, dw.req_first, dw.n_req, dw.n_frags,
+                                 AppRef(arena=arena2, cap=cap), None, flags=a.flags, fixed_req_size=a.fixed_req_size,
+                                 mtu=w.mtu)
+            ctx.gather_batch_raw(a2)
+            assert torch.equal(arena2, arena) and ctx.get_cursor(0) == nxt
+            pos = nxt
+            junk = torch.full((1 << 18,), rep, dtype=torch.uint8, device=DEV)
+            assert int(junk[3]) == rep
     ctx.close()
