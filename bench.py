@@ -43,7 +43,7 @@ MEASURED_TRAFFIC = {
     (5, 4, "k_gather"): 817.6e6, (5, 4, "k_scatter"): 549.3e6,
 }
 # the same for the reference's own 64-byte header (bench.py --ref64)
-MEASURED_TRAFFIC_REF64 = {}
+MEASURED_TRAFFIC_REF64 = {(2, 32, "k_gather"): 655.5e6, (2, 32, "k_scatter"): 4.8e6}
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 
@@ -83,6 +83,9 @@ def parse():
                     help="skip the single-batch legs (eager, HIP graphs on 1, 2 and 4 streams)")
     ap.add_argument("--general", action="store_true",
                     help="always run the descriptor pass (do not declare the fragmenting rule)")
+    ap.add_argument("--leg", choices=["host-engine", "pipeline"], default=None,
+                    help="run one leg alone and print its object (for a kernel trace of that leg): the C++ "
+                         "engine's batched calls over P2pRpcRr objects, or the receive pipeline at whole-call bursts")
     ap.add_argument("--tx-in-order", action="store_true",
                     help="response frames take their TX slots in ring order (the generator's default "
                          "is a random permutation of the TX ring, the hardest order for the scatter)")
@@ -723,6 +726,15 @@ def main() -> int:
     _log(f"staging {w.name} x {bpl} batches per launch")
     pool = Pool(w, bpl, a.rotate_mb, extra, rule=rule)
     _log(f"{len(pool.items)} ring copies staged")
+
+    if a.leg:
+        res = host_engine_batched(pool, max(20, min(a.steps, 200))) if a.leg == "host-engine" else \
+            device_pipeline(pool, calls=4, bursts=(65536, 0))
+        print(json.dumps({a.leg: res}))
+        ctx.close()
+        if ctx_tx is not None:
+            ctx_tx.close()
+        return 0
 
     if a.calib_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").fill_(3)

@@ -305,6 +305,14 @@ const char *sg_hip_last_error(const sg_hip_ctx *ctx); /* ctx may be NULL: creati
 int sg_hip_abi_version(void);
 void *sg_hip_stream(sg_hip_ctx *ctx); /* the hipStream_t work is launched on */
 
+/* The address of the hardware queue that `stream` (NULL: the context's own) dispatches to, as a
+ * kernel launched on it sees it.  The runtime multiplexes streams over a handful of hardware
+ * queues, and streams that share one run their kernels one after the other whatever the streams'
+ * own order: a caller that wants two streams to run side by side (the pull of the next call's
+ * tables beside the current call's copy) creates streams until two of them answer differently.
+ * Launches a one-wavefront kernel on the stream and waits for it.  No counterpart in the reference. */
+int sg_hip_stream_queue(sg_hip_ctx *ctx, void *stream, uint64_t *queue_out);
+
 /* Waits for everything enqueued on the context and returns SG_E_DATA if any
  * kernel since the last sync refused part of its input. */
 int sg_hip_sync(sg_hip_ctx *ctx);

@@ -45,7 +45,7 @@ SYMBOLS = [
     "sg_hip_sync", "sg_hip_gather", "sg_hip_scatter", "sg_hip_swap_hdrs", "sg_hip_set_hdrs", "sg_hip_gather_batch",
     "sg_hip_scatter_batch", "sg_hip_reassemble", "sg_hip_set_cursor", "sg_hip_get_cursor", "sg_hip_set_profiling",
     "sg_hip_kernel_time", "sg_hip_gather_batch_static", "sg_hip_reassemble_reset", "sg_hip_reassemble_evict",
-    "sg_hip_set_slot_index", "sg_hip_get_slot_index", "sg_hip_shunt_batch", "sg_hip_pack_tables",
+    "sg_hip_set_slot_index", "sg_hip_get_slot_index", "sg_hip_shunt_batch", "sg_hip_pack_tables", "sg_hip_stream_queue",
 ]
 
 SLOT_FREE, SLOT_RX_COMPLETE, SLOT_WORK_COMPLETE, SLOT_TX_COMPLETE = 0, 1, 2, 3
@@ -157,6 +157,7 @@ def load() -> C.CDLL:
     lib.sg_hip_gather_batch.argtypes = [P, C.POINTER(GatherArgs)]
     lib.sg_hip_scatter_batch.argtypes = [P, C.POINTER(ScatterArgs)]
     lib.sg_hip_shunt_batch.argtypes = [P, C.POINTER(GatherArgs), C.POINTER(ScatterArgs)]
+    lib.sg_hip_stream_queue.argtypes = [P, P, C.POINTER(C.c_uint64)]
     lib.sg_hip_pack_tables.argtypes = [P, C.POINTER(PackArgs)]
     lib.sg_hip_gather_batch_static.argtypes = [C.c_int, P, C.POINTER(GatherArgs), P, P]
     lib.sg_hip_reassemble.argtypes = [P, C.POINTER(ReassembleArgs), C.POINTER(C.c_uint32 * 4)]

@@ -117,6 +117,7 @@ struct sg_hip_ctx {
   Run *h_runs = nullptr;
   uint32_t h_runs_cap = 0;
   uint64_t *h_ptrs = nullptr;
+  uint64_t *h_probe = nullptr;   // pinned: what a probe launch saw of itself (queue address, dispatch id), twice
   uint32_t *h_status = nullptr;  // pinned: [0] copy of status (read back only after a refusal), [1] the refusal flag
   volatile uint32_t *h_flag = nullptr;
   // profiling
@@ -565,10 +566,11 @@ static int create_impl(sg_hip_ctx *c, int device_id, const sg_hip_cfg *cfg)
   // its own.  Two probe launches show whether this runtime hands them out: if their pairs agree,
   // or come back empty, calls on this context keep to the kernel behind the call.
   {
-    volatile uint64_t *probe = c->h_ptrs;
+    HIP_TRY(nullptr, hipHostMalloc(&c->h_probe, 4 * sizeof(uint64_t), hipHostMallocDefault));
+    volatile uint64_t *probe = c->h_probe;
     probe[0] = probe[1] = probe[2] = probe[3] = 0;
-    k_stamp_probe<<<1, kWave, 0, c->stream>>>(c->h_ptrs);
-    k_stamp_probe<<<1, kWave, 0, c->stream>>>(c->h_ptrs + 2);
+    k_stamp_probe<<<1, kWave, 0, c->stream>>>(c->h_probe);
+    k_stamp_probe<<<1, kWave, 0, c->stream>>>(c->h_probe + 2);
     HIP_TRY(nullptr, hipGetLastError());
     HIP_TRY(nullptr, hipStreamSynchronize(c->stream));
     c->sc.stamps_ok = probe[0] != 0 && probe[2] != 0 && !(probe[0] == probe[2] && probe[1] == probe[3]);
@@ -633,10 +635,25 @@ void sg_hip_destroy(sg_hip_ctx *c)
   if (c->h_runs) (void)hipHostFree(c->h_runs);
   if (c->h_ptrs) (void)hipHostFree(c->h_ptrs);
   if (c->h_status) (void)hipHostFree(c->h_status);
+  if (c->h_probe) (void)hipHostFree(c->h_probe);
   if (c->h_counts) (void)hipHostFree(c->h_counts);
   (void)hipFree(c->ra_mem);
   if (c->own_stream && c->stream) (void)hipStreamDestroy(c->stream);
   delete c;
+}
+
+int sg_hip_stream_queue(sg_hip_ctx *c, void *stream, uint64_t *queue_out)
+{
+  if (!c || !queue_out) return fail(c, SG_E_INVAL, "null argument");
+  DeviceGuard g(c->device);
+  hipStream_t st = stream ? static_cast<hipStream_t>(stream) : c->stream;
+  volatile uint64_t *probe = c->h_probe;
+  probe[0] = 0;
+  k_stamp_probe<<<1, kWave, 0, st>>>(c->h_probe);
+  HIP_TRY(c, hipGetLastError());
+  HIP_TRY(c, hipStreamSynchronize(st));
+  *queue_out = probe[0];
+  return SG_OK;
 }
 
 int sg_hip_sync(sg_hip_ctx *c)

@@ -159,6 +159,9 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
   sg_frag_table *tables = nullptr;
   uint32_t n_tables = 0;
   hipStream_t pack_stream = nullptr;
+  hipStream_t tx_stream = nullptr;  // the scatter context's stream (made here so that its hardware queue can be chosen)
+  // no stream on a hardware queue of its own was to be had: the work then runs one after the other
+  bool pack_queue_shared = false, tx_queue_shared = false;
 
   void fail(const char *what, int rc, const sg_hip_ctx *c = nullptr) const
   {
@@ -230,6 +233,28 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
     else (void)hipStreamSynchronize(stream(dir));
   }
 
+  // A stream that dispatches to another hardware queue than those in `avoid` (streams that share a
+  // queue run one after the other, and the runtime deals its few queues out in turns): streams are
+  // made until one answers differently, the others given back.  Falls back to the first made;
+  // *shared then says so.
+  hipStream_t stream_apart(const uint64_t *avoid, int n_avoid, bool *shared)
+  {
+    hipStream_t tried[8], found = nullptr;
+    int n_tried = 0;
+    for (; n_tried < 8 && !found; n_tried++) {
+      if (hipStreamCreateWithFlags(&tried[n_tried], hipStreamNonBlocking) != hipSuccess) break;
+      uint64_t q = 0;
+      bool apart = sg_hip_stream_queue(ctx, tried[n_tried], &q) == SG_OK && q != 0;
+      for (int k = 0; k < n_avoid; k++) apart = apart && q != avoid[k];
+      if (apart) found = tried[n_tried];
+    }
+    *shared = !found;
+    if (!found && n_tried) found = tried[0];
+    for (int i = 0; i < n_tried; i++)
+      if (tried[i] != found) (void)hipStreamDestroy(tried[i]);
+    return found;
+  }
+
   // Every request of the batch keeps a table of this engine's, all counted from one base that
   // lies at or below `ring`: the device can pull them.
   bool can_pull(P2pRpcRr *const *rrs, uint32_t n, const SgRingView &ring) const
@@ -279,7 +304,14 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
     device_id = _device_id;
     sg_hip_cfg cfg{sizeof(sg_hip_cfg), max_reqs, max_frames, 0, stream};
     ctx = sg_hip_create(device_id, &cfg);
-    sg_hip_cfg cfg_tx{sizeof(sg_hip_cfg), max_reqs, max_frames, 0, nullptr};  // the scatter side on a stream of its own
+    if (ctx) {
+      // the scatter side on a stream of its own, on another hardware queue than the gather's
+      OnDevice on(device_id);
+      uint64_t q_g = 0;
+      (void)sg_hip_stream_queue(ctx, nullptr, &q_g);
+      tx_stream = stream_apart(&q_g, 1, &tx_queue_shared);
+    }
+    sg_hip_cfg cfg_tx{sizeof(sg_hip_cfg), max_reqs, max_frames, 0, tx_stream};
     ctx_tx = ctx ? sg_hip_create(device_id, &cfg_tx) : nullptr;
     if (!ctx || !ctx_tx) {
       // nothing can be moved without the device: say so and stop, as checkCudaErrors did
@@ -306,6 +338,7 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
       }
     if (tables) (void)hipHostFree(tables);
     sg_hip_destroy(ctx_tx);
+    if (tx_stream) (void)hipStreamDestroy(tx_stream);
     sg_hip_destroy(ctx);
 #ifdef PROFILE_MODE
     PROF_PRINT("GatherBatch-host", GBatchHostNs);
@@ -334,10 +367,14 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
       tables = nullptr;
       return nullptr;
     }
-    if (hipStreamCreateWithFlags(&pack_stream, hipStreamNonBlocking) != hipSuccess) {
+    // the pull has to run BESIDE the copies: a stream on a hardware queue of its own
+    uint64_t q[2] = {0, 0};
+    (void)sg_hip_stream_queue(ctx, nullptr, &q[0]);
+    (void)sg_hip_stream_queue(ctx_tx, nullptr, &q[1]);
+    pack_stream = stream_apart(q, 2, &pack_queue_shared);
+    if (!pack_stream) {
       (void)hipHostFree(tables);
       tables = nullptr;
-      pack_stream = nullptr;
       return nullptr;
     }
     std::memset(tables, 0xff, sizeof(sg_frag_table) * (size_t)n);
@@ -504,6 +541,8 @@ class P2pRpcSgHipEngine : public P2pRpcSgEngine {
     a.n_frags = (uint32_t)n_frags;
     a.app = app;
     a.offsets_out = offsets_out_dev;
+    // (asking large calls to advance the cursor themselves, SG_F_SELF_ADVANCE, so that no kernel trails
+    // the call, was measured here: 125 -> 135 us per step of 512 requests in 220672 fragments)
     a.flags = flags | (rule_mtu && fixed_req_size ? SG_F_RULE_FRAGS : 0u);
     a.mtu = rule_mtu;
     a.fixed_req_size = fixed_req_size;

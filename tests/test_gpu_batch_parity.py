@@ -24,12 +24,23 @@ MODES = {
 }
 
 
+# the reference's own 64-byte p2p_rpc_hdr (src/p2p_rpc.h:10-17; lengths from a table, as from the
+# NIC) at the full size of the configurations the benchmark runs it on
+REF64_CASES = [(2, None), (1, None), (5, None), (3, None)]
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("cfg,n_req", REF64_CASES)
+def test_gather_scatter_bit_exact_with_the_reference_header(ctx, cfg, n_req, mode):
+    test_gather_scatter_bit_exact(ctx, cfg, n_req, mode, profile=synth.HDR_REF64)
+
+
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("cfg,n_req", CASES)
-def test_gather_scatter_bit_exact(ctx, cfg, n_req, mode):
+def test_gather_scatter_bit_exact(ctx, cfg, n_req, mode, profile=synth.HDR_BL58):
     fixed, rule, fuse = MODES[mode]["fixed"], MODES[mode]["rule"], MODES[mode]["fuse"]
-    w = synth.make_workload(cfg, n_req)
-    print(f"case cfg={cfg} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} mode={mode}",
+    w = synth.make_workload(cfg, n_req, profile=profile)
+    print(f"case cfg={cfg} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames} mode={mode} profile={profile}",
           flush=True)
     dw = DeviceWorkload(w)
     ctx.set_cursor(0, 0)
