@@ -387,14 +387,17 @@ int sg_hip_scatter_batch(sg_hip_ctx *ctx, const sg_scatter_args *args);
  * (src/splitrpc_server/p2p_rpc_dpdk_server.cc:117-150 and :158-189).  The
  * result is that of sg_hip_gather_batch(ctx, gather) followed by
  * sg_hip_scatter_batch(ctx, scatter).  Where both halves are single-kernel
- * calls of one wavefront per fragment that advance their cursors themselves
- * (SG_F_RULE_FRAGS gather and a scatter of one response size, fragments and
- * frames of at most 2016 bytes, no slot ring, no short-frame kernels of their
- * own) and neither touches the other's memory (the TX ring apart from the RX
- * ring, the response buffers apart from the request buffers), both travel in
- * ONE launch: a call of a batch or two costs more in launches than in bytes,
- * and this halves them.  Any other pair of calls is made as two calls, gather
- * first.  Synchronous unless both argument blocks carry SG_F_ASYNC. */
+ * calls on packed arenas whose kernels advance their cursors themselves
+ * (SG_F_RULE_FRAGS gather of fragments of at most 2016 bytes, short last
+ * fragments included; a scatter of one response size in frames of at most
+ * 2016 bytes, or of frames of at most 128 bytes without the full UDP
+ * checksum; no slot ring), the two together are no more wavefronts than the
+ * chip holds at once (8192), and neither touches the other's memory (the TX
+ * ring apart from the RX ring, the response buffers apart from the request
+ * buffers), both travel in ONE launch: a call of a batch or two costs more
+ * in launches than in bytes, and this halves them.  Any other pair of calls
+ * is made as two calls, gather first (larger calls are faster that way, on a
+ * stream each).  Synchronous unless both argument blocks carry SG_F_ASYNC. */
 int sg_hip_shunt_batch(sg_hip_ctx *ctx, const sg_gather_args *gather, const sg_scatter_args *scatter);
 
 /* Fragment tables the device reads where the receive thread writes them.

@@ -974,26 +974,6 @@ __global__ __launch_bounds__(kBlock) void k_scatter(ScatterArgs a)
   scatter_body<FULL_CSUM, FUSED, LONG, DEFER, ADV>(a, blockIdx.x, 0);
 }
 
-// One pass of the shunter's loop (src/splitrpc_server/p2p_rpc_dpdk_server.cc:117-189) in ONE
-// launch: the first s_blocks workgroups scatter the responses that are done (one response size),
-// the others gather the requests that became ready (declared rule), each half exactly as the
-// kernel of its own would.  For calls of a batch or two a launch costs more than the bytes it
-// moves; this halves the launches of a step.  Both halves advance their cursors themselves.
-// The scatter's wavefronts live longest (a header to fetch, rewrite and store besides the
-// payload) and are few: they are dispatched first so that they end with the others, not after.
-struct alignas(64) ShuntArgs {
-  GatherRuleArgs g;
-  ScatterArgs s;
-  uint32_t s_blocks;
-};
-
-template <bool FULL_CSUM>
-__global__ __launch_bounds__(kBlock) void k_shunt(ShuntArgs a)
-{
-  if (blockIdx.x >= a.s_blocks) gather_rule_body<false, 0, true>(a.g, blockIdx.x - a.s_blocks, offsetof(ShuntArgs, g));
-  else scatter_body<FULL_CSUM, true, false, false, true>(a.s, blockIdx.x, offsetof(ShuntArgs, s));
-}
-
 // Second phase of the full UDP checksum of long frames: one thread per frame
 // folds the sums its wavefronts left and writes the field (bytes 40, 41).
 // Frames that were not written (refused) carry no mark and are left alone;
@@ -1039,7 +1019,7 @@ __global__ __launch_bounds__(kBlock) void k_udp_finish(ScatterArgs a)
 // frames then go through k_scatter).  Addressing is per lane, the header is two
 // 16-bit words per lane, sums are row reductions.
 template <int L, bool FULL_CSUM, bool ADV>
-__device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_t wave)
+__device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_t wave, size_t kernarg_base = 0)
 {
   constexpr uint32_t G = kWave / L;
   // every argument of the common path in one burst of scalar loads (left to their first uses they
@@ -1103,7 +1083,7 @@ __device__ __forceinline__ void scatter_small_wave(const ScatterArgs &a, uint32_
   bool plain;
   if (last_only && a.n_plan) {
     // every group has the response's last frame: one plan entry for the wavefront
-    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(offsetof(ScatterArgs, plan))) + (per_req - 1));
+    const u32x8 fp = sload(reinterpret_cast<const u32x8 *>(kernarg_at(kernarg_base + offsetof(ScatterArgs, plan))) + (per_req - 1));
     from = reinterpret_cast<uint8_t *>(((uint64_t)fp[1] << 32 | fp[0]) + (uint64_t)r * fp[4]);
     plain = live && len != 0 && fp[7] == 0;
   } else {
@@ -1167,6 +1147,38 @@ template <int L, bool FULL_CSUM, bool ADV>
 __global__ __launch_bounds__(kBlock) void k_scatter_small(ScatterArgs a)
 {
   scatter_small_wave<L, FULL_CSUM, ADV>(a, blockIdx.x * kWavesPerBlock + threadIdx.x / kWave);
+}
+
+// One pass of the shunter's loop (src/splitrpc_server/p2p_rpc_dpdk_server.cc:117-189) in ONE
+// launch: the first s_blocks workgroups scatter the responses that are done (one response size),
+// the others gather the requests that became ready (declared rule), each half exactly as the
+// kernel of its own would.  Both halves advance their cursors themselves.  For calls that the chip
+// holds at once (a batch or two) a launch costs more than the bytes it moves; this halves the
+// launches of a step.  The scatter's wavefronts live longest (a header to fetch, rewrite and store
+// besides the payload) and are few: their workgroups come first, so that they end with the others,
+// not after.  (Larger calls lose by sharing a launch -- 8 resnet50-sized batches 30.2 -> 32.2 us
+// per step, 2048 lenet-sized ones 86.4 -> 96.9 us, wherever in the grid the scatter's workgroups
+// are put: first, or spread through the gather's in groups of eight, one per XCD -- and are made
+// as two calls on a stream each.)
+// G_SMALL: the gather's short last fragments go SMALL lanes each (gather_rule_body); S_SMALL: all
+// of the scatter's frames are short and go S_SMALL lanes each (scatter_small_wave).
+struct alignas(64) ShuntArgs {
+  GatherRuleArgs g;
+  ScatterArgs s;
+  uint32_t s_blocks;
+};
+
+template <int G_SMALL, int S_SMALL, bool FULL_CSUM>
+__global__ __launch_bounds__(kBlock) void k_shunt(ShuntArgs a)
+{
+  const uint32_t b = blockIdx.x;
+  if (b >= a.s_blocks) {
+    gather_rule_body<false, G_SMALL, true>(a.g, b - a.s_blocks, offsetof(ShuntArgs, g));
+  } else if (S_SMALL) {
+    scatter_small_wave<(S_SMALL ? S_SMALL : 8), FULL_CSUM, true>(a.s, b * kWavesPerBlock + threadIdx.x / kWave, offsetof(ShuntArgs, s));
+  } else {
+    scatter_body<FULL_CSUM, true, false, false, true>(a.s, b, offsetof(ShuntArgs, s));
+  }
 }
 
 // ---------------------------------------------------------------------------

@@ -39,6 +39,9 @@ SHARED = {
     "full-udp-checksum": lambda p: synth.make_custom([2800] * 33, [2799] * 33, seed=72, profile=p,
                                                      flags=synth.F_UDP_CSUM_FULL | synth.F_IPV4_CSUM),
     "one-request": lambda p: synth.make_custom([1400 * 9 + 1], [1400], seed=73, profile=p),
+    # short last fragments riding in the gather's half, eight short frames to a wavefront in the scatter's
+    "lenet-9": lambda p: synth.make_workload(1, 9, profile=p),
+    "lenet-1500": lambda p: synth.make_workload(1, 1500, profile=p),   # 6128 wavefronts: the most that shares
 }
 
 
@@ -48,7 +51,7 @@ def test_one_launch_moves_what_two_calls_move(name, profile):
     w = SHARED[name](profile)
     print(f"case shunt shared {name} profile={profile} n_req={w.n_req} frags={w.n_frags} frames={w.n_resp_frames}",
           flush=True)
-    ctx = SgContext(0)
+    ctx = SgContext(0, max_reqs=8192, max_frames=1 << 17)
     dw = DeviceWorkload(w)
     total = int(w.req_sizes.sum())
     cap = 2 * total + 4096 + 10  # no whole number of batches fills the arena: the third call wraps
@@ -83,10 +86,13 @@ def test_one_launch_moves_what_two_calls_move(name, profile):
 APART = {
     # (workload, why the two calls keep kernels of their own)
     "jumbo": lambda: synth.make_workload(5, 1),                     # frames of several wavefronts
-    "lenet": lambda: synth.make_workload(1, 9),                     # short frames, several to a wavefront
+    "short-frames-16-lanes": lambda: synth.make_custom([300] * 50, [300] * 50, seed=78),  # short frames, 16 lanes each
     "bert": lambda: synth.make_workload(3, 20),                     # tensors; short last fragments
     "mixed-echo": lambda: synth.make_workload(4, 50),               # variable sizes, answered in place
     "sizes-differ": lambda: synth.make_custom([4200] * 12, [100 + 333 * k for k in range(12)], seed=74),
+    # more wavefronts than the chip holds at once: faster as two calls
+    "lenet-4096": lambda: synth.make_workload(1, 4096),
+    "two-frames-3000": lambda: synth.make_custom([4200] * 3000, [2800] * 3000, seed=77, flags=synth.F_UDP_CSUM_PSEUDO),
 }
 
 
