@@ -719,8 +719,10 @@ def main() -> int:
 
     def contexts(wl, b):
         mr, mf = max(4096, wl.n_req * b), max(65536, max(wl.n_frags, wl.n_resp_frames) * b)
-        # gather and scatter each on a context (and stream) of their own, unless one stream is asked for
-        return SgContext(0, max_reqs=mr, max_frames=mf), (None if a.one_stream else SgContext(0, max_reqs=mr, max_frames=mf))
+        # gather and scatter each on a context (and stream) of their own, unless one stream is asked for; the
+        # second stream on another hardware queue than the first, or the two would never run side by side
+        c0 = SgContext(0, max_reqs=mr, max_frames=mf)
+        return c0, (None if a.one_stream else SgContext.apart_from([c0], 0, max_reqs=mr, max_frames=mf))
 
     ctx, ctx_tx = contexts(w, bpl)
     _log(f"staging {w.name} x {bpl} batches per launch")
@@ -870,7 +872,9 @@ def main() -> int:
                    "kernel_us": round(ks["k_gather"][0] * 1e3, 3),
                    "kernel_frac_of_hbm_peak": round(b1 / (ks["k_gather"][0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
                    if ks["k_gather"][0] > 0 else None}
-            more = [SgContext(0, max_reqs=4096, max_frames=65536) for _ in range(3)]
+            more = []
+            for _ in range(3):
+                more.append(SgContext.apart_from([ctx] + more, 0, max_reqs=4096, max_frames=65536))
             n_native = max(a.steps, 400)
             for n_ctx in (1, 2, 4):
                 one[f"native_loop_{n_ctx}_stream{'s' if n_ctx > 1 else ''}"] = fig(

@@ -116,6 +116,35 @@ class SgContext:
     def sync(self) -> None:
         self._check(self.lib.sg_hip_sync(self.h))
 
+    def stream_queue(self, stream: Optional[int] = None) -> int:
+        """Address of the hardware queue the context's stream (or ``stream``)
+        dispatches to: streams that share one run their kernels one after the
+        other."""
+        q = C.c_uint64(0)
+        self._check(self.lib.sg_hip_stream_queue(self.h, C.c_void_p(stream) if stream else None, C.byref(q)))
+        return int(q.value)
+
+    @classmethod
+    def apart_from(cls, others: Sequence["SgContext"], device: int = 0, **kw) -> "SgContext":
+        """A context whose stream dispatches to another hardware queue than
+        those of ``others`` (the runtime deals its few hardware queues out to
+        streams in turns, so two contexts made at different times may share
+        one, and calls queued to them then never overlap).  Falls back to the
+        last one made."""
+        taken = {o.stream_queue() for o in others}
+        spare, found = [], None
+        for _ in range(8):
+            c = cls(device, **kw)
+            if c.stream_queue() not in taken:
+                found = c
+                break
+            spare.append(c)
+        if found is None:
+            found = spare.pop()
+        for c in spare:
+            c.close()
+        return found
+
     def set_cursor(self, which: int, value: int) -> None:
         self._check(self.lib.sg_hip_set_cursor(self.h, which, value))
 
