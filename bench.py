@@ -584,8 +584,8 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
             continue
         bound = min(burst // per + 2, dw.n_req)           # requests one burst can complete
         mf = max(65536, bound * per, burst)
-        ctx_ra = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=mf)
         ctx_sg = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=mf)
+        ctx_ra = SgContext.apart_from([ctx_sg], 0, max_reqs=max(4096, dw.n_req), max_frames=mf)  # another hardware queue
         i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
         # reassembly output, twice: while the copy reads one set the next burst fills the other
         sets = [dict(fs=i32(mf), fl=i32(mf), rf=i32(4097 + dw.n_req), hdr=i32(4096 + dw.n_req), counts=i32(4))
