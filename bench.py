@@ -36,14 +36,38 @@ HBM_PEAK_GBS = 8000.0
 # bert's scatter is both of its kernels (full frames + short remainder frames), jumbo's the copy
 # phase without the 1.9 MB of the checksum-finishing kernel.
 MEASURED_TRAFFIC = {
-    (2, 32, "k_gather"): 653.6e6, (2, 32, "k_scatter"): 4.7e6,
-    (1, 2048, "k_gather"): 450.5e6, (1, 2048, "k_scatter"): 22.5e6,
-    (3, 512, "k_gather"): 585.7e6, (3, 512, "k_scatter"): 934.7e6,
-    (4, 8, "k_gather"): 661.9e6, (4, 8, "k_scatter"): 676.0e6,
-    (5, 4, "k_gather"): 817.6e6, (5, 4, "k_scatter"): 549.3e6,
+    (2, 32, "k_gather"): 653.3e6, (2, 32, "k_scatter"): 4.8e6,
+    (1, 2048, "k_gather"): 450.1e6, (1, 2048, "k_scatter"): 22.4e6,
+    (3, 512, "k_gather"): 586.8e6, (3, 512, "k_scatter"): 934.9e6,
+    (4, 8, "k_gather"): 661.3e6, (4, 8, "k_scatter"): 675.9e6,
+    (5, 4, "k_gather"): 818.0e6, (5, 4, "k_scatter"): 548.6e6,
 }
 # the same for the reference's own 64-byte header (bench.py --ref64)
 MEASURED_TRAFFIC_REF64 = {(2, 32, "k_gather"): 655.5e6, (2, 32, "k_scatter"): 4.8e6}
+# The kernel sources those counter runs were made with (SHA-256).  A change to either file may change
+# what the kernels move: `roofline.traffic` is then reported as null until the two counter passes have
+# been run again and the figures above and these digests brought up to date (a CPU test holds them
+# against the tree).
+TRAFFIC_MEASURED_WITH = {
+    "splitrpc_amd/csrc/sg_kernels_copy.h": "526d7000c8e7758c4accd6f38c4db3fcdb20738a7c8dbdd92c6877a1758de5f8",
+    "splitrpc_amd/csrc/sg_device.h": "2e221986fd3ad868a696eb88ddc07a195d82b2e5b0fd4799e904894cc08aca4c",
+}
+
+
+def traffic_is_current() -> bool:
+    """Whether the kernel sources are the ones MEASURED_TRAFFIC was measured with."""
+    import hashlib
+    here = os.path.dirname(os.path.abspath(__file__))
+    for rel, digest in TRAFFIC_MEASURED_WITH.items():
+        try:
+            with open(os.path.join(here, rel), "rb") as f:
+                if hashlib.sha256(f.read()).hexdigest() != digest:
+                    return False
+        except OSError:
+            return False
+    return True
+
+
 WORKLOAD_NAMES = {1: "lenet", 2: "resnet50", 3: "bert", 4: "mixed", 5: "jumbo"}
 
 
@@ -577,12 +601,19 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
     per, per_resp = -(-size // w.mtu), -(-rsize // w.mtu)
     n_arr = int(dw.arrivals.numel())
     out = {"arrivals_per_call": n_arr, "requests_per_call": dw.n_req, "calls": calls}
+    # position in the arrival stream of every request's last fragment (the batch's order, tiled over the call)
+    at = np.empty(w.n_slots, np.int64)
+    at[w.arrivals] = np.arange(w.n_frags)
+    last = np.array([at[w.frag_slot[int(w.req_first[r]):int(w.req_first[r + 1])]].max() for r in range(w.n_req)])
+    done_at = np.concatenate([last + i * w.n_frags for i in range(n_arr // w.n_frags)])
     total_bytes = (pool.gather_bytes + pool.scatter_bytes) * calls
     for burst in bursts:
         burst = burst or n_arr
         if burst > n_arr:
             continue
-        bound = min(burst // per + 2, dw.n_req)           # requests one burst can complete
+        # requests a burst can complete: a request is complete with its last arrival, and arrival
+        # orders that interleave the requests of a batch complete many of them within one burst
+        bound = int(np.bincount(done_at // burst).max())
         mf = max(65536, bound * per, burst)
         ctx_sg = SgContext(0, max_reqs=max(4096, dw.n_req), max_frames=mf)
         ctx_ra = SgContext.apart_from([ctx_sg], 0, max_reqs=max(4096, dw.n_req), max_frames=mf)  # another hardware queue
@@ -758,7 +789,7 @@ def main() -> int:
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     b2b = back_to_back(ctx, pool, dom, min(a.steps, 100))
     # the counters were read with the default kernels and headers only
-    traffic_known = not (a.general or a.ref64 or a.no_small or a.no_remap)
+    traffic_known = not (a.general or a.ref64 or a.no_small or a.no_remap) and traffic_is_current()
     headline_roofs = roofline_of(pool, kt, traffic_known)
 
     _log("kernel times and back-to-back done; reassembly")
@@ -1012,7 +1043,9 @@ def main() -> int:
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((a.workload, bpl, dom)) if traffic_known else None,
-                     "traffic_unit": "HBM bytes per launch (rocprofv3 --pmc, see profiles/)",
+                     "traffic_unit": "HBM bytes per launch (rocprofv3 --pmc, see profiles/)"
+                                     if traffic_is_current() else
+                                     "null: the kernel sources have changed since the counter runs (TRAFFIC_MEASURED_WITH)",
                      "bytes_per_launch": dom_bytes, "avg_kernel_us": round(dom_ms * 1e3, 3),
                      # the same call launched back to back, two events around the burst (all of the
                      # call's kernels and the gaps between launches, no per-launch event)

@@ -172,6 +172,16 @@ def test_bench_has_measured_traffic_for_every_default_call():
             assert bench.MEASURED_TRAFFIC[(cfg, bpl, kernel)] > 0
 
 
+def test_measured_traffic_belongs_to_the_kernel_sources_in_the_tree():
+    """The traffic figures are counter readings of particular kernels: after a
+    change to the kernel sources they have to be taken again (the commands
+    head profiles/copy_kernels_all_workloads_traffic_time_instructions.txt),
+    and bench.MEASURED_TRAFFIC / TRAFFIC_MEASURED_WITH updated with them.
+    Until then the bench line reports `traffic` as null."""
+    import bench
+    assert bench.traffic_is_current(), "kernel sources changed since roofline.traffic was measured"
+
+
 def test_client_patterns_and_checks_through_the_cpu_path():
     """The reference clients' request patterns and reply checks
     (lib_loadgen/echo_client.cc, vec_add_client.cc) around the oracle's gather
