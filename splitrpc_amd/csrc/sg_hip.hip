@@ -1363,7 +1363,7 @@ int sg_hip_pack_tables(sg_hip_ctx *c, const sg_pack_args *a)
     p.blob_dst = a->blob_dst;
     p.blob_words = a->blob_words;
     const uint32_t blocks = (a->blob_words + 4 * kBlock - 1) / (4 * kBlock);
-    k_pack_tables<64><<<blocks > 256 ? 256u : blocks, kBlock, 0, a->stream ? static_cast<hipStream_t>(a->stream) : c->stream>>>(p);
+    k_pack_tables<16><<<blocks > 256 ? 256u : blocks, kBlock, 0, a->stream ? static_cast<hipStream_t>(a->stream) : c->stream>>>(p);
     HIP_TRY(c, hipGetLastError());
     return SG_OK;
   }
@@ -1395,16 +1395,15 @@ int sg_hip_pack_tables(sg_hip_ctx *c, const sg_pack_args *a)
   p.blob_dst = a->blob_dst;
   p.blob_words = a->blob_words;
   hipStream_t st = a->stream ? static_cast<hipStream_t>(a->stream) : c->stream;
-  // lanes per request by the average number of fragments (a lane takes four entries per step).  A
-  // wavefront per request even for the longest tables: the pull is bound by the bus, and the fewer
-  // wavefronts wait on it, the more slots are left to the copy kernel that runs beside it.
-  const uint32_t avg = a->n_frags / a->n_req;
-  const uint32_t lanes = avg <= 32 ? 16u : 64u;
+  // Sixteen lanes per request, whatever the tables' length: the pull is bound by the bus either way
+  // (512 tables of 431 entries: 21 us with 16 or with 64 lanes each), but reads across the bus that
+  // are in flight hold up the memory traffic of a copy kernel running beside them -- a gather of
+  // 104 us took 114 us beside a pull with 64 lanes per request and 106 us beside one with 16.
+  constexpr uint32_t lanes = 16;
   p.req_blocks = (a->n_req + kBlock / lanes - 1) / (kBlock / lanes);
   const uint32_t copy_blocks = a->blob_words ? (a->blob_words + 4 * kBlock - 1) / (4 * kBlock) : 0u;
   const uint32_t grid = p.req_blocks + (copy_blocks > 64 ? 64u : copy_blocks);
-  if (lanes == 16) k_pack_tables<16><<<grid, kBlock, 0, st>>>(p);
-  else k_pack_tables<64><<<grid, kBlock, 0, st>>>(p);
+  k_pack_tables<lanes><<<grid, kBlock, 0, st>>>(p);
   HIP_TRY(c, hipGetLastError());
   return SG_OK;
 }
