@@ -568,7 +568,8 @@ def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, 
     return dt
 
 
-def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 65536, 0)) -> dict:
+def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 65536, 0), n_queues: int = 4,
+                    queues_up_to: int = 65536) -> dict:
     """The receive path end to end on the device, burst after burst and no
     host wait in between, from a native loop (sgh_pipeline_loop_gpu of
     libsg_host.so): sg_hip_reassemble files a burst's arrivals (requests that
@@ -582,7 +583,9 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
       one_stream   the calls of a burst one after the other on one context
       overlapped   the reassembly on a context (stream) of its own, its output
                    tables double-buffered, events between the two streams: burst
-                   k + 1 is filed while burst k is gathered and answered"""
+                   k + 1 is filed while burst k is gathered and answered
+      N_queues     (bursts of up to `queues_up_to` arrivals) N receive queues side
+                   by side, each a one_stream pipeline of its own (_pipeline_queues)"""
     import ctypes as C
     import numpy as np
     import torch
@@ -594,9 +597,15 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
     host = _host_lib()
     host.sgh_pipeline_loop_gpu.restype = C.c_double
     host.sgh_pipeline_loop_gpu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
+    host.sgh_pipeline_queues_gpu.restype = C.c_double
+    host.sgh_pipeline_queues_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]
     dev = "cuda:0"
     items = pool.items
     dw = items[0]
+    # ring copies for the queues of the side-by-side form: no two queues on one copy at a time
+    from splitrpc_amd.engine import DeviceWorkload
+    items_q = list(items) + [DeviceWorkload(w, copies=pool.bpl, unique_tokens=True)
+                             for _ in range(max(0, n_queues - len(items)))]
     size, rsize = int(w.req_sizes[0]), int(w.resp_sizes[0])
     per, per_resp = -(-size // w.mtu), -(-rsize // w.mtu)
     n_arr = int(dw.arrivals.numel())
@@ -678,7 +687,89 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
         ctx_sg.close()
         del sets, req_arena, resp_arena, tx_ring, gas, sas, ras, by_item
         torch.cuda.empty_cache()
+        if burst <= queues_up_to:
+            res[f"{n_queues}_queues"] = _pipeline_queues(host, pool, items_q, n_queues, calls, burst, bound, mf, size,
+                                                         rsize, per, per_resp, n_arr, total_bytes)
     return out
+
+
+def _pipeline_queues(host, pool, items, n_queues, calls, burst, bound, mf, size, rsize, per, per_resp, n_arr,
+                     total_bytes) -> dict:
+    """`n_queues` receive queues side by side, each the one-stream pipeline of
+    device_pipeline with a context (stream on a hardware queue of its own where
+    one is to be had, reassembly table, cursors), tables, arenas and TX ring of
+    its own, each fed `calls` calls' worth of arrivals from ring copies no other
+    queue is on at the time (sgh_pipeline_queues_gpu: one thread queues burst k
+    of every queue, then burst k + 1).  Wall time over all queues' arrivals."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from splitrpc_amd import capi
+    from splitrpc_amd.engine import AppRef, RingRef, SgContext, to_dev
+    w = pool.w
+    dev = "cuda:0"
+    dw = items[0]
+    A = capi.F_ASYNC
+    i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
+    ctxs, keep, ras, gas, sas = [], [], [], [], []
+    for q in range(n_queues):
+        kw = dict(max_reqs=max(4096, dw.n_req), max_frames=mf)
+        ctx = SgContext.apart_from(ctxs, 0, **kw) if ctxs else SgContext(0, **kw)
+        ctxs.append(ctx)
+        t = dict(fs=i32(mf), fl=i32(mf), rf=i32(4097 + dw.n_req), hdr=i32(4096 + dw.n_req), counts=i32(4))
+        req_cap, resp_cap = 4 * bound * size, 4 * bound * rsize
+        req_arena = torch.zeros(req_cap, dtype=torch.uint8, device=dev)
+        resp_arena = torch.zeros(resp_cap, dtype=torch.uint8, device=dev)
+        tx_ring = torch.zeros(bound * per_resp * w.slot_size, dtype=torch.uint8, device=dev)
+        tx = RingRef(tx_ring, bound * per_resp, w.slot_size, w.profile)
+        tx_slot = to_dev(np.arange(bound * per_resp, dtype=np.uint32), dev)
+        resp_first = to_dev((np.arange(bound + 1) * per_resp).astype(np.uint32), dev)
+        keep.append((t, req_arena, resp_arena, tx_ring, tx_slot, resp_first))
+        by_item = {}
+        for call in range(calls):
+            k = (call + q) % len(items)
+            it = items[k]
+            if k not in by_item:
+                by_item[k] = (
+                    ctx.gather_args(it.rx, t["fs"], None, t["rf"], bound, bound * per,
+                                    AppRef(arena=req_arena, cap=req_cap), None, flags=A | capi.F_RULE_FRAGS,
+                                    fixed_req_size=size, mtu=w.mtu, counts=t["counts"]),
+                    ctx.scatter_args(it.rx, tx, tx_slot, None, resp_first, None, rsize, bound, bound * per_resp,
+                                     w.mtu, AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A,
+                                     hdr_src_req=t["hdr"], counts=t["counts"]))
+            for b in range(0, n_arr, burst):
+                ras.append(ctx.reassemble_args(it.rx, it.arrivals[b:b + burst], min(burst, n_arr - b), t["fs"], t["fl"],
+                                               t["rf"], req_hdr_slot=t["hdr"], counts_out=t["counts"], flags=A))
+                gas.append(by_item[k][0])
+                sas.append(by_item[k][1])
+    n_bursts = len(ras) // n_queues
+    arr = lambda xs: (C.c_void_p * len(xs))(*[C.addressof(x) for x in xs])
+    c_ctx = (C.c_void_p * n_queues)(*[c.h for c in ctxs])
+    c_ras, c_gas, c_sas = arr(ras), arr(gas), arr(sas)
+    best = None
+    for rep in range(3):
+        for c in ctxs:
+            c.reassemble_reset()
+        torch.cuda.synchronize()
+        dt = host.sgh_pipeline_queues_gpu(c_ctx, n_queues, c_ras, c_gas, c_sas, n_bursts)
+        if dt < 0:
+            raise RuntimeError(f"sgh_pipeline_queues_gpu failed: {dt} {[c.lib.sg_hip_last_error(c.h) for c in ctxs]}")
+        best = dt if best is None else min(best, dt)
+    left = sum(int(k[0]["counts"].cpu()[3]) for k in keep)
+    hw = len(set(c.stream_queue() for c in ctxs))
+    res = {"hardware_queues": hw,
+           "us_per_burst": round(best / (n_bursts * n_queues) * 1e6, 2),
+           "arrivals_per_sec": round(n_arr * calls * n_queues / best, 1),
+           "requests_per_sec": round(dw.n_req * calls * n_queues / best, 1),
+           "payload_Gbit_per_sec": round(8.0 * size * dw.n_req * calls * n_queues / best / 1e9, 1),
+           "GBps": round(total_bytes * n_queues / best / 1e9, 1),
+           "frac_of_hbm_peak": round(total_bytes * n_queues / best / 1e9 / HBM_PEAK_GBS, 4),
+           "requests_left_in_flight": left}
+    for c in ctxs:
+        c.close()
+    del keep, ras, gas, sas
+    torch.cuda.empty_cache()
+    return res
 
 
 def roofline_of(pool: Pool, kt, traffic_known: bool = True) -> dict:

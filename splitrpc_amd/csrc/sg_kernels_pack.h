@@ -30,7 +30,8 @@ struct PackArgs {
   uint32_t req_blocks;  // workgroups that pull tables; the ones behind them copy the blob
 };
 
-// L lanes per request (a request of a few fragments does not fill a workgroup).
+// L lanes per request, each taking four entries per step (the host launches L = 16 whatever the
+// tables' length: what a pull costs the copy kernel beside it grows with the bus reads in flight).
 // An entry that is no payload start of the ring becomes slot 0xffffffff, which
 // the gather and scatter kernels refuse.
 template <int L>

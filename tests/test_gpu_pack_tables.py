@@ -36,11 +36,11 @@ def _tables_of(w, dw, pkt_base, order, n_tables):
                                           ("ragged", synth.HDR_BL58), ("medium", synth.HDR_BL58)])
 def test_pulled_tables_equal_the_tables_a_host_walk_makes(name, profile, where):
     if name == "lenet":
-        w = synth.make_workload(1, 40, profile=profile)      # 3 fragments per request: 16 lanes each
+        w = synth.make_workload(1, 40, profile=profile)      # 3 fragments per request: one step of a group's lanes
     elif name == "resnet50":
-        w = synth.make_workload(2, 3, profile=profile)       # 431 fragments: a workgroup each
+        w = synth.make_workload(2, 3, profile=profile)       # 431 fragments: seven steps of sixteen lanes
     elif name == "medium":
-        w = synth.make_custom([1400 * 40 + 7] * 9, [64] * 9, seed=81, profile=profile)  # 41: a wavefront each
+        w = synth.make_custom([1400 * 40 + 7] * 9, [64] * 9, seed=81, profile=profile)  # 41: one step
     else:
         rng = np.random.default_rng(8)
         w = synth.make_custom([int(x) for x in rng.integers(0, 60000, 37)], [64] * 37, seed=82, profile=profile)

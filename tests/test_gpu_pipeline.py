@@ -482,3 +482,96 @@ def test_reassembly_on_a_stream_of_its_own_beside_the_copy(burst):
     assert ctx_sg.get_cursor(0) == cur0 and ctx_sg.get_cursor(1) == cur1
     ctx_ra.close()
     ctx_sg.close()
+
+
+def test_receive_queues_side_by_side_from_a_native_loop():
+    """Three receive queues, each with a context (stream, reassembly table,
+    cursors), rings and tables of its own, every queue's bursts filed,
+    gathered and answered from one native loop with no host wait
+    (sgh_pipeline_queues_gpu of libsg_host.so): each queue's request arena,
+    TX ring and cursors against the oracle's reassembly, gather and scatter
+    replayed burst by burst."""
+    import ctypes as C
+    from splitrpc_amd import build
+    host = C.CDLL(build.HOST_LIB)
+    host.sgh_pipeline_queues_gpu.restype = C.c_double
+    host.sgh_pipeline_queues_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]
+    n_queues, burst, n_reqs, resp_size = 3, 16, 30, 3000
+    per_req, A = 3, capi.F_ASYNC
+    queues = []
+    for q in range(n_queues):
+        w = synth.make_custom([4200] * n_reqs, [resp_size] * n_reqs, seed=70 + q,
+                              flags=synth.F_UDP_CSUM_PSEUDO | synth.F_IPV4_CSUM)
+        order = np.random.default_rng(20 + q).permutation(w.arrivals)
+        per_resp = synth.num_frames(resp_size, w.mtu)
+        ctx = SgContext(0, max_reqs=64, max_frames=4096)
+        ctx.reassemble_reset()
+        t = Tables(64, 4096)
+        rx = RingRef(torch.from_numpy(w.ring).to(DEV), w.n_slots, w.slot_size, w.profile)
+        bound = min(burst, n_reqs)
+        tx_slots = np.random.default_rng(30 + q).permutation(bound * per_resp).astype(np.uint32)
+        tx_init = np.random.default_rng(40 + q).integers(0, 256, bound * per_resp * w.slot_size, dtype=np.uint8)
+        tx_ring = torch.from_numpy(tx_init).to(DEV)
+        tx = RingRef(tx_ring, bound * per_resp, w.slot_size, w.profile)
+        req_cap, resp_cap = n_reqs * 4200 + 100 + q, 7 * resp_size + 50
+        req_arena = torch.zeros(req_cap, dtype=torch.uint8, device=DEV)
+        resp_np = np.random.default_rng(50 + q).integers(0, 256, resp_cap, dtype=np.uint8)
+        resp_arena = torch.from_numpy(resp_np).to(DEV)
+        arr = to_dev(np.ascontiguousarray(order, np.uint32), DEV)
+        tx_slot_dev = to_dev(tx_slots, DEV)
+        resp_first = to_dev((np.arange(bound + 1) * per_resp).astype(np.uint32), DEV)
+        ga = ctx.gather_args(rx, t.fs, None, t.rf, bound, bound * per_req, AppRef(arena=req_arena, cap=req_cap), None,
+                             flags=A | capi.F_RULE_FRAGS, fixed_req_size=4200, mtu=w.mtu, counts=t.counts)
+        sa = ctx.scatter_args(rx, tx, tx_slot_dev, None, resp_first, None, resp_size, bound, bound * per_resp, w.mtu,
+                              AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A, hdr_src_req=t.hdr,
+                              counts=t.counts)
+        ras = [ctx.reassemble_args(rx, arr[b:b + burst], min(burst, len(order) - b), t.fs, t.fl, t.rf, t.tok,
+                                   req_hdr_slot=t.hdr, counts_out=t.counts, flags=A)
+               for b in range(0, len(order), burst)]
+        start = req_cap - 5000 - 100 * q
+        ctx.set_cursor(0, start)
+        ctx.set_cursor(1, 0)
+        queues.append(dict(w=w, order=order, ctx=ctx, t=t, rx=rx, tx_slots=tx_slots, tx_init=tx_init, tx_ring=tx_ring,
+                           tx=tx, req_cap=req_cap, resp_cap=resp_cap, req_arena=req_arena, resp_np=resp_np,
+                           resp_arena=resp_arena, arr=arr, keep=(tx_slot_dev, resp_first), ga=ga, sa=sa, ras=ras,
+                           start=start, bound=bound, per_resp=per_resp))
+    n_bursts = len(queues[0]["ras"])
+    assert all(len(q["ras"]) == n_bursts for q in queues)
+    ptrs = lambda xs: (C.c_void_p * len(xs))(*[C.addressof(x) for x in xs])
+    c_ctx = (C.c_void_p * n_queues)(*[q["ctx"].h for q in queues])
+    c_ras = ptrs([ra for q in queues for ra in q["ras"]])
+    c_ga = ptrs([q["ga"] for q in queues for _ in range(n_bursts)])
+    c_sa = ptrs([q["sa"] for q in queues for _ in range(n_bursts)])
+    torch.cuda.synchronize()
+    print(f"case queues={n_queues} bursts={n_bursts} of {burst}", flush=True)
+    dt = host.sgh_pipeline_queues_gpu(c_ctx, n_queues, c_ras, c_ga, c_sa, n_bursts)
+    assert dt > 0, (dt, [q["ctx"].lib.sg_hip_last_error(q["ctx"].h) for q in queues])
+    torch.cuda.synchronize()
+    for qi, q in enumerate(queues):
+        w, order = q["w"], q["order"]
+        efs, efl, erf, _ = oracle.reassemble(w, arrivals=order)
+        slot_req = {int(s): r for r in range(n_reqs) for s in efs[erf[r]:erf[r + 1]]}
+        want_req = np.zeros(q["req_cap"], np.uint8)
+        want_tx = q["tx_init"].copy()
+        cur0, cur1, done = q["start"], 0, 0
+        pos_done = np.zeros(n_reqs, int)
+        for b in range(0, len(order), burst):
+            for sl in order[b:b + burst]:
+                pos_done[slot_req[int(sl)]] += 1
+            now = int((pos_done == per_req).sum())
+            if now > done:
+                r0, r1 = done, now
+                sub = _sub(w, efs[erf[r0]:erf[r1]], efl[erf[r0]:erf[r1]], erf[r0:r1 + 1] - erf[r0], None,
+                           q["tx_slots"], efs[erf[r0:r1]], resp_size)
+                want_req, _, cur0 = oracle.gather(sub, arena_cap=q["req_cap"], cursor=cur0, out=want_req)
+                sub.tx_n_slots = q["bound"] * q["per_resp"]
+                _, cur1 = oracle.scatter(sub, w.ring, want_tx, q["resp_np"], arena_cap=q["resp_cap"], cursor=cur1)
+            done = now
+        assert done == n_reqs
+        got = q["req_arena"].cpu().numpy()
+        assert np.array_equal(got, want_req), (qi, first_diff(got, want_req))
+        got = q["tx_ring"].cpu().numpy()
+        assert np.array_equal(got, want_tx), (qi, first_diff(got, want_tx))
+        assert q["ctx"].get_cursor(0) == cur0 and q["ctx"].get_cursor(1) == cur1, qi
+    for q in queues:
+        q["ctx"].close()
