@@ -598,7 +598,8 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
     host.sgh_pipeline_loop_gpu.restype = C.c_double
     host.sgh_pipeline_loop_gpu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
     host.sgh_pipeline_queues_gpu.restype = C.c_double
-    host.sgh_pipeline_queues_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]
+    host.sgh_pipeline_queues_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
+                                             C.c_int]
     dev = "cuda:0"
     items = pool.items
     dw = items[0]
@@ -700,7 +701,8 @@ def _pipeline_queues(host, pool, items, n_queues, calls, burst, bound, mf, size,
     one is to be had, reassembly table, cursors), tables, arenas and TX ring of
     its own, each fed `calls` calls' worth of arrivals from ring copies no other
     queue is on at the time (sgh_pipeline_queues_gpu: one thread queues burst k
-    of every queue, then burst k + 1).  Wall time over all queues' arrivals."""
+    of every queue, then burst k + 1; or a thread per queue).  Wall time over
+    all queues' arrivals."""
     import ctypes as C
     import numpy as np
     import torch
@@ -746,25 +748,26 @@ def _pipeline_queues(host, pool, items, n_queues, calls, burst, bound, mf, size,
     arr = lambda xs: (C.c_void_p * len(xs))(*[C.addressof(x) for x in xs])
     c_ctx = (C.c_void_p * n_queues)(*[c.h for c in ctxs])
     c_ras, c_gas, c_sas = arr(ras), arr(gas), arr(sas)
-    best = None
-    for rep in range(3):
-        for c in ctxs:
-            c.reassemble_reset()
-        torch.cuda.synchronize()
-        dt = host.sgh_pipeline_queues_gpu(c_ctx, n_queues, c_ras, c_gas, c_sas, n_bursts)
-        if dt < 0:
-            raise RuntimeError(f"sgh_pipeline_queues_gpu failed: {dt} {[c.lib.sg_hip_last_error(c.h) for c in ctxs]}")
-        best = dt if best is None else min(best, dt)
-    left = sum(int(k[0]["counts"].cpu()[3]) for k in keep)
     hw = len(set(c.stream_queue() for c in ctxs))
-    res = {"hardware_queues": hw,
-           "us_per_burst": round(best / (n_bursts * n_queues) * 1e6, 2),
-           "arrivals_per_sec": round(n_arr * calls * n_queues / best, 1),
-           "requests_per_sec": round(dw.n_req * calls * n_queues / best, 1),
-           "payload_Gbit_per_sec": round(8.0 * size * dw.n_req * calls * n_queues / best / 1e9, 1),
-           "GBps": round(total_bytes * n_queues / best / 1e9, 1),
-           "frac_of_hbm_peak": round(total_bytes * n_queues / best / 1e9 / HBM_PEAK_GBS, 4),
-           "requests_left_in_flight": left}
+    res = {"hardware_queues": hw}
+    for form, threaded in (("one_thread", 0), ("thread_per_queue", 1)):
+        best = None
+        for rep in range(3):
+            for c in ctxs:
+                c.reassemble_reset()
+            torch.cuda.synchronize()
+            dt = host.sgh_pipeline_queues_gpu(c_ctx, n_queues, c_ras, c_gas, c_sas, n_bursts, threaded)
+            if dt < 0:
+                raise RuntimeError(f"sgh_pipeline_queues_gpu failed: {dt} {[c.lib.sg_hip_last_error(c.h) for c in ctxs]}")
+            best = dt if best is None else min(best, dt)
+        left = sum(int(k[0]["counts"].cpu()[3]) for k in keep)
+        res[form] = {"us_per_burst": round(best / (n_bursts * n_queues) * 1e6, 2),
+                     "arrivals_per_sec": round(n_arr * calls * n_queues / best, 1),
+                     "requests_per_sec": round(dw.n_req * calls * n_queues / best, 1),
+                     "payload_Gbit_per_sec": round(8.0 * size * dw.n_req * calls * n_queues / best / 1e9, 1),
+                     "GBps": round(total_bytes * n_queues / best / 1e9, 1),
+                     "frac_of_hbm_peak": round(total_bytes * n_queues / best / 1e9 / HBM_PEAK_GBS, 4),
+                     "requests_left_in_flight": left}
     for c in ctxs:
         c.close()
     del keep, ras, gas, sas

@@ -721,30 +721,48 @@ double sgh_pipeline_loop_gpu(sg_hip_ctx *ra, sg_hip_ctx *sg, const sg_reassemble
 
 // Several receive queues side by side, each with a context (stream, reassembly table, cursors) of
 // its own, as a NIC spreads flows over its RX queues and the reference keeps an rr pool per queue:
-// burst k of every queue is filed and its completed requests gathered and answered
-// (sg_hip_reassemble + sg_hip_shunt_batch on the queue's context) before burst k + 1 of any queue,
-// all from this one thread and without a host wait.  ras / ga / sa hold n_queues * n_bursts entries,
-// queue q's burst k at [q * n_bursts + k].  Small bursts are a chain of short dependent launches
-// per queue; the queues' chains run beside each other on the device.  Returns the seconds the loop
-// took, every context drained, or a negative error code.
+// every burst of a queue is filed and its completed requests gathered and answered
+// (sg_hip_reassemble + sg_hip_shunt_batch on the queue's context), without a host wait.  ras / ga /
+// sa hold n_queues * n_bursts entries, queue q's burst k at [q * n_bursts + k].  Small bursts are a
+// chain of short dependent launches per queue; the queues' chains run beside each other on the
+// device.  threaded == 0: this thread queues burst k of every queue before burst k + 1 of any;
+// else a thread per queue, as the reference runs a shunter thread per transport.  Returns the
+// seconds the loop took, every context drained, or a negative error code.
 double sgh_pipeline_queues_gpu(sg_hip_ctx *const *ctxs, uint32_t n_queues, const sg_reassemble_args *const *ras,
-                               const sg_gather_args *const *ga, const sg_scatter_args *const *sa, uint32_t n_bursts)
+                               const sg_gather_args *const *ga, const sg_scatter_args *const *sa, uint32_t n_bursts,
+                               int threaded)
 {
   if (!ctxs || !ras || !ga || !sa || n_queues == 0) return (double)SG_E_INVAL;
   int rc = SG_OK;
   for (uint32_t q = 0; q < n_queues && rc == SG_OK; q++) rc = ctxs[q] ? sg_hip_sync(ctxs[q]) : SG_E_INVAL;
-  const uint64_t t0 = getCurNs();
-  for (uint32_t k = 0; k < n_bursts && rc == SG_OK; k++) {
-    for (uint32_t q = 0; q < n_queues && rc == SG_OK; q++) {
-      const size_t at = (size_t)q * n_bursts + k;
-      rc = sg_hip_reassemble(ctxs[q], ras[at], nullptr);
-      if (rc == SG_OK) rc = sg_hip_shunt_batch(ctxs[q], ga[at], sa[at]);
-    }
+  if (rc != SG_OK) return (double)rc;
+  auto burst = [&](uint32_t q, uint32_t k) {
+    const size_t at = (size_t)q * n_bursts + k;
+    int r = sg_hip_reassemble(ctxs[q], ras[at], nullptr);
+    if (r == SG_OK) r = sg_hip_shunt_batch(ctxs[q], ga[at], sa[at]);
     // a caller takes the counts in now and then; it also keeps the queues from growing without bound
-    if (rc == SG_OK && (k & 255u) == 255u)
-      for (uint32_t q = 0; q < n_queues && rc == SG_OK; q++) rc = sg_hip_sync(ctxs[q]);
+    if (r == SG_OK && (k & 255u) == 255u) r = sg_hip_sync(ctxs[q]);
+    return r;
+  };
+  const uint64_t t0 = getCurNs();
+  if (threaded) {
+    std::vector<int> rcs(n_queues, SG_OK);
+    std::vector<std::thread> threads;
+    for (uint32_t q = 0; q < n_queues; q++)
+      threads.emplace_back([&, q] {
+        int r = SG_OK;
+        for (uint32_t k = 0; k < n_bursts && r == SG_OK; k++) r = burst(q, k);
+        if (r == SG_OK) r = sg_hip_sync(ctxs[q]);
+        rcs[q] = r;
+      });
+    for (auto &t : threads) t.join();
+    for (int r : rcs)
+      if (r != SG_OK && rc == SG_OK) rc = r;
+  } else {
+    for (uint32_t k = 0; k < n_bursts && rc == SG_OK; k++)
+      for (uint32_t q = 0; q < n_queues && rc == SG_OK; q++) rc = burst(q, k);
+    for (uint32_t q = 0; q < n_queues && rc == SG_OK; q++) rc = sg_hip_sync(ctxs[q]);
   }
-  for (uint32_t q = 0; q < n_queues && rc == SG_OK; q++) rc = sg_hip_sync(ctxs[q]);
   const double dt = (double)(getCurNs() - t0) * 1e-9;
   return rc == SG_OK ? dt : (double)rc;
 }

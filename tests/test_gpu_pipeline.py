@@ -484,18 +484,21 @@ def test_reassembly_on_a_stream_of_its_own_beside_the_copy(burst):
     ctx_sg.close()
 
 
-def test_receive_queues_side_by_side_from_a_native_loop():
+@pytest.mark.parametrize("threaded", [0, 1])
+def test_receive_queues_side_by_side_from_a_native_loop(threaded):
     """Three receive queues, each with a context (stream, reassembly table,
     cursors), rings and tables of its own, every queue's bursts filed,
-    gathered and answered from one native loop with no host wait
-    (sgh_pipeline_queues_gpu of libsg_host.so): each queue's request arena,
+    gathered and answered from a native loop with no host wait
+    (sgh_pipeline_queues_gpu of libsg_host.so, from one thread or from a
+    thread per queue): each queue's request arena,
     TX ring and cursors against the oracle's reassembly, gather and scatter
     replayed burst by burst."""
     import ctypes as C
     from splitrpc_amd import build
     host = C.CDLL(build.HOST_LIB)
     host.sgh_pipeline_queues_gpu.restype = C.c_double
-    host.sgh_pipeline_queues_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]
+    host.sgh_pipeline_queues_gpu.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32,
+                                             C.c_int]
     n_queues, burst, n_reqs, resp_size = 3, 16, 30, 3000
     per_req, A = 3, capi.F_ASYNC
     queues = []
@@ -543,8 +546,8 @@ def test_receive_queues_side_by_side_from_a_native_loop():
     c_ga = ptrs([q["ga"] for q in queues for _ in range(n_bursts)])
     c_sa = ptrs([q["sa"] for q in queues for _ in range(n_bursts)])
     torch.cuda.synchronize()
-    print(f"case queues={n_queues} bursts={n_bursts} of {burst}", flush=True)
-    dt = host.sgh_pipeline_queues_gpu(c_ctx, n_queues, c_ras, c_ga, c_sa, n_bursts)
+    print(f"case queues={n_queues} bursts={n_bursts} of {burst} threaded={threaded}", flush=True)
+    dt = host.sgh_pipeline_queues_gpu(c_ctx, n_queues, c_ras, c_ga, c_sa, n_bursts, threaded)
     assert dt > 0, (dt, [q["ctx"].lib.sg_hip_last_error(q["ctx"].h) for q in queues])
     torch.cuda.synchronize()
     for qi, q in enumerate(queues):
