@@ -19,7 +19,9 @@
  * sg_hip_last_error() gives the text of the last failure on a context.
  * No exceptions cross the ABI.  A context is used by one thread at a time
  * (the reference constructs and uses its engine on the shunter thread,
- * src/splitrpc_server/p2p_rpc_dpdk_server.cc:79-87).
+ * src/splitrpc_server/p2p_rpc_dpdk_server.cc:79-87); different contexts may
+ * be used from different threads at the same time (a shunter thread per
+ * receive queue, each with a context of its own).
  */
 #ifndef SG_HIP_H
 #define SG_HIP_H
