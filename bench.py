@@ -460,12 +460,15 @@ def native_shunt_loop(ctxs, pool: "Pool", steps: int, latency: bool = False):
     return runs[len(runs) // 2]
 
 
-def host_engine_batched(pool: "Pool", steps: int) -> dict:
+def host_engine_batched(pool: "Pool", steps: int, default_only: bool = False) -> dict:
     """The batched calls of the C++ drop-in, P2pRpcSgHipEngine::gather_batch(P2pRpcRr **) and
     scatter_batch(P2pRpcRr **), over the requests of one default call held as P2pRpcRr objects
     (sgh_engine_loop_gpu of libsg_host.so): with the engine walking every fragment on the host,
     and with the requests' fragment tables kept where the device reads them.  Response headers
-    come from the connections' templates here (fresh response buffers, rr_set_hdr)."""
+    come from the connections' templates here (fresh response buffers, rr_set_hdr).  With the tables
+    attached the engine decides per call: from 49152 fragments (frames) on the device pulls them,
+    smaller calls' tables the calling thread walks and leaves in pinned memory for the kernels to
+    read.  `default_only`: just that form (a call of another size than the default)."""
     import ctypes as C
     import numpy as np
     w = pool.w
@@ -484,6 +487,8 @@ def host_engine_batched(pool: "Pool", steps: int) -> dict:
     out = {"requests": dw.n_req, "fragments": dw.n_frags, "response_frames": dw.n_frames}
     total = pool.gather_bytes + pool.scatter_bytes
     for mode, name in ((0, "tables_walked_by_the_host"), (1, "tables_pulled_by_the_device")):
+        if default_only and mode == 0:
+            continue
         res = np.zeros(16, np.float64)
         rc = host.sgh_engine_loop_gpu(0, mode, len(items), pv(bases), dw.rx.n_slots, w.slot_size, w.profile, pv(fs),
                                       pv(fl), dw.n_req, per, int(w.req_sizes[0]), dw.req_app.cap, w.mtu,
@@ -499,6 +504,8 @@ def host_engine_batched(pool: "Pool", steps: int) -> dict:
                      "host_us_per_scatter_batch_call": round(float(res[9]) * 1e-3, 2),
                      "gather_batch_host_ns_[N,Mean,p90,p95,p99,min,max]": [round(float(x), 2) for x in res[1:8]],
                      "scatter_batch_host_ns_[N,Mean,p90,p95,p99,min,max]": [round(float(x), 2) for x in res[8:15]]}
+    if default_only:
+        return out["tables_pulled_by_the_device"]
     # the reference's own call through the same engine: one synchronous gather(rr, stub) per request
     res = np.zeros(16, np.float64)
     rc = host.sgh_engine_loop_gpu(0, 2, len(items), pv(bases), dw.rx.n_slots, w.slot_size, w.profile, pv(fs), pv(fl),
@@ -1029,6 +1036,12 @@ def main() -> int:
     if not a.no_single:
         _log("C++ engine, batched calls over P2pRpcRr objects")
         host_engine = host_engine_batched(pool, max(50, min(a.steps, 200)))
+        if host_engine is not None and bpl != 1:
+            # one batch per call, as the reference's shunter makes them: tables attached, the engine's choice
+            p1 = Pool(w, 1, 128, extra, rule=rule)
+            host_engine["single_batch_call"] = host_engine_batched(p1, 500, default_only=True)
+            del p1
+            torch.cuda.empty_cache()
 
     _log("per-request calls")
     per_req = per_request_calls(ctx, pool.items[0]) if not w.in_tensor_sizes else None

@@ -202,7 +202,8 @@ int sgh_ring_stress(uint32_t n_threads, uint32_t per_thread, uint32_t capacity)
 // with the application slots' state words published by the device and walked
 // by the worker's batching window on the host; 3 the same with the requests'
 // fragment tables kept where the device reads them, so that the batched calls
-// walk no fragment on the host.  The request arena
+// walk no fragment on the host (the form large calls take, forced here); 4 is 2
+// with the walked tables copied to the device instead of read in place.  The request arena
 // (n_done * req_size bytes) and the TX ring are copied back for inspection.
 // Fixed-size requests (req_size) as in the reference.  Returns completed
 // requests or a negative error.
@@ -229,12 +230,18 @@ int64_t sgh_serve_gpu(int device_id, const uint8_t *ring_host, uint32_t n_slots,
     pool.setup_and_init_rr_pool(srv, req_size);
     release_conn_info(srv);
     P2pRpcSgHipEngine engine(device_id);
+    if (per_request == 4) {
+      // the tables the thread walks brought over by a kernel, as calls too large to be read in place are
+      engine.in_place_max_bytes = 0;
+      per_request = 2;
+    }
     if (per_request == 3) {
       // the requests' fragment tables where the device reads them: written below as fragments are
       // filed, pulled by the batched calls
       sg_frag_table *t = engine.frag_tables((uint32_t)pool.get_pool_size());
       if (!t) return -18;
       pool.attach_frag_tables(t, (size_t)pool.get_pool_size(), (uintptr_t)d_ring & ~(uintptr_t)1);
+      engine.pull_min_items = 0;  // every call of this (small) run pulls its tables
       tables_pulled = true;
       per_request = 2;
     }

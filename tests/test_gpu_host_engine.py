@@ -45,7 +45,8 @@ def p(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
 
-@pytest.mark.parametrize("per_request", [1, 0, 2, 3], ids=["per-request", "batched", "batched-tx", "tables-pulled"])
+@pytest.mark.parametrize("per_request", [1, 0, 2, 3, 4],
+                         ids=["per-request", "batched", "batched-tx", "tables-pulled", "batched-tx-staged"])
 @pytest.mark.parametrize("mirror", [1, 0], ids=["mirrored", "plain"])
 @pytest.mark.parametrize("cfg,n,profile", [(1, 12, synth.HDR_BL58), (2, 3, synth.HDR_BL58),
                                            (2, 2, synth.HDR_REF64), (5, 1, synth.HDR_BL58)])
