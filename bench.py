@@ -576,7 +576,7 @@ def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, 
 
 
 def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 65536, 0), n_queues: int = 4,
-                    queues_up_to: int = 65536) -> dict:
+                    queues_up_to: int = 1 << 30) -> dict:
     """The receive path end to end on the device, burst after burst and no
     host wait in between, from a native loop (sgh_pipeline_loop_gpu of
     libsg_host.so): sg_hip_reassemble files a burst's arrivals (requests that
