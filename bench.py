@@ -532,9 +532,11 @@ def graph_step_time(w, extra: int, rule: bool, rotate_mb: int, steps: int = 16, 
     from splitrpc_amd.engine import SgContext
     lanes = []
     for _ in range(streams):
-        stream = torch.cuda.Stream()
-        ctx = SgContext(0, max_reqs=max(4096, w.n_req), max_frames=max(65536, w.n_frags, w.n_resp_frames),
-                        stream=stream.cuda_stream)
+        # every lane's stream on a hardware queue of its own where one is to be had: graphs replayed
+        # on streams that share a queue run one after the other
+        kw = dict(max_reqs=max(4096, w.n_req), max_frames=max(65536, w.n_frags, w.n_resp_frames))
+        ctx = SgContext.apart_from([l[1] for l in lanes], 0, **kw) if lanes else SgContext(0, **kw)
+        stream = torch.cuda.ExternalStream(ctx.stream, device="cuda:0")
         pool = Pool(w, 1, max(64, rotate_mb // streams), extra, rule=rule)
 
         def one(i, ctx=ctx, pool=pool):
