@@ -1291,18 +1291,28 @@ int sg_hip_shunt_batch(sg_hip_ctx *c, const sg_gather_args *g, const sg_scatter_
   if (!c || !g || !s) return fail(c, SG_E_INVAL, "null argument");
   DeviceGuard guard(c->device);
   const uint32_t async = g->flags & s->flags & SG_F_ASYNC;
-  // what the scatter writes (TX slots) and reads (responses) against what the gather reads (RX
-  // slots) and writes (requests): halves that touch each other's memory run one after the other
-  bool apart = !ranges_overlap(s->tx.base, (uint64_t)s->tx.n_slots * s->tx.slot_size, g->ring.base,
-                               (uint64_t)g->ring.n_slots * g->ring.slot_size);
-  if (g->app.n_tensors == 0 && s->app.n_tensors == 0)
-    apart = apart && !ranges_overlap(s->app.arena, s->app.arena_cap, g->app.arena, g->app.arena_cap);
-  else if (g->app.n_tensors == 0 || s->app.n_tensors == 0)
-    apart = false;  // an arena against tensors: not looked into
-  else
-    for (uint32_t i = 0; i < g->app.n_tensors; i++)
-      for (uint32_t j = 0; j < s->app.n_tensors; j++)
-        apart = apart && g->app.tensor_base[i] != s->app.tensor_base[j];
+  // What the gather writes (requests) against everything the scatter touches (responses, the ring
+  // its headers come from, TX slots), and what the scatter writes (TX slots) against what the gather
+  // reads (RX slots): halves that touch each other's memory run one after the other.  Application
+  // memory is an arena or, tensor-major, n_req rows per tensor.
+  struct Range { const void *p; uint64_t n; };
+  auto app_ranges = [](const sg_app_desc &app, uint32_t n_req, Range *out) {
+    uint32_t k = 0;
+    if (app.n_tensors == 0) out[k++] = Range{app.arena, app.arena_cap * (app.arena_mirrored ? 2u : 1u)};
+    else
+      for (uint32_t t = 0; t < app.n_tensors && t < SG_MAX_TENSORS; t++)
+        out[k++] = Range{app.tensor_base[t], app.tensor_size[t] * n_req};
+    return k;
+  };
+  Range gw[SG_MAX_TENSORS + 1], st[SG_MAX_TENSORS + 3];
+  const uint32_t n_gw = app_ranges(g->app, g->n_req, gw);
+  uint32_t n_st = app_ranges(s->app, s->n_req, st);
+  const Range s_tx{s->tx.base, (uint64_t)s->tx.n_slots * s->tx.slot_size};
+  st[n_st++] = s_tx;
+  st[n_st++] = Range{s->rx.base, (uint64_t)s->rx.n_slots * s->rx.slot_size};
+  bool apart = !ranges_overlap(s_tx.p, s_tx.n, g->ring.base, (uint64_t)g->ring.n_slots * g->ring.slot_size);
+  for (uint32_t i = 0; i < n_gw; i++)
+    for (uint32_t j = 0; j < n_st; j++) apart = apart && !ranges_overlap(gw[i].p, gw[i].n, st[j].p, st[j].n);
   // Both halves are looked at before either is launched: a call the host refuses launches nothing.
   // A half that cannot share a launch leaves no trace; both are then made as calls of their own.
   ShuntHalf h;
