@@ -165,7 +165,13 @@ typedef struct sg_app_desc {
 
 /* One gather batch: the fragment tables of n_req reassembled requests in
  * compact CSR form (what P2pRpcRr::payload_bufs holds per request,
- * src/p2p_rpc_rr_ng.h:29-31, with pointers reduced to slot indices). */
+ * src/p2p_rpc_rr_ng.h:29-31, with pointers reduced to slot indices).
+ * "device" below is memory the device can read: device memory, or -- for the
+ * tables of a small call, a few tens of KB -- pinned host memory, which the
+ * kernels then read across the bus (that saves the copy and the launch that
+ * makes it; tables of large calls belong in device memory: bus reads in
+ * flight beside a copy kernel slow it down).  The same holds for the tables of
+ * sg_scatter_args. */
 typedef struct sg_gather_args {
   sg_ring_desc ring;
   const uint32_t *frag_slot; /* device, n_frags: ring slot of each fragment; requests in
