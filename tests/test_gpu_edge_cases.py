@@ -753,3 +753,41 @@ def test_reused_descriptors_are_held_against_the_call_that_uses_them(ctx):
     dw.scatter(ctx, fixed=False, reuse=True)
     exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.req_app.cap)
     assert np.array_equal(dw.ring.cpu().numpy(), exp_tx)
+
+
+@pytest.mark.parametrize("mode", ["scan", "rule", "one-launch"])
+@pytest.mark.parametrize("cfg,n", [(2, 1), (1, 40), (4, 30)])
+def test_tables_of_a_small_call_read_from_pinned_host_memory(ctx, cfg, n, mode):
+    """The CSR tables of a call (fragment slots, lengths, request and response
+    tables, response sizes) left in pinned host memory, where the kernels read
+    them across the bus -- what the C++ engine does for calls whose tables the
+    calling thread walks: results as with tables in device memory."""
+    w = synth.make_workload(cfg, n)
+    one_size = bool((w.req_sizes == w.req_sizes[0]).all())
+    if mode != "scan" and not one_size:
+        pytest.skip("the fragmenting rule needs one request size")
+    print(f"case pinned tables cfg={cfg} n={n} mode={mode}", flush=True)
+    dw = DeviceWorkload(w)
+    pin = lambda t: t.cpu().pin_memory() if t is not None else None
+    g = dw.gather_call(ctx, 0, use_frag_len=True, rule=mode != "scan")
+    s = dw.scatter_call(ctx, 0, fuse=mode != "scan")
+    keep = [pin(dw.frag_slot), pin(dw.frag_len), pin(dw.req_first), pin(dw.tx_slot), pin(dw.hdr_src_slot),
+            pin(dw.resp_first), pin(dw.resp_size)]
+    g.frag_slot, g.frag_len, g.req_first = keep[0].data_ptr(), keep[1].data_ptr(), keep[2].data_ptr()
+    s.tx_slot, s.hdr_src_slot, s.resp_first = keep[3].data_ptr(), keep[4].data_ptr(), keep[5].data_ptr()
+    if s.resp_size:
+        s.resp_size = keep[6].data_ptr()
+    ctx.set_cursor(0, 0)
+    ctx.set_cursor(1, 0)
+    if mode == "one-launch":
+        ctx.shunt_batch_raw(g, s)
+    else:
+        ctx.gather_batch_raw(g)
+        ctx.scatter_batch_raw(s)
+    exp, eoffs, _ = expected_gather(w, arena_cap=dw.req_app.cap)
+    got = dw.req_arena.cpu().numpy()
+    assert np.array_equal(got, exp), first_diff(got, exp)
+    assert np.array_equal(dw.req_offsets.cpu().numpy().view(np.uint64), eoffs)
+    exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
+    got = dw.tx_ring.cpu().numpy()
+    assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
