@@ -726,6 +726,20 @@ double sgh_pipeline_loop_gpu(sg_hip_ctx *ra, sg_hip_ctx *sg, const sg_reassemble
   return rc == SG_OK ? dt : (double)rc;
 }
 
+// Slot indices of `n` payload pointers of a ring, by the walk the batched calls make (a shift for
+// slots of a power of two bytes) and by the single-pointer form (a division): both into their
+// output, -1 where a pointer is no payload start of the ring.  Host only.
+void sgh_slots_of_payloads(uint64_t base, uint32_t n_slots, uint32_t slot_size, uint32_t profile,
+                           const uint64_t *payloads, uint32_t n, int64_t *by_walk, int64_t *by_division)
+{
+  SgRingView view{sg_ring_desc{(void *)(uintptr_t)base, n_slots, slot_size, profile, 0}};
+  const SgRingView::Walk slot_of = view.walk();
+  for (uint32_t i = 0; i < n; i++) {
+    by_walk[i] = slot_of((uintptr_t)payloads[i]);
+    by_division[i] = view.slot_of_payload((uintptr_t)payloads[i]);
+  }
+}
+
 // Several receive queues side by side, each with a context (stream, reassembly table, cursors) of
 // its own, as a NIC spreads flows over its RX queues and the reference keeps an rr pool per queue:
 // every burst of a queue is filed and its completed requests gathered and answered

@@ -152,6 +152,33 @@ def test_pointer_ring_multi_producer_multi_consumer(host):
 
 # ---------------------------------------------------------------- client patterns (load generator)
 
+@pytest.mark.parametrize("slot_size", [2048, 9216, 1536, 4096])
+@pytest.mark.parametrize("profile", [0, 1])
+def test_slot_of_a_payload_pointer_by_shift_and_by_division(host, slot_size, profile):
+    """The batched calls turn payload pointers into slot indices with a shift
+    where slots are a power of two bytes and a division elsewhere: both forms
+    against the arithmetic, on payload starts, pointers off a payload start
+    and pointers outside the ring."""
+    host.sgh_slots_of_payloads.argtypes = [C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_uint32,
+                                           C.c_void_p, C.c_void_p]
+    host.sgh_slots_of_payloads.restype = None
+    rng = np.random.default_rng(slot_size + profile)
+    base, n_slots, hl = 0x7F0000001000 + 2 * int(rng.integers(0, 64)), 777, 64 if profile else 58
+    slots = rng.integers(0, n_slots, 4000)
+    good = base + slots * slot_size + hl
+    off = good + rng.integers(1, slot_size, 4000)                     # inside a slot, not at its payload
+    outside = np.concatenate([base + (n_slots + rng.integers(0, 9, 50)) * slot_size + hl,      # behind the ring
+                              base - rng.integers(1, 5, 50) * slot_size + hl,                  # in front of it
+                              np.array([base, base + hl - 1, 0], np.int64)])
+    p = np.ascontiguousarray(np.concatenate([good, off, outside]).astype(np.uint64))
+    want = np.concatenate([slots, np.full(off.size + outside.size, -1)]).astype(np.int64)
+    by_walk, by_div = np.zeros(p.size, np.int64), np.zeros(p.size, np.int64)
+    pv = lambda x: x.ctypes.data_as(C.c_void_p)
+    host.sgh_slots_of_payloads(base, n_slots, slot_size, profile, pv(p), p.size, pv(by_walk), pv(by_div))
+    assert np.array_equal(by_div, want)
+    assert np.array_equal(by_walk, want)
+
+
 def test_state_word_wait_is_bounded(host):
     """AppRrRunNotify waits on the calling thread: the word has to be set by
     somebody else.  Another thread setting it ends the wait; nobody setting it
