@@ -21,22 +21,28 @@ static inline uint64_t getCurNs()
   return (uint64_t)ts.tv_sec * 1000000000ull + (uint64_t)ts.tv_nsec;
 }
 
-// The sample at index round(p * (N - 1)) of the sorted samples (0 for none).
-static inline double getPercentile(std::vector<uint64_t> &v, double p)
+// Index of the p-quantile among N sorted samples: round(p * (N - 1)).
+static inline size_t sg_quantile_index(double p, size_t n)
 {
-  if (v.empty()) return 0.0;
-  const size_t k = (size_t)std::llround(p * (double)(v.size() - 1));
+  return n ? (size_t)std::llround(p * (double)(n - 1)) : 0;
+}
+
+// The sample at that index of the sorted samples (0 for none).  The vector is left as it was.
+static inline double getPercentile(const std::vector<uint64_t> &v, double p)
+{
+  const size_t k = sg_quantile_index(p, v.size());
   if (k >= v.size()) return 0.0;
-  std::nth_element(v.begin(), v.begin() + k, v.end());
-  return (double)v[k];
+  std::vector<uint64_t> sorted(v);
+  std::sort(sorted.begin(), sorted.end());
+  return (double)sorted[k];
 }
 
 static inline double getMean(const std::vector<uint64_t> &v)
 {
-  double mean = 0.0;
-  uint64_t n = 0;
-  for (uint64_t x : v) mean += ((double)x - mean) / (double)++n;
-  return mean;
+  if (v.empty()) return 0.0;
+  long double sum = 0.0L;
+  for (uint64_t x : v) sum += (long double)x;
+  return (double)(sum / (long double)v.size());
 }
 
 // The seven numbers of the summary line, in its order.
@@ -44,17 +50,18 @@ struct SgStatLine {
   double v[7];  // N, mean, p90, p95, p99, min, max
 };
 
+// One sort serves the three quantiles and both ends.
 static inline SgStatLine sg_stat_line(std::vector<uint64_t> v)
 {
   SgStatLine s{};
   s.v[0] = (double)v.size();
   if (v.empty()) return s;
   s.v[1] = getMean(v);
-  s.v[2] = getPercentile(v, 0.90);
-  s.v[3] = getPercentile(v, 0.95);
-  s.v[4] = getPercentile(v, 0.99);
-  s.v[5] = (double)*std::min_element(v.begin(), v.end());
-  s.v[6] = (double)*std::max_element(v.begin(), v.end());
+  std::sort(v.begin(), v.end());
+  const double q[3] = {0.90, 0.95, 0.99};
+  for (int i = 0; i < 3; i++) s.v[2 + i] = (double)v[sg_quantile_index(q[i], v.size())];
+  s.v[5] = (double)v.front();
+  s.v[6] = (double)v.back();
   return s;
 }
 
