@@ -524,7 +524,8 @@ double sgh_step_loop_gpu(sg_hip_ctx *g, sg_hip_ctx *s, const sg_gather_args *con
 // arena, response arena of item k).
 //   mode 0  batched: gather_batch(P2pRpcRr **) + scatter_batch(P2pRpcRr **) per step, the engine
 //           walking every fragment on the host
-//   mode 1  the same with the requests' fragment tables kept where the device reads them
+//   mode 1  the same with the requests' fragment tables kept where the device reads them: calls of
+//           engine.pull_min_items fragments (frames) or more have them pulled by the device
 //   mode 2  the reference's call: one synchronous gather(rr, stub) per request, `steps` calls
 // out[0]: seconds per step (per call in mode 2) over the whole loop, the device drained at the
 // end; out[1..7] / out[8..14]: [N, mean, p90, p95, p99, min, max] of the nanoseconds the
