@@ -791,3 +791,26 @@ def test_tables_of_a_small_call_read_from_pinned_host_memory(ctx, cfg, n, mode):
     exp_tx, _, _ = expected_scatter(w, exp, resp_cap=dw.resp_app.cap)
     got = dw.tx_ring.cpu().numpy()
     assert np.array_equal(got, exp_tx), first_diff(got, exp_tx)
+
+
+def test_hardware_queue_of_a_stream(ctx):
+    """sg_hip_stream_queue: the same answer for a stream every time it is asked,
+    a non-zero one, also for a stream the context does not own; contexts made
+    apart from each other sit on different hardware queues where the runtime
+    has more than one to give."""
+    q1, q2 = ctx.stream_queue(), ctx.stream_queue()
+    assert q1 != 0 and q1 == q2
+    s = torch.cuda.Stream()
+    qs = ctx.stream_queue(s.cuda_stream)
+    assert qs != 0 and qs == ctx.stream_queue(s.cuda_stream)
+    assert ctx.lib.sg_hip_stream_queue(ctx.h, None, None) == capi.SG_E_INVAL
+    others = [ctx]
+    for _ in range(2):
+        others.append(SgContext.apart_from(others, 0))
+    queues = [c.stream_queue() for c in others]
+    print("case hardware queues", [hex(q) for q in queues], flush=True)
+    assert all(q != 0 for q in queues)
+    for c in others[1:]:
+        c.close()
+    if len(set(queues)) < 2:
+        pytest.skip("the runtime gave every stream the same hardware queue (GPU_MAX_HW_QUEUES=1?)")
