@@ -159,6 +159,9 @@ class Pool:
 
 
 MIN_TIMED_MS = 50.0
+# bursts of up to this many arrivals are reassembled in workgroups of 256 threads (SG_F_SMALL_GROUPS)
+# where the reassembly runs beside a copy
+BESIDE_UP_TO = 65536
 
 
 def stat_line(ns) -> list:
@@ -592,7 +595,8 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
       one_stream   the calls of a burst one after the other on one context
       overlapped   the reassembly on a context (stream) of its own, its output
                    tables double-buffered, events between the two streams: burst
-                   k + 1 is filed while burst k is gathered and answered
+                   k + 1 is filed while burst k is gathered and answered (in
+                   workgroups of 256 threads, which find room beside the copy)
       N_queues     (bursts of up to `queues_up_to` arrivals) N receive queues side
                    by side, each a one_stream pipeline of its own (_pipeline_queues)"""
     import ctypes as C
@@ -648,7 +652,8 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
         tx_slot = to_dev(np.arange(bound * per_resp, dtype=np.uint32), dev)
         resp_first = to_dev((np.arange(bound + 1) * per_resp).astype(np.uint32), dev)
         A = capi.F_ASYNC
-        ras, gas, sas = [], [], []
+        # ras_beside: the same calls in workgroups of 256 threads, for the form whose reassembly runs beside the copy
+        ras, ras_beside, gas, sas = [], [], [], []
         by_item = {}
         for call in range(calls):
             it = items[call % len(items)]
@@ -664,14 +669,15 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
                         ctx_sg.scatter_args(it.rx, tx, tx_slot, None, resp_first, None, rsize, bound, bound * per_resp,
                                             w.mtu, AppRef(arena=resp_arena, cap=resp_cap), None, w.flags | A,
                                             hdr_src_req=t["hdr"], counts=t["counts"]))
-                ras.append(ctx_sg.reassemble_args(it.rx, it.arrivals[b:b + burst], min(burst, n_arr - b), t["fs"],
-                                                  t["fl"], t["rf"], req_hdr_slot=t["hdr"], counts_out=t["counts"],
-                                                  flags=A))
+                for lst, fl_ in ((ras, A), (ras_beside, A | capi.F_SMALL_GROUPS)):
+                    lst.append(ctx_sg.reassemble_args(it.rx, it.arrivals[b:b + burst], min(burst, n_arr - b), t["fs"],
+                                                      t["fl"], t["rf"], req_hdr_slot=t["hdr"], counts_out=t["counts"],
+                                                      flags=fl_))
                 gas.append(by_item[key][0])
                 sas.append(by_item[key][1])
         n_bursts = len(ras)
         arr = lambda xs: (C.c_void_p * len(xs))(*[C.addressof(x) for x in xs])
-        c_ras, c_gas, c_sas = arr(ras), arr(gas), arr(sas)
+        c_ras, c_ras_beside, c_gas, c_sas = arr(ras), arr(ras_beside), arr(gas), arr(sas)
         res = {}
         for form in ("one_stream", "overlapped"):
             c_ra = ctx_sg if form == "one_stream" else ctx_ra
@@ -679,8 +685,9 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
             for rep in range(3):
                 c_ra.reassemble_reset()
                 torch.cuda.synchronize()
-                dt = host.sgh_pipeline_loop_gpu(c_ra.h, ctx_sg.h, c_ras, c_gas, c_sas, n_bursts,
-                                                1 if form == "overlapped" else 0)
+                beside = form == "overlapped" and burst <= BESIDE_UP_TO
+                dt = host.sgh_pipeline_loop_gpu(c_ra.h, ctx_sg.h, c_ras_beside if beside else c_ras,
+                                                c_gas, c_sas, n_bursts, 1 if form == "overlapped" else 0)
                 if dt < 0:
                     raise RuntimeError(f"sgh_pipeline_loop_gpu failed: {dt} {ctx_sg.lib.sg_hip_last_error(ctx_sg.h)}")
                 best = dt if best is None else min(best, dt)
@@ -695,7 +702,7 @@ def device_pipeline(pool: "Pool", calls: int = 6, bursts=(1024, 4096, 16384, 655
         out[str(burst)] = res
         ctx_ra.close()
         ctx_sg.close()
-        del sets, req_arena, resp_arena, tx_ring, gas, sas, ras, by_item
+        del sets, req_arena, resp_arena, tx_ring, gas, sas, ras, ras_beside, by_item
         torch.cuda.empty_cache()
         if burst <= queues_up_to:
             res[f"{n_queues}_queues"] = _pipeline_queues(host, pool, items_q, n_queues, calls, burst, bound, mf, size,
@@ -722,6 +729,10 @@ def _pipeline_queues(host, pool, items, n_queues, calls, burst, bound, mf, size,
     dw = items[0]
     A = capi.F_ASYNC
     i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
+    # a queue's reassembly runs beside the other queues' copies: workgroups of 256 threads -- up to
+    # bursts of 65536 arrivals; a whole call's reassembly takes slots from the copy for longer than it
+    # gains by not waiting for the copy's end (130 us per burst with workgroups of 1024 threads, 137 with 256)
+    ra_flags = capi.F_SMALL_GROUPS if burst <= BESIDE_UP_TO else 0
     ctxs, keep, ras, gas, sas = [], [], [], [], []
     for q in range(n_queues):
         kw = dict(max_reqs=max(4096, dw.n_req), max_frames=mf)
@@ -750,7 +761,8 @@ def _pipeline_queues(host, pool, items, n_queues, calls, burst, bound, mf, size,
                                      hdr_src_req=t["hdr"], counts=t["counts"]))
             for b in range(0, n_arr, burst):
                 ras.append(ctx.reassemble_args(it.rx, it.arrivals[b:b + burst], min(burst, n_arr - b), t["fs"], t["fl"],
-                                               t["rf"], req_hdr_slot=t["hdr"], counts_out=t["counts"], flags=A))
+                                               t["rf"], req_hdr_slot=t["hdr"], counts_out=t["counts"],
+                                               flags=A | ra_flags))
                 gas.append(by_item[k][0])
                 sas.append(by_item[k][1])
     n_bursts = len(ras) // n_queues

@@ -94,6 +94,12 @@ extern "C" {
                                           calls of few wavefronts; a call that publishes slot states
                                           always has the kernel behind it. */
 #define SG_F_TAIL_KERNEL (1u << 21)    /* the opposite: always the kernel behind the call (for experiments) */
+#define SG_F_SMALL_GROUPS (1u << 22)   /* sg_hip_reassemble: the call is meant to run BESIDE a long copy
+                                          kernel of another stream (another receive queue's gather, or
+                                          this queue's previous burst): its kernels then come in
+                                          workgroups of 256 threads, which find room on a chip that such a
+                                          kernel keeps full, where the usual ones of 1024 wait until it
+                                          ends.  Same results.  A call that runs alone is faster without. */
 
 /* States of an application slot (APP_RR_STATUS, src/p2p_rpc_app_ctx.h:22). */
 #define SG_SLOT_FREE 0u

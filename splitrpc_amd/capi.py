@@ -34,6 +34,7 @@ F_NO_SMALL = 1 << 18
 F_FORCE_SMALL = 1 << 19
 F_SELF_ADVANCE = 1 << 20
 F_TAIL_KERNEL = 1 << 21
+F_SMALL_GROUPS = 1 << 22
 
 ABI_VERSION = 3  # SG_HIP_ABI_VERSION of include/sg_hip.h these mirrors were written against
 MAX_BI_SIZE = 1024

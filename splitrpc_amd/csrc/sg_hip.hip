@@ -1497,7 +1497,7 @@ int ra_state(sg_hip_ctx *c, RaArgs *r, bool *fresh)
   const uint32_t n_max = c->max_frames;
   const uint32_t cells = pow2_at_least(4ull * c->max_reqs < 2 * kRaBucket ? 2 * kRaBucket : 4ull * c->max_reqs);
   const uint32_t records = pow2_at_least(c->max_reqs);
-  const size_t n_blk = (n_max + kRaBlock - 1) / kRaBlock + 1;
+  const size_t n_blk = (n_max + kRaSmallBlock - 1) / kRaSmallBlock + 1;  // a total per workgroup of k_ra_flag, the small ones
   const size_t bytes = (size_t)cells * (8 + 8 + 4 * 4) + (size_t)records * SG_MAX_BI_SIZE * 8 + (size_t)records * 4 +
                        kRaWords * 4 + (size_t)n_max * (3 * 4 + 8) + n_blk * 8 + 256;
   *fresh = false;
@@ -1605,7 +1605,10 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *coun
   r.req_size = a->req_size;
   r.max_req = c->max_reqs;
   r.max_frag = c->max_frames;
-  r.n_blocks = (a->n_arrivals + kRaBlock - 1) / kRaBlock;
+  // workgroups of 256 threads where the caller says the call runs beside a long kernel
+  const bool small_groups = (a->flags & SG_F_SMALL_GROUPS) != 0;
+  r.blk_size = small_groups ? kRaSmallBlock : kRaBlock;
+  r.n_blocks = (a->n_arrivals + r.blk_size - 1) / r.blk_size;
   r.frag_slot = a->frag_slot;
   r.frag_len = a->frag_len;
   r.req_first = a->req_first;
@@ -1620,10 +1623,17 @@ int sg_hip_reassemble(sg_hip_ctx *c, const sg_reassemble_args *a, uint32_t *coun
     // a NIC burst (an empty one still leaves its counts): one workgroup, one launch
     k_ra_burst<<<1, kRaTakeBlock, 0, c->stream>>>(r);
   } else {
-    k_ra_insert<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
-    k_ra_flag<<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
-    k_ra_scan<<<1, kRaBlock, 0, c->stream>>>(r);
-    k_ra_emit<<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
+    if (small_groups) {
+      k_ra_insert<kRaSmallBlock><<<r.n_blocks, kRaSmallBlock, 0, c->stream>>>(r);
+      k_ra_flag<kRaSmallBlock><<<r.n_blocks, kRaSmallBlock, 0, c->stream>>>(r);
+      k_ra_scan<kRaSmallBlock><<<1, kRaSmallBlock, 0, c->stream>>>(r);
+      k_ra_emit<kRaSmallBlock><<<r.n_blocks, kRaSmallBlock, 0, c->stream>>>(r);
+    } else {
+      k_ra_insert<kRaTakeBlock><<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
+      k_ra_flag<kRaBlock><<<r.n_blocks, kRaBlock, 0, c->stream>>>(r);
+      k_ra_scan<kRaBlock><<<1, kRaBlock, 0, c->stream>>>(r);
+      k_ra_emit<kRaTakeBlock><<<g_take, kRaTakeBlock, 0, c->stream>>>(r);
+    }
   }
   rc = prof_end(c);
   if (rc != SG_OK) return rc;

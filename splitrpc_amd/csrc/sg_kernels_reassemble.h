@@ -78,6 +78,7 @@ struct RaArgs {
   unsigned long long *arr_pack;  // (1 << 32 | fragments) at the completing arrival, else 0; then its local scan
   unsigned long long *blk;       // workgroup totals, then their scan
   uint32_t n_blocks;
+  uint32_t blk_size;  // threads per workgroup of k_ra_flag: one entry of blk each
   // outputs
   uint32_t *frag_slot, *frag_len, *req_first, *req_hdr_slot;
   uint64_t *req_token;
@@ -179,9 +180,16 @@ __device__ __forceinline__ uint32_t ra_find_cell(const RaArgs &a, unsigned long 
 // on eight XCDs add to takes some 70 ns, one after the other: 0.29 ms of a 0.35-ms k_ra_insert on a
 // burst of 131072 new requests.)  Every thread of the workgroup has to call this.
 constexpr int kRaTakeBlock = 1024;
+// The same steps in workgroups of kRaSmallBlock threads, for a call that runs beside a long copy
+// kernel of another stream: a workgroup of sixteen wavefronts finds no room on a chip that such a
+// kernel keeps full (it needs sixteen free slots on one CU at once) and waits until that kernel
+// ends; one of four wavefronts takes the slots the copy's own workgroups leave.  Four times the
+// additions to the ring words, which is why this is not the form of a call that runs alone.
+constexpr int kRaSmallBlock = 256;
+template <int B>
 __device__ __forceinline__ uint32_t ra_block_take(uint32_t *word, uint32_t n_wave, uint32_t *lds)
 {
-  constexpr uint32_t kWaves = kRaTakeBlock / kWave;
+  constexpr uint32_t kWaves = B / kWave;
   const uint32_t wv = threadIdx.x / kWave;
   if ((threadIdx.x & (kWave - 1)) == 0) lds[wv] = n_wave;
   __syncthreads();
@@ -203,10 +211,11 @@ __device__ __forceinline__ uint32_t ra_block_take(uint32_t *word, uint32_t n_wav
 // (returns happen in k_ra_emit), so a position at or beyond the tail read here means the pool is
 // exhausted: the cell then gets no record, the call is refused, and k_ra_scan puts the head back
 // to the tail.
+template <int B>
 __device__ __forceinline__ void ra_open_cells(const RaArgs &a, bool claimed, uint32_t cell, uint32_t lane, uint32_t *lds)
 {
   const unsigned long long cl = __ballot(claimed);
-  const uint32_t base = ra_block_take(&a.words[kRaHead], (uint32_t)__popcll(cl), lds);
+  const uint32_t base = ra_block_take<B>(&a.words[kRaHead], (uint32_t)__popcll(cl), lds);
   if (claimed) {
     const uint32_t h = base + (uint32_t)__popcll(cl & ((1ull << lane) - 1ull));
     const uint32_t tail = a.words[kRaTail];
@@ -249,7 +258,7 @@ struct RaMine {
   unsigned long long pack = 0;
 };
 
-template <bool FUSED>
+template <bool FUSED, int B>
 __device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint32_t *take, RaMine &mine)
 {
   const uint32_t n = ra_n(a);
@@ -329,7 +338,7 @@ __device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint
     }
   }
   // the cells this wavefront has claimed get their records (a lane claims one cell at most)
-  ra_open_cells(a, opened != kRaNoCell, opened, lane, take);
+  ra_open_cells<B>(a, opened != kRaNoCell, opened, lane, take);
   mine.cell = cell;
   mine.len = len;
   mine.fidx = fidx;
@@ -346,11 +355,12 @@ __device__ __forceinline__ void ra_insert_step(const RaArgs &a, uint32_t i, uint
   if (lane == 0 && lost) atomicAdd(&a.words[kRaDropped], (uint32_t)__popcll(lost));
 }
 
-__global__ __launch_bounds__(kRaTakeBlock) void k_ra_insert(RaArgs a)
+template <int B>
+__global__ __launch_bounds__(B) void k_ra_insert(RaArgs a)
 {
-  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
+  __shared__ uint32_t take[B / kWave + 1];
   RaMine mine;
-  ra_insert_step<false>(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take, mine);
+  ra_insert_step<false, B>(a, blockIdx.x * B + threadIdx.x, take, mine);
 }
 
 __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell, unsigned long long acc)
@@ -359,7 +369,7 @@ __device__ __forceinline__ bool ra_complete(const RaArgs &a, uint32_t cell, unsi
 }
 
 // Returns the workgroup's packed (requests, fragments) total.
-template <bool FUSED>
+template <bool FUSED, int B>
 __device__ __forceinline__ uint64_t ra_flag_step(const RaArgs &a, uint32_t i, uint64_t *wave_tot, RaMine &mine)
 {
   const uint32_t n = ra_n(a);
@@ -385,17 +395,18 @@ __device__ __forceinline__ uint64_t ra_flag_step(const RaArgs &a, uint32_t i, ui
     }
   }
   uint64_t tot;
-  const uint64_t ex = block_exclusive_scan<kRaBlock>(pack, wave_tot, &tot);
+  const uint64_t ex = block_exclusive_scan<B>(pack, wave_tot, &tot);
   mine.pack = pack ? (ex | (1ull << 63)) : 0;  // top bit: "a request completes here"
   if (!FUSED && i < n) a.arr_pack[i] = mine.pack;
   return tot;
 }
 
-__global__ __launch_bounds__(kRaBlock) void k_ra_flag(RaArgs a)
+template <int B>
+__global__ __launch_bounds__(B) void k_ra_flag(RaArgs a)
 {
-  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  __shared__ uint64_t wave_tot[B / kWave];
   RaMine mine;
-  const uint64_t tot = ra_flag_step<false>(a, blockIdx.x * kRaBlock + threadIdx.x, wave_tot, mine);
+  const uint64_t tot = ra_flag_step<false, B>(a, blockIdx.x * B + threadIdx.x, wave_tot, mine);
   if (threadIdx.x == 0) a.blk[blockIdx.x] = tot;
 }
 
@@ -434,17 +445,19 @@ __device__ __forceinline__ uint32_t ra_scan_finish(const RaArgs &a, uint64_t run
   return overflow;
 }
 
-__global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
+// B: this kernel's own workgroup size; a.blk_size: that of the k_ra_flag before it (a total per workgroup).
+template <int B>
+__global__ __launch_bounds__(B) void k_ra_scan(RaArgs a)
 {
-  __shared__ uint64_t wave_tot[kRaBlock / kWave];
+  __shared__ uint64_t wave_tot[B / kWave];
   const uint32_t n = ra_n(a);
-  const uint32_t n_blocks = (n + kRaBlock - 1) / kRaBlock;
+  const uint32_t n_blocks = (n + a.blk_size - 1) / a.blk_size;
   uint64_t run = 0;
-  for (uint32_t base = 0; base < n_blocks; base += kRaBlock) {
+  for (uint32_t base = 0; base < n_blocks; base += B) {
     const uint32_t b = base + threadIdx.x;
     const uint64_t v = b < n_blocks ? a.blk[b] : 0;
     uint64_t tot;
-    const uint64_t ex = block_exclusive_scan<kRaBlock>(v, wave_tot, &tot);
+    const uint64_t ex = block_exclusive_scan<B>(v, wave_tot, &tot);
     if (b < n_blocks) a.blk[b] = run + ex;
     run += tot;
   }
@@ -455,7 +468,7 @@ __global__ __launch_bounds__(kRaBlock) void k_ra_scan(RaArgs a)
 // into the output tables in sequence order, the record is emptied and returned
 // to the free ring, the cell is emptied.  The request's rank and first fragment
 // index hang on that arrival (arr_pack there plus its workgroup's scanned total).
-template <bool FUSED>
+template <bool FUSED, int B>
 __device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32_t *take, bool overflow, const RaMine &mine)
 {
   const uint32_t n = ra_n(a);
@@ -467,13 +480,13 @@ __device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32
     cell = FUSED ? mine.cell : a.arr_cell[i];
     const unsigned long long p = FUSED ? mine.pack : a.arr_pack[i];
     completes = cell != kRaNoCell && (p >> 63) && !overflow;
-    if (completes) v = (p & ~(1ull << 63)) + (FUSED ? 0ull : a.blk[i / kRaBlock]);  // one workgroup: nothing before it
+    if (completes) v = (p & ~(1ull << 63)) + (FUSED ? 0ull : a.blk[i / B]);  // one workgroup: nothing before it
     // the position of a request's last arrival counts per call
     if (cell != kRaNoCell && !completes) a.last[cell] = 0;
   }
   unsigned long long todo = __ballot(completes);
   // reap_rr for all of this workgroup's requests: one addition to the ring's tail
-  const uint32_t tail0 = ra_block_take(&a.words[kRaTail], (uint32_t)__popcll(todo), take);
+  const uint32_t tail0 = ra_block_take<B>(&a.words[kRaTail], (uint32_t)__popcll(todo), take);
   // requests of a few fragments are handed over by the completing lane itself, all such lanes
   // at once; the wavefront then walks the larger ones together
   constexpr uint32_t kOwn = 8;
@@ -541,10 +554,11 @@ __device__ __forceinline__ void ra_emit_step(const RaArgs &a, uint32_t i, uint32
   }
 }
 
-__global__ __launch_bounds__(kRaTakeBlock) void k_ra_emit(RaArgs a)
+template <int B>
+__global__ __launch_bounds__(B) void k_ra_emit(RaArgs a)
 {
-  __shared__ uint32_t take[kRaTakeBlock / kWave + 1];
-  ra_emit_step<false>(a, blockIdx.x * kRaTakeBlock + threadIdx.x, take, a.words[kRaOverflow] != 0, RaMine());
+  __shared__ uint32_t take[B / kWave + 1];
+  ra_emit_step<false, B>(a, blockIdx.x * B + threadIdx.x, take, a.words[kRaOverflow] != 0, RaMine());
 }
 
 // A burst of at most kRaTakeBlock arrivals: the four steps by one workgroup in one launch.
@@ -556,12 +570,12 @@ __global__ __launch_bounds__(kRaTakeBlock) void k_ra_burst(RaArgs a)
   __shared__ uint32_t overflow;
   const uint32_t i = threadIdx.x;
   RaMine mine;
-  ra_insert_step<true>(a, i, take, mine);
+  ra_insert_step<true, kRaTakeBlock>(a, i, take, mine);
   __syncthreads();
-  const uint64_t tot = ra_flag_step<true>(a, i, wave_tot, mine);
+  const uint64_t tot = ra_flag_step<true, kRaBlock>(a, i, wave_tot, mine);
   if (threadIdx.x == 0) overflow = ra_scan_finish<true>(a, tot);
   __syncthreads();
-  ra_emit_step<true>(a, i, take, overflow != 0, mine);
+  ra_emit_step<true, kRaTakeBlock>(a, i, take, overflow != 0, mine);
 }
 
 // Empties the table: every cell, every record, all records back in the ring.

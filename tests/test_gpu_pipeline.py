@@ -38,7 +38,7 @@ class Tables:
                 self.tok[:n_req].cpu().numpy().view(np.uint64), u32(self.hdr[:n_req]))
 
 
-def _feed_in_bursts(ctx, w, order, burst, tabs, len_nic=None, req_size=0):
+def _feed_in_bursts(ctx, w, order, burst, tabs, len_nic=None, req_size=0, flags=0):
     rx = RingRef(torch.from_numpy(w.ring).to(DEV), w.n_slots, w.slot_size, w.profile)
     arr = to_dev(np.ascontiguousarray(order, np.uint32), DEV)
     ln = to_dev(len_nic, DEV) if len_nic is not None else None
@@ -51,7 +51,8 @@ def _feed_in_bursts(ctx, w, order, burst, tabs, len_nic=None, req_size=0):
         b, n = nxt, min(burst() if callable(burst) else burst, len(order) - nxt)
         nxt += n
         n_req, n_frag, in_flight = ctx.reassemble(rx, arr[b:b + n], n, tabs.fs, tabs.fl, tabs.rf, tabs.tok,
-                                                  ln, req_size, req_hdr_slot=tabs.hdr, counts_out=tabs.counts)
+                                                  ln, req_size, req_hdr_slot=tabs.hdr, counts_out=tabs.counts,
+                                                  flags=flags)
         assert tabs.counts.cpu().tolist() == [n_req, n_frag, ctx.last_dropped, in_flight]
         peak = max(peak, in_flight)
         s, l, f, t, h = tabs.take(n_req, n_frag)
@@ -85,18 +86,20 @@ def test_resnet_sized_requests_arrive_in_bursts_of_64(order_kind):
     ctx.close()
 
 
+@pytest.mark.parametrize("flags", [0, capi.F_SMALL_GROUPS], ids=["groups-of-1024", "groups-of-256"])
 @pytest.mark.parametrize("burst", [1000, 1024, 1025, 2500])
-def test_bursts_around_the_size_one_workgroup_takes(burst):
+def test_bursts_around_the_size_one_workgroup_takes(burst, flags):
     """A burst of up to 1024 arrivals is sorted by one workgroup in one launch,
-    a larger one by four kernels: the same stream in bursts on either side of
-    that size (requests carried across calls both ways) gives what the oracle
-    makes of the whole stream."""
+    a larger one by four kernels (of 1024-thread workgroups, or of 256-thread
+    ones as for a call that runs beside a long kernel): the same stream in
+    bursts on either side of that size (requests carried across calls both
+    ways) gives what the oracle makes of the whole stream."""
     w = synth.make_workload(4, 700)
     order = np.random.default_rng(burst).permutation(w.arrivals)
     ctx = SgContext(0, max_reqs=1024, max_frames=8192)
     ctx.reassemble_reset()
     tabs = Tables(1024, 8192)
-    fs, fl, first, tok, hdr, peak = _feed_in_bursts(ctx, w, order, burst, tabs)
+    fs, fl, first, tok, hdr, peak = _feed_in_bursts(ctx, w, order, burst, tabs, flags=flags)
     efs, efl, erf, etok = oracle.reassemble(w, arrivals=order)
     assert np.array_equal(tok, etok) and np.array_equal(first, erf)
     assert np.array_equal(fs, efs) and np.array_equal(fl, efl)

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def device_reassemble(ctx, w, arrivals, len_nic=None, req_size=0, ring=None, max_reqs=8192, reset=True):
+def device_reassemble(ctx, w, arrivals, len_nic=None, req_size=0, ring=None, max_reqs=8192, reset=True, flags=0):
     n = len(arrivals)
     if reset:
         ctx.reassemble_reset()  # the context is shared: nothing of an earlier case may still be in flight
@@ -25,31 +25,37 @@ def device_reassemble(ctx, w, arrivals, len_nic=None, req_size=0, ring=None, max
     tok = torch.zeros(max_reqs, dtype=torch.int64, device=DEV)
     ln = to_dev(len_nic, DEV) if len_nic is not None else None
     n_req, n_frag, n_left = ctx.reassemble(rx, to_dev(np.ascontiguousarray(arrivals, np.uint32), DEV), n, fs, fl, rf,
-                                           tok, ln, req_size)
+                                           tok, ln, req_size, flags=flags)
     return (fs[:n_frag].cpu().numpy().view(np.uint32), fl[:n_frag].cpu().numpy().view(np.uint32),
             rf[:n_req + 1].cpu().numpy().view(np.uint32), tok[:n_req].cpu().numpy().view(np.uint64), n_left, rx,
             (fs, fl, rf))
 
 
+# workgroups of 1024 threads, and of 256 as for a call that runs beside a long kernel (SG_F_SMALL_GROUPS)
+GROUPS = pytest.mark.parametrize("flags", [0, capi.F_SMALL_GROUPS], ids=["groups-of-1024", "groups-of-256"])
+
+
+@GROUPS
 @pytest.mark.parametrize("cfg,n", [(1, None), (2, 3), (2, None), (3, None), (4, 300), (4, None), (5, 2)])
-def test_reassembly_matches_oracle(ctx, cfg, n):
+def test_reassembly_matches_oracle(ctx, cfg, n, flags):
     w = synth.make_workload(cfg, n)
-    print(f"case reassemble cfg={cfg} n_req={w.n_req} arrivals={len(w.arrivals)}", flush=True)
+    print(f"case reassemble cfg={cfg} n_req={w.n_req} arrivals={len(w.arrivals)} flags={flags:#x}", flush=True)
     rng = np.random.default_rng(cfg)
     for arr in (w.arrivals, rng.permutation(w.arrivals)):
-        got = device_reassemble(ctx, w, arr)
+        got = device_reassemble(ctx, w, arr, flags=flags)
         want = oracle.reassemble(w, arrivals=arr)
         for g, e, name in zip(got[:4], want, ("frag_slot", "frag_len", "req_first", "req_token")):
             assert np.array_equal(g, e), name
         assert got[4] == 0
 
 
-def test_reassembly_ref64_by_request_size(ctx):
+@GROUPS
+def test_reassembly_ref64_by_request_size(ctx, flags):
     w = synth.make_workload(2, 4, profile=synth.HDR_REF64)
     len_nic = np.zeros(w.n_slots, np.uint32)
     len_nic[w.frag_slot] = w.frag_len
     size = int(w.req_sizes[0])
-    got = device_reassemble(ctx, w, w.arrivals, len_nic=len_nic, req_size=size)
+    got = device_reassemble(ctx, w, w.arrivals, len_nic=len_nic, req_size=size, flags=flags)
     want = oracle.reassemble(w, req_size=size, frag_len_nic=len_nic)
     for g, e in zip(got[:4], want):
         assert np.array_equal(g, e)
